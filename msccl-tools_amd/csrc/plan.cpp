@@ -1,0 +1,365 @@
+// Host side of the MSCCL-IR executor: table validation, connection matching, dry run, geometry.
+// Nothing in this file touches the GPU, so it is exercised by CPU-only tests through the C ABI.
+#include "plan.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <sstream>
+#include <tuple>
+
+namespace mscclx {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+int fail(int code, const std::string& msg) {
+  g_last_error = msg;
+  return code;
+}
+
+int dtype_size(int dtype) {
+  switch (dtype) {
+    case MSCCLX_U8: case MSCCLX_I8: return 1;
+    case MSCCLX_F16: case MSCCLX_BF16: return 2;
+    case MSCCLX_I32: case MSCCLX_U32: case MSCCLX_F32: return 4;
+    case MSCCLX_I64: case MSCCLX_U64: case MSCCLX_F64: return 8;
+    default: return 0;
+  }
+}
+
+// algorithmic traffic factor per step type: one read + one write per transfer edge (booked at the
+// receiving step) and one more operand read per reduction.
+static int algo_factor(int type) {
+  switch (type) {
+    case MSCCLX_OP_RECV: case MSCCLX_OP_RCS: case MSCCLX_OP_COPY: return 2;
+    case MSCCLX_OP_RRC: case MSCCLX_OP_RRS: case MSCCLX_OP_RRCS: case MSCCLX_OP_REDUCE: return 3;
+    default: return 0;
+  }
+}
+
+static const char* op_name(int t) {
+  static const char* names[] = {"nop", "s", "r", "rcs", "rrs", "rrc", "rrcs", "cpy", "re"};
+  return (t >= 0 && t <= 8) ? names[t] : "?";
+}
+
+static std::string where(const mscclx_plan& p, int tb_row, int step) {
+  std::ostringstream os;
+  os << "rank " << p.tbs[tb_row].rank << " tb " << p.tbs[tb_row].local_id << " step " << step;
+  return os.str();
+}
+
+// One pass of all step lists with `depth` messages per connection (0 = unbounded).  The program is
+// a deterministic dataflow network (FIFOs + monotone step counters), so whether it finishes does
+// not depend on the order in which ready threadblocks are advanced.
+int simulate(const mscclx_plan& plan, int depth) {
+  const int ntb = (int)plan.tbs.size();
+  std::vector<int> pc(ntb, 0);
+  std::vector<int64_t> head(plan.conns.size(), 0), tail(plan.conns.size(), 0);
+  size_t remaining = plan.ops.size();
+  while (remaining) {
+    size_t progressed = 0;
+    for (int t = 0; t < ntb; ++t) {
+      const Tb& tb = plan.tbs[t];
+      const int n = tb.op_end - tb.op_begin;
+      while (pc[t] < n) {
+        const Op& op = plan.ops[tb.op_begin + pc[t]];
+        if (op.depid >= 0) {
+          const int dep_row = plan.rank_tb_begin[tb.rank] + op.depid;
+          if (!(pc[dep_row] > op.deps)) break;
+        }
+        const bool rcv = is_recv_type(op.type), snd = is_send_type(op.type);
+        if (rcv && head[tb.recv_conn] <= tail[tb.recv_conn]) break;
+        if (snd && depth > 0 && head[tb.send_conn] - tail[tb.send_conn] >= depth) break;
+        if (rcv) ++tail[tb.recv_conn];
+        if (snd) ++head[tb.send_conn];
+        ++pc[t];
+        ++progressed;
+      }
+    }
+    if (!progressed) {
+      std::ostringstream os;
+      os << "deadlock with connection depth " << depth << "; blocked:";
+      int shown = 0;
+      for (int t = 0; t < ntb && shown < 6; ++t) {
+        const Tb& tb = plan.tbs[t];
+        if (pc[t] < tb.op_end - tb.op_begin) {
+          os << " [" << where(plan, t, pc[t]) << " " << op_name(plan.ops[tb.op_begin + pc[t]].type) << "]";
+          ++shown;
+        }
+      }
+      return fail(MSCCLX_ERR_DEADLOCK, os.str());
+    }
+    remaining -= progressed;
+  }
+  return MSCCLX_OK;
+}
+
+static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
+  if (d->nranks <= 0 || d->ntbs < 0 || d->nops < 0) return fail(MSCCLX_ERR_INVALID_ARG, "negative table size");
+  if (!d->rank_chunks || (d->ntbs && !d->tbs) || (d->nops && !d->ops)) return fail(MSCCLX_ERR_INVALID_ARG, "null table pointer");
+  p->nranks = d->nranks;
+  p->rank_chunks.assign(d->rank_chunks, d->rank_chunks + (size_t)d->nranks * 3);
+  for (int32_t v : p->rank_chunks)
+    if (v < 0) return fail(MSCCLX_ERR_BAD_IR, "negative buffer extent");
+
+  p->tbs.resize(d->ntbs);
+  p->ops.resize(d->nops);
+  p->rank_tb_begin.assign(d->nranks + 1, 0);
+  int prev_rank = 0, expect_begin = 0;
+  for (int t = 0; t < d->ntbs; ++t) {
+    const int32_t* r = d->tbs + (size_t)t * MSCCLX_TB_COLS;
+    Tb& tb = p->tbs[t];
+    tb.rank = r[0]; tb.send = r[1]; tb.recv = r[2]; tb.chan = r[3]; tb.op_begin = r[4]; tb.op_end = r[5];
+    if (tb.rank < 0 || tb.rank >= d->nranks) return fail(MSCCLX_ERR_BAD_IR, "threadblock row " + std::to_string(t) + ": rank out of range");
+    if (tb.rank < prev_rank) return fail(MSCCLX_ERR_BAD_IR, "threadblock rows must be grouped by ascending rank");
+    if (tb.send < -1 || tb.send >= d->nranks || tb.recv < -1 || tb.recv >= d->nranks)
+      return fail(MSCCLX_ERR_BAD_IR, "threadblock row " + std::to_string(t) + ": peer out of range");
+    if (tb.send == tb.rank || tb.recv == tb.rank) return fail(MSCCLX_ERR_BAD_IR, "threadblock row " + std::to_string(t) + ": a rank cannot be its own peer");
+    if (tb.chan < 0) return fail(MSCCLX_ERR_BAD_IR, "threadblock row " + std::to_string(t) + ": negative channel");
+    if (tb.op_begin != expect_begin || tb.op_end < tb.op_begin || tb.op_end > d->nops)
+      return fail(MSCCLX_ERR_BAD_IR, "threadblock row " + std::to_string(t) + ": step ranges must tile the op table in order");
+    expect_begin = tb.op_end;
+    prev_rank = tb.rank;
+    p->rank_tb_begin[tb.rank + 1]++;
+  }
+  if (expect_begin != d->nops) return fail(MSCCLX_ERR_BAD_IR, "op table has rows no threadblock owns");
+  for (int r = 0; r < d->nranks; ++r) p->rank_tb_begin[r + 1] += p->rank_tb_begin[r];
+  for (int t = 0; t < d->ntbs; ++t) p->tbs[t].local_id = t - p->rank_tb_begin[p->tbs[t].rank];
+
+  // steps
+  for (int t = 0; t < d->ntbs; ++t) {
+    Tb& tb = p->tbs[t];
+    const int ntb_rank = p->rank_tb_begin[tb.rank + 1] - p->rank_tb_begin[tb.rank];
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      const int32_t* r = d->ops + (size_t)o * MSCCLX_OP_COLS;
+      Op& op = p->ops[o];
+      op.type = r[0]; op.srcbuf = r[1]; op.srcoff = r[2]; op.dstbuf = r[3]; op.dstoff = r[4];
+      op.cnt = r[5]; op.depid = r[6]; op.deps = r[7]; op.hasdep = r[8] ? 1 : 0;
+      const std::string at = where(*p, t, o - tb.op_begin);
+      if (op.type < MSCCLX_OP_NOP || op.type > MSCCLX_OP_REDUCE) return fail(MSCCLX_ERR_BAD_IR, at + ": unknown step type " + std::to_string(op.type));
+      if (op.type != MSCCLX_OP_NOP && op.cnt < 1) return fail(MSCCLX_ERR_BAD_IR, at + ": cnt must be >= 1");
+      auto check_ref = [&](int buf, int off, const char* what) -> int {
+        if (buf < 0 || buf > 2) return fail(MSCCLX_ERR_BAD_IR, at + ": bad " + what + " buffer");
+        const int extent = p->rank_chunks[(size_t)tb.rank * 3 + buf];
+        if (off < 0 || (int64_t)off + op.cnt > extent)
+          return fail(MSCCLX_ERR_BAD_IR, at + ": " + what + " chunks [" + std::to_string(off) + "," + std::to_string((int64_t)off + op.cnt) +
+                                             ") outside the buffer's " + std::to_string(extent) + " chunks");
+        return MSCCLX_OK;
+      };
+      int rc;
+      if (reads_local_src(op.type) && (rc = check_ref(op.srcbuf, op.srcoff, "source"))) return rc;
+      if (touches_local_dst(op.type) && (rc = check_ref(op.dstbuf, op.dstoff, "destination"))) return rc;
+      if (is_send_type(op.type)) {
+        if (tb.send < 0) return fail(MSCCLX_ERR_BAD_IR, at + ": sending step in a threadblock without a send peer");
+        op.send_seq = tb.nsend++;
+      }
+      if (is_recv_type(op.type)) {
+        if (tb.recv < 0) return fail(MSCCLX_ERR_BAD_IR, at + ": receiving step in a threadblock without a recv peer");
+        op.recv_seq = tb.nrecv++;
+      }
+      if (is_reduce_type(op.type)) p->has_reduce = true;
+      if ((op.depid < 0) != (op.deps < 0)) return fail(MSCCLX_ERR_BAD_IR, at + ": depid and deps must both be set or both be -1");
+      if (op.depid >= 0) {
+        if (op.depid >= ntb_rank) return fail(MSCCLX_ERR_BAD_IR, at + ": depid names no threadblock of this rank");
+        const Tb& dep = p->tbs[p->rank_tb_begin[tb.rank] + op.depid];
+        if (op.deps >= dep.op_end - dep.op_begin) return fail(MSCCLX_ERR_BAD_IR, at + ": deps beyond the last step of threadblock " + std::to_string(op.depid));
+      }
+      p->algorithmic_units += (uint64_t)op.cnt * algo_factor(op.type);
+    }
+  }
+  // A step somebody waits for must publish its completion even if the emitter forgot hasdep.
+  for (int t = 0; t < d->ntbs; ++t) {
+    const Tb& tb = p->tbs[t];
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      const Op& op = p->ops[o];
+      if (op.depid >= 0) {
+        const Tb& dep = p->tbs[p->rank_tb_begin[tb.rank] + op.depid];
+        p->ops[dep.op_begin + op.deps].hasdep = 1;
+      }
+    }
+  }
+
+  // connections: exactly one producing and one consuming threadblock per (src, dst, chan)
+  std::map<std::tuple<int, int, int>, int> conn_id;
+  auto get_conn = [&](int src, int dst, int chan) {
+    auto key = std::make_tuple(src, dst, chan);
+    auto it = conn_id.find(key);
+    if (it != conn_id.end()) return it->second;
+    Conn c; c.src = src; c.dst = dst; c.chan = chan;
+    p->conns.push_back(c);
+    return conn_id[key] = (int)p->conns.size() - 1;
+  };
+  for (int t = 0; t < d->ntbs; ++t) {
+    Tb& tb = p->tbs[t];
+    if (tb.nsend) {
+      const int c = get_conn(tb.rank, tb.send, tb.chan);
+      if (p->conns[c].send_tb >= 0)
+        return fail(MSCCLX_ERR_BAD_IR, "rank " + std::to_string(tb.rank) + ": threadblocks " + std::to_string(p->tbs[p->conns[c].send_tb].local_id) + " and " +
+                                           std::to_string(tb.local_id) + " both send to rank " + std::to_string(tb.send) + " on channel " + std::to_string(tb.chan));
+      p->conns[c].send_tb = t;
+      tb.send_conn = c;
+    }
+    if (tb.nrecv) {
+      const int c = get_conn(tb.recv, tb.rank, tb.chan);
+      if (p->conns[c].recv_tb >= 0)
+        return fail(MSCCLX_ERR_BAD_IR, "rank " + std::to_string(tb.rank) + ": threadblocks " + std::to_string(p->tbs[p->conns[c].recv_tb].local_id) + " and " +
+                                           std::to_string(tb.local_id) + " both receive from rank " + std::to_string(tb.recv) + " on channel " + std::to_string(tb.chan));
+      p->conns[c].recv_tb = t;
+      tb.recv_conn = c;
+    }
+  }
+  for (size_t c = 0; c < p->conns.size(); ++c) {
+    Conn& cn = p->conns[c];
+    std::ostringstream name;
+    name << "connection " << cn.src << "->" << cn.dst << " channel " << cn.chan;
+    if (cn.send_tb < 0) return fail(MSCCLX_ERR_BAD_IR, name.str() + " has a receiver but no sender");
+    if (cn.recv_tb < 0) return fail(MSCCLX_ERR_BAD_IR, name.str() + " has a sender but no receiver");
+    const Tb& s = p->tbs[cn.send_tb];
+    const Tb& r = p->tbs[cn.recv_tb];
+    if (s.nsend != r.nrecv)
+      return fail(MSCCLX_ERR_BAD_IR, name.str() + ": " + std::to_string(s.nsend) + " sends but " + std::to_string(r.nrecv) + " receives");
+    cn.nmsg = s.nsend;
+    int ro = r.op_begin;
+    for (int so = s.op_begin; so < s.op_end; ++so) {
+      if (!is_send_type(p->ops[so].type)) continue;
+      while (!is_recv_type(p->ops[ro].type)) ++ro;
+      if (p->ops[so].cnt != p->ops[ro].cnt)
+        return fail(MSCCLX_ERR_BAD_IR, name.str() + ": message " + std::to_string(p->ops[so].send_seq) + " is sent with cnt " + std::to_string(p->ops[so].cnt) +
+                                           " but received with cnt " + std::to_string(p->ops[ro].cnt));
+      cn.max_cnt = std::max(cn.max_cnt, p->ops[so].cnt);
+      ++ro;
+    }
+  }
+  return MSCCLX_OK;
+}
+
+static int thread_index(int threads) {
+  switch (threads) { case 64: return 0; case 128: return 1; case 256: return 2; case 512: return 3; default: return -1; }
+}
+
+int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
+                    int num_cus, const int capacity_by_threads[4], Geometry* out) {
+  const int elem = dtype_size(dtype);
+  if (!elem) return fail(MSCCLX_ERR_INVALID_ARG, "unknown dtype " + std::to_string(dtype));
+  if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
+  Geometry g;
+  g.vector_path = (chunk_bytes % 16 == 0) ? 1 : 0;
+  g.unit_bytes = g.vector_path ? 16 : elem;
+  g.chunk_units = chunk_bytes / g.unit_bytes;
+  const int ntbs = (int)plan.tbs.size();
+  if (ntbs == 0) return fail(MSCCLX_ERR_BAD_IR, "the algorithm has no threadblocks");
+
+  // threads per workgroup: as asked, else the largest of 256/128/64 with which every threadblock is resident
+  int threads = cfg.threads;
+  if (threads) {
+    if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
+  } else {
+    threads = 256;
+    while (threads > 64 && capacity_by_threads[thread_index(threads)] < ntbs) threads /= 2;
+  }
+  const int capacity = capacity_by_threads[thread_index(threads)];
+  if (capacity < ntbs)
+    return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks must be resident at once but only " + std::to_string(capacity) +
+                                         " workgroups of " + std::to_string(threads) + " threads fit on the device");
+  g.threads = threads;
+
+  // slices: enough workgroups to cover the chip a few times, never cutting a chunk below 2 KiB
+  const uint64_t min_slice_units = std::max<uint64_t>(1, 2048 / g.unit_bytes);
+  const int64_t max_by_size = (int64_t)std::max<uint64_t>(1, g.chunk_units / min_slice_units);
+  int64_t slices = cfg.slices;
+  if (slices < 0) return fail(MSCCLX_ERR_INVALID_ARG, "slices must be >= 0");
+  if (!slices) {
+    const int64_t target = std::min<int64_t>(capacity, (int64_t)2 * num_cus);
+    slices = std::max<int64_t>(1, target / ntbs);
+    slices = std::min(slices, max_by_size);
+    if (slices >= 8) slices -= slices % 8;
+  }
+  if ((uint64_t)slices > g.chunk_units) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");
+  if (slices * (int64_t)ntbs > capacity)
+    return fail(MSCCLX_ERR_CAPACITY, std::to_string(slices * (int64_t)ntbs) + " workgroups requested but only " + std::to_string(capacity) + " can be resident");
+  g.slices = (int)slices;
+
+  const uint64_t longest_slice = (g.chunk_units + slices - 1) / slices;
+  int64_t piece_bytes = cfg.piece_bytes;
+  if (piece_bytes < 0) return fail(MSCCLX_ERR_INVALID_ARG, "piece_bytes must be >= 0");
+  if (!piece_bytes) piece_bytes = 64 * 1024;
+  uint64_t piece_units = std::max<uint64_t>(1, (uint64_t)piece_bytes / g.unit_bytes);
+  piece_units = std::min(piece_units, longest_slice);
+  if (piece_units > 0x7fffffffu / 64) return fail(MSCCLX_ERR_INVALID_ARG, "piece too large");
+  g.piece_units = (uint32_t)piece_units;
+  g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
+
+  int depth = cfg.fifo_depth;
+  if (depth < 0) return fail(MSCCLX_ERR_INVALID_ARG, "fifo_depth must be >= 0");
+  if (depth) {
+    int rc = simulate(plan, depth);
+    if (rc) return rc;
+  } else {
+    depth = 1;
+    while (simulate(plan, depth) != MSCCLX_OK) {
+      if (++depth > 4096) return fail(MSCCLX_ERR_DEADLOCK, "the program does not finish with any connection depth up to 4096");
+    }
+    depth = std::max(depth, 4);
+  }
+  g.depth = depth;
+
+  uint64_t fifo_units = 0;
+  for (const Conn& c : plan.conns) fifo_units += (uint64_t)depth * c.max_cnt * g.piece_units;
+  g.slice_fifo_units = fifo_units;
+  g.sync_slice_words = (uint64_t)(plan.tbs.size() + 2 * plan.conns.size()) * kSyncStrideWords;
+  g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
+  const uint64_t sync_bytes = (2 * g.sync_words * 8 + 255) / 256 * 256;
+  g.fifo_byte_off = sync_bytes;
+  g.workspace_bytes = sync_bytes + fifo_units * g.slices * g.unit_bytes + 256;
+  *out = g;
+  return MSCCLX_OK;
+}
+
+}  // namespace mscclx
+
+using namespace mscclx;
+
+extern "C" {
+
+int mscclx_version(void) { return MSCCLX_VERSION; }
+const char* mscclx_last_error(void) { return g_last_error.c_str(); }
+
+int mscclx_plan_create(const mscclx_plan_desc* desc, mscclx_plan** out) {
+  if (!desc || !out) return fail(MSCCLX_ERR_INVALID_ARG, "null argument");
+  *out = nullptr;
+  mscclx_plan* p = new mscclx_plan();
+  int rc = build_plan(desc, p);
+  if (rc) {
+    delete p;
+    return rc;
+  }
+  *out = p;
+  return MSCCLX_OK;
+}
+
+int mscclx_plan_destroy(mscclx_plan* plan) {
+  if (!plan) return MSCCLX_OK;
+  if (plan->dev) destroy_device_state(plan->dev);
+  delete plan;
+  return MSCCLX_OK;
+}
+
+int mscclx_plan_simulate(const mscclx_plan* plan, int32_t fifo_depth) {
+  if (!plan || fifo_depth < 0) return fail(MSCCLX_ERR_INVALID_ARG, "bad argument");
+  return simulate(*plan, fifo_depth);
+}
+
+int mscclx_plan_min_fifo_depth(const mscclx_plan* plan) {
+  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
+  int rc = simulate(*plan, 0);
+  if (rc) return rc;  // not even unbounded connections help
+  for (int d = 1; d <= 4096; ++d)
+    if (simulate(*plan, d) == MSCCLX_OK) return d;
+  return fail(MSCCLX_ERR_DEADLOCK, "needs a connection depth above 4096");
+}
+
+uint64_t mscclx_plan_algorithmic_units(const mscclx_plan* plan) { return plan ? plan->algorithmic_units : 0; }
+
+}  // extern "C"

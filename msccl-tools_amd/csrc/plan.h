@@ -1,0 +1,132 @@
+// Internal host/device structures of the MSCCL-IR executor (not part of the C ABI).
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "mscclx.h"
+
+namespace mscclx {
+
+// One <step>, plus what plan_create derives for it.
+struct Op {
+  int32_t type, srcbuf, srcoff, dstbuf, dstoff, cnt, depid, deps, hasdep;
+  int32_t send_seq = -1;  // position among this threadblock's send-type steps
+  int32_t recv_seq = -1;  // position among this threadblock's recv-type steps
+};
+
+struct Tb {
+  int32_t rank, send, recv, chan, op_begin, op_end;
+  int32_t local_id = 0;    // <tb id>
+  int32_t send_conn = -1;  // connection this threadblock produces into
+  int32_t recv_conn = -1;  // connection this threadblock consumes from
+  int32_t nsend = 0, nrecv = 0;
+};
+
+// FIFO (sender rank, receiver rank, channel).
+struct Conn {
+  int32_t src, dst, chan;
+  int32_t send_tb = -1, recv_tb = -1;  // global threadblock rows
+  int32_t nmsg = 0;                    // messages per pass
+  int32_t max_cnt = 0;                 // largest message, in chunks
+};
+
+inline bool is_send_type(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
+inline bool is_recv_type(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
+inline bool is_reduce_type(int t) { return t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE; }
+inline bool reads_local_src(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE; }
+inline bool touches_local_dst(int t) { return is_recv_type(t) || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE; }
+
+// ---- device-side images (plain data, uploaded at bind) ----
+struct DevOp {
+  int32_t type, cnt;
+  int32_t src_slot, srcoff;  // src_slot = rank*3 + buffer: index into the buffer pointer table
+  int32_t dst_slot, dstoff;
+  int32_t dep_tb, dep_step;  // global threadblock row / step, or -1
+  int32_t dep_nops;          // number of steps of the threadblock depended on
+  int32_t hasdep;
+  int32_t send_seq, recv_seq;
+};
+
+struct DevTb {
+  int32_t op_begin, nops;
+  int32_t send_conn, recv_conn;
+  int32_t nsend, nrecv;
+  int32_t rank, pad;
+};
+
+struct DevConn {
+  uint64_t fifo_off;    // offset of this connection's slots inside one slice's FIFO region, in units
+  uint32_t slot_units;  // units per slot = max_cnt * piece_units
+  uint32_t pad;
+};
+
+struct Geometry {
+  uint64_t chunk_units = 0;   // units (16-byte vectors or elements) per chunk
+  uint32_t unit_bytes = 0;
+  uint32_t piece_units = 0;
+  int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
+  int32_t passes = 0;
+  uint64_t slice_fifo_units = 0;  // FIFO units one slice needs (all connections)
+  uint64_t sync_words = 0;        // uint64 words of ONE synchronisation area (there are two)
+  uint64_t sync_slice_words = 0;  // words per slice inside an area
+  uint64_t workspace_bytes = 0;
+  uint64_t fifo_byte_off = 0;     // where the FIFO region starts inside the workspace
+};
+
+struct KernelParams {
+  const DevTb* tbs;
+  const DevOp* ops;
+  const DevConn* conns;
+  void* const* bufs;            // [nranks*3]
+  unsigned long long* sync_cur; // this launch's counters
+  unsigned long long* sync_nxt; // next launch's counters (cleared by this launch)
+  unsigned char* fifo;
+  mscclx_status* host_status;   // pinned host memory
+  uint64_t chunk_units;
+  uint64_t slice_fifo_units;
+  uint64_t sync_slice_words;
+  uint64_t timeout_ticks;
+  uint32_t piece_units;
+  int32_t slices, depth, ntbs, nconns;
+};
+
+constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
+constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
+
+struct DeviceState;  // defined in exec.hip
+
+}  // namespace mscclx
+
+struct mscclx_plan {
+  int32_t nranks = 0;
+  std::vector<int32_t> rank_chunks;  // [nranks*3]
+  std::vector<mscclx::Tb> tbs;
+  std::vector<mscclx::Op> ops;
+  std::vector<mscclx::Conn> conns;
+  std::vector<int32_t> rank_tb_begin;  // [nranks+1] first global tb row of each rank
+  bool has_reduce = false;
+  uint64_t algorithmic_units = 0;
+
+  // set by configure
+  bool configured = false;
+  size_t chunk_bytes = 0;
+  int32_t dtype = 0, redop = 0;
+  int32_t timeout_ms = 10000;
+  mscclx::Geometry geo;
+
+  // set by bind
+  mscclx::DeviceState* dev = nullptr;
+};
+
+namespace mscclx {
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+int dtype_size(int dtype);
+// Host dry run of one pass; returns MSCCLX_OK or MSCCLX_ERR_DEADLOCK (error text names a blocked step).
+int simulate(const mscclx_plan& plan, int depth);
+// Pure geometry decision (no HIP): max_wgs = resident workgroup capacity per thread count.
+int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
+                    int num_cus, const int capacity_by_threads[4], Geometry* out);
+void destroy_device_state(DeviceState* d);
+}  // namespace mscclx

@@ -1,0 +1,132 @@
+"""The C-ABI library without a GPU: it loads, exports every declared symbol, and its host half
+(table validation, connection matching, dry run, geometry) behaves."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import ir_samples
+from msccl.executor import (EXPORTED_SYMBOLS, IRError, MscclxError, Plan, parse_algo_xml)
+from msccl.executor import binding
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(mscclx_lib):
+    header = open(os.path.join(ROOT, "include", "mscclx.h")).read()
+    declared = set(re.findall(r"\b(mscclx_[a-z_]+)\s*\(", header))
+    assert declared == set(EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(mscclx_lib, name), name
+    assert mscclx_lib.mscclx_version() == 1
+
+
+def test_struct_layouts_match_header():
+    assert ctypes.sizeof(binding.Config) == 32
+    assert ctypes.sizeof(binding.Info) == 48
+    assert ctypes.sizeof(binding.Status) == 32
+
+
+def test_tables_from_xml():
+    t = parse_algo_xml(ir_samples.FUSION_CHAIN_XML)
+    assert (t.ngpus, t.ntbs, t.nops, t.coll, t.inplace) == (3, 3, 5, "allreduce", True)
+    assert t.rank_chunks.tolist() == [[3, 0, 0]] * 3
+    assert t.tbs.tolist() == [[0, 1, 2, 0, 0, 2], [1, 2, 0, 0, 2, 4], [2, 0, 1, 0, 4, 5]]
+    assert t.ops[:, 0].tolist() == [1, 3, 4, 2, 6]  # s rcs | rrs r | rrcs
+    assert t.algorithmic_units() == 30
+
+
+def test_xml_errors():
+    with pytest.raises(IRError):
+        parse_algo_xml("<nope/>")
+    with pytest.raises(IRError):
+        parse_algo_xml(ir_samples.FUSION_CHAIN_XML.replace('type="rcs"', 'type="xyz"'))
+    with pytest.raises(IRError):
+        parse_algo_xml(ir_samples.FUSION_CHAIN_XML.replace('<gpu id="2"', '<gpu id="5"'))
+
+
+def test_plan_create_and_dry_run(mscclx_lib):
+    p = Plan(parse_algo_xml(ir_samples.ring_allreduce_xml(8)))
+    assert p.algorithmic_units() == 5 * 7 * 8  # 5(n-1) chunk moves per chunk index
+    with pytest.raises(MscclxError) as e:
+        p.simulate(1)  # fused ring: every rank holds one outgoing message and wants to push another
+    assert e.value.code == binding.ERR_DEADLOCK and "rrs" in e.value.message
+    assert p.simulate(2) == 0
+    assert p.simulate(0) == 0
+    assert p.min_fifo_depth() == 2
+    assert Plan(parse_algo_xml(ir_samples.allpairs_allreduce_xml(4))).min_fifo_depth() == 1
+
+
+def _mutated(xml, old, new, count=1):
+    assert old in xml
+    return parse_algo_xml(xml.replace(old, new, count))
+
+
+@pytest.mark.parametrize("old,new,needle", [
+    ('type="rcs" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="3"', 'type="rcs" srcbuf="i" srcoff="0" dstbuf="i" dstoff="1" cnt="3"', "outside"),
+    ('<tb id="0" send="1" recv="2"', '<tb id="0" send="-1" recv="2"', "without a send peer"),
+    ('type="rrcs" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="3"', 'type="rrcs" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="2"', "cnt"),
+    ('type="rrcs"', 'type="rrc"', "receiver"),
+    ('<step s="1" type="r" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="3" depid="-1" deps="-1"', '<step s="1" type="r" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="3" depid="4" deps="0"', "depid"),
+])
+def test_plan_create_rejects_bad_ir(mscclx_lib, old, new, needle):
+    with pytest.raises(MscclxError) as e:
+        Plan(_mutated(ir_samples.FUSION_CHAIN_XML, old, new))
+    assert e.value.code == binding.ERR_BAD_IR
+    assert needle in e.value.message
+
+
+def test_two_senders_on_one_connection_rejected(mscclx_lib):
+    xml = ir_samples.ring_allreduce_xml(4, instances=2).replace('chan="1"', 'chan="0"')
+    with pytest.raises(MscclxError) as e:
+        Plan(parse_algo_xml(xml))
+    assert "both send" in e.value.message
+
+
+def test_unfed_receive_is_a_bad_connection(mscclx_lib):
+    with pytest.raises(MscclxError) as e:
+        Plan(parse_algo_xml(ir_samples.RRC_CPY_NOP_XML.replace('type="s"', 'type="nop"')))
+    assert "no sender" in e.value.message
+
+
+def test_dependency_cycle_is_a_deadlock(mscclx_lib):
+    # tb0 step0 waits for tb1 step1, tb1 step0 waits for tb0 step0
+    xml = ir_samples.RRC_CPY_NOP_XML.replace('type="rrc" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="1" depid="-1" deps="-1"',
+                                             'type="rrc" srcbuf="i" srcoff="0" dstbuf="i" dstoff="0" cnt="1" depid="1" deps="1"')
+    p = Plan(parse_algo_xml(xml))
+    with pytest.raises(MscclxError) as e:
+        p.simulate(0)
+    assert e.value.code == binding.ERR_DEADLOCK
+
+
+def test_geometry_without_a_device(mscclx_lib):
+    p = Plan(parse_algo_xml(ir_samples.ring_allgather_xml(8, 4)))  # 32 threadblocks
+    info = p.configure(8 << 20, "int32", max_workgroups=2048)
+    assert info.vector_path == 1 and info.threads == 256
+    assert info.slices == 16 and info.workgroups == 512          # 2 workgroups per CU of a 256-CU part
+    assert info.piece_bytes == 64 * 1024 and info.fifo_depth == 4
+    assert info.passes == (8 << 20) // 16 // (64 * 1024)
+    assert info.connections == 32
+    assert info.algorithmic_units * (8 << 20) == 2 * 7 * 8 * (32 << 20)   # 2(n-1) n S_in
+    # FIFO: 32 connections x 16 slices x 4 slots x 64 KiB
+    assert info.workspace_bytes >= 32 * 16 * 4 * 64 * 1024
+    # element path when the chunk is not a multiple of 16 bytes
+    info = p.configure(1000 * 4 + 4, "int32", max_workgroups=2048)
+    assert info.vector_path == 0
+    with pytest.raises(MscclxError):
+        p.configure(6, "int32", max_workgroups=2048)              # not a multiple of the element
+    with pytest.raises(MscclxError) as e:
+        p.configure(8 << 20, "int32", max_workgroups=16)          # 32 threadblocks cannot be resident
+    assert e.value.code == binding.ERR_CAPACITY
+    with pytest.raises(MscclxError) as e:
+        p.configure(8 << 20, "int32", max_workgroups=2048, fifo_depth=1)
+    assert e.value.code == binding.ERR_DEADLOCK
+
+
+def test_launch_before_bind_is_a_state_error(mscclx_lib):
+    p = Plan(parse_algo_xml(ir_samples.FUSION_CHAIN_XML))
+    with pytest.raises(MscclxError) as e:
+        p.launch()
+    assert e.value.code == binding.ERR_STATE

@@ -1,0 +1,185 @@
+"""HIP executor vs the NumPy interpreter on the same seeded inputs, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import ir_samples
+from oracle import collectives as oc
+from oracle import ir_interp as oi
+
+pytestmark = pytest.mark.gpu
+
+NP2TORCH = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16, "int32": torch.int32,
+            "uint8": torch.uint8, "int8": torch.int8, "int64": torch.int64, "float64": torch.float64}
+
+
+def make_inputs(n, elems, dtype, seed):
+    out = []
+    for r in range(n):
+        rng = np.random.default_rng(1000 * seed + r)
+        if dtype in ("float32", "float64"):
+            out.append((rng.random(elems, dtype=np.float32) * 2 - 1).astype(oi.DTYPES[dtype]))
+        elif dtype == "float16":
+            out.append((rng.random(elems, dtype=np.float32) * 2 - 1).astype(np.float16))
+        elif dtype == "bfloat16":
+            out.append(oi.f32_to_bf16_bits(rng.standard_normal(elems, dtype=np.float32)))
+        else:
+            info = np.iinfo(oi.DTYPES[dtype])
+            out.append(rng.integers(info.min, info.max, elems, dtype=np.int64, endpoint=True).astype(oi.DTYPES[dtype]))
+    return out
+
+
+def to_torch(x, dtype):
+    if dtype == "bfloat16":
+        return torch.from_numpy(x.view(np.int16)).view(torch.bfloat16)
+    return torch.from_numpy(x)
+
+
+def to_numpy(t, dtype):
+    t = t.cpu()
+    if dtype == "bfloat16":
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()
+
+
+def run_both(xml, chunk_elems, dtype, seed=1, redop="sum", in_elems=None, **knobs):
+    """Returns (gpu buffers, oracle buffers) as lists over ranks of {'i','o'} numpy arrays."""
+    from msccl.executor import Executor, collective_buffers, DTYPE_SIZES
+    algo = oi.parse_xml(xml)
+    n = algo.ngpus
+    esz = DTYPE_SIZES[dtype]
+    if in_elems is None:
+        if algo.coll == "allgather" and algo.inplace:
+            in_elems = algo.gpus[0].o_chunks * chunk_elems // n
+        else:
+            in_elems = algo.gpus[0].i_chunks * chunk_elems
+    x = make_inputs(n, in_elems, dtype, seed)
+    # oracle
+    bufs = oc.place_inputs(algo, x, chunk_elems, dtype)
+    oi.Interpreter(algo).run(bufs, chunk_elems, dtype, redop)
+    # device
+    ex = Executor(xml)
+    print(f"case: {algo.name} n={n} dtype={dtype} chunk_elems={chunk_elems} knobs={knobs}", flush=True)
+    info = ex.setup(chunk_elems * esz, dtype, redop, **knobs)
+    ins, outs, _ = collective_buffers(ex.tables, chunk_elems * esz, dtype, inputs=[to_torch(v, dtype) for v in x])
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    got = [{"i": to_numpy(ins[r], dtype) if ins[r] is not None else np.zeros(0, oi.DTYPES[dtype]),
+            "o": to_numpy(outs[r], dtype) if outs[r] is not None else np.zeros(0, oi.DTYPES[dtype])} for r in range(n)]
+    return got, bufs, ex, info
+
+
+def assert_same(got, want, keys=("i", "o")):
+    for r, (g, w) in enumerate(zip(got, want)):
+        for k in keys:
+            gv, wv = g[k].view(np.uint8), w[k].view(np.uint8)
+            assert gv.shape == wv.shape, (r, k, gv.shape, wv.shape)
+            if not np.array_equal(gv, wv):
+                bad = np.flatnonzero(gv != wv)
+                raise AssertionError(f"rank {r} buffer {k}: {bad.size} bytes differ, first at byte {bad[0]}")
+
+
+def test_fusion_chain_f32():
+    got, want, _, _ = run_both(ir_samples.FUSION_CHAIN_XML, 1024, "float32")
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "int32", "uint8", "float64", "int64", "int8"])
+def test_ring_allreduce_dtypes(dtype):
+    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(8), 4096, dtype)
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("redop", ["prod", "max", "min"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "int32"])
+def test_ring_allreduce_redops(dtype, redop):
+    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(4), 2048, dtype, redop=redop)
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("n,inst", [(2, 1), (8, 4), (5, 2)])
+def test_ring_allgather(n, inst):
+    got, want, _, _ = run_both(ir_samples.ring_allgather_xml(n, inst), 8192, "int32")
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("n", [2, 4, 8])
+def test_allpairs_scratch_and_deps(n):
+    got, want, _, _ = run_both(ir_samples.allpairs_allreduce_xml(n), 4096, "float32")
+    assert_same(got, want)
+
+
+def test_rrc_cpy_nop():
+    got, want, _, _ = run_both(ir_samples.RRC_CPY_NOP_XML, 1000 * 4, "int32")
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("chunk_elems,dtype", [(1, "float32"), (3, "float32"), (4, "float32"), (1001, "float16"),
+                                               (7, "uint8"), (16, "uint8"), (100003, "int32")])
+def test_ragged_chunk_sizes(chunk_elems, dtype):
+    """Chunks that are not a multiple of 16 bytes take the element path; tiny chunks leave most
+    slices empty-handed, so the geometry must shrink."""
+    got, want, _, info = run_both(ir_samples.ring_allreduce_xml(4), chunk_elems, dtype)
+    assert_same(got, want)
+
+
+@pytest.mark.parametrize("knobs", [
+    dict(slices=1, piece_bytes=4096, fifo_depth=2, threads=64),
+    dict(slices=3, piece_bytes=16 * 7, fifo_depth=3, threads=128),
+    dict(slices=16, piece_bytes=1 << 20, fifo_depth=8, threads=512),
+    dict(slices=8, piece_bytes=65536, fifo_depth=2, threads=256),
+])
+def test_geometry_knobs(knobs):
+    got, want, _, info = run_both(ir_samples.ring_allreduce_xml(8, 2), 40000, "float32", **knobs)
+    assert info.slices == knobs["slices"] and info.threads == knobs["threads"]
+    assert_same(got, want)
+    got, want, _, _ = run_both(ir_samples.allpairs_allreduce_xml(5), 40000, "bfloat16", **knobs)
+    assert_same(got, want)
+
+
+def test_relaunch_reuses_counters():
+    """Launch several times on the same binding: the counter areas alternate and are re-armed."""
+    from msccl.executor import Executor, collective_buffers
+    xml = ir_samples.ring_allgather_xml(8, 2)
+    algo = oi.parse_xml(xml)
+    E = 5000
+    ex = Executor(xml)
+    ex.setup(E * 4, "int32")
+    for it in range(5):
+        x = make_inputs(8, 2 * E, "int32", seed=50 + it)
+        ins, outs, res = collective_buffers(ex.tables, E * 4, "int32", inputs=[torch.from_numpy(v) for v in x])
+        if it == 0:
+            keep = (ins, outs, res)
+        else:  # same device buffers, new contents
+            for r in range(8):
+                keep[1][r].copy_(outs[r])
+        ex.run(keep[0], keep[1])
+        want = np.concatenate(x)
+        for r in range(8):
+            assert np.array_equal(keep[2][r].cpu().numpy(), want), (it, r)
+
+
+def test_watchdog_reports_instead_of_hanging():
+    """A 1 ms watchdog while a receive legitimately waits for tens of milliseconds: the waiting
+    workgroup must give up cleanly (every wave exits, the producer still finishes), the error names
+    the waiting step, and the next launch with the default limit works and is correct."""
+    from msccl.executor import Executor, MscclxError, collective_buffers
+    xml = ir_samples.slow_producer_xml(24)
+    nbytes = 64 << 20
+    ex = Executor(xml)
+    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, piece_bytes=65536)
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    print("case: watchdog launch", flush=True)
+    ex.launch()
+    with pytest.raises(MscclxError) as e:
+        ex.wait()
+    assert "watchdog" in str(e.value) and "rank 1 tb 0 step 0" in str(e.value) and "incoming message" in str(e.value)
+    torch.cuda.synchronize()
+    # same plan, sane limit: completes and delivers
+    ex2 = Executor(xml)
+    ex2.setup(nbytes, "uint8", slices=4)
+    ins, outs, _ = collective_buffers(ex2.tables, nbytes, "uint8", inputs=x)
+    ex2.run(ins, outs)
+    assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
