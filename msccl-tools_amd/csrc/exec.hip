@@ -11,9 +11,11 @@
 //   flag[tb]   = pass*nsteps + step + 1 of the last finished step with hasdep=1     (depid/deps wait)
 //   head[conn] = messages produced;  tail[conn] = messages consumed                  (FIFO hand-off)
 // Wave 0 polls up to three conditions at once, one per lane; a barrier releases the other waves.
-// A producer publishes with a release store after a workgroup barrier; a consumer's successful poll
-// is followed by an acquire fence.  Two counter areas alternate between launches: a launch clears
-// the area the next launch will use, so no memset sits between launches.
+// Payload is read and written with device-scope (sc1) accesses only, so a producer publishes by
+// waiting for its stores to be acknowledged, a workgroup barrier, and a counter store; a consumer
+// reads the payload after its poll succeeds.  No cache-wide write-back or invalidate is issued.
+// Two counter areas alternate between launches: a launch clears the area the next launch will
+// use, so no memset sits between launches.
 //
 // Every wait is bounded by a wall-clock watchdog; on expiry the workgroup raises the area's abort
 // word, all other workgroups see it in their own waits, and every wave leaves the kernel.
@@ -39,12 +41,15 @@ typedef unsigned long long u64;
   } while (0)
 
 // ------------------------------------------------------------------------------------------------
-// element-wise reducers
+// element-wise reducers.  Reducer<DT, OP>::combine<S>(a, b) reduces two storage words of type S
+// (one element of 1/2/4/8 bytes, or 16 bytes of elements) element by element.
 // ------------------------------------------------------------------------------------------------
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
 template <int OP, typename T>
-__device__ __forceinline__ T red_scalar(T a, T b) {
-  if (OP == MSCCLX_SUM) return a + b;
-  if (OP == MSCCLX_PROD) return a * b;
+__device__ __forceinline__ T red_int(T a, T b) {
+  if (OP == MSCCLX_SUM) return (T)(a + b);
+  if (OP == MSCCLX_PROD) return (T)(a * b);
   if (OP == MSCCLX_MAX) return a > b ? a : b;
   return a < b ? a : b;
 }
@@ -72,134 +77,138 @@ __device__ __forceinline__ unsigned short f32_to_bf16(float f) {  // round to ne
 __device__ __forceinline__ float f16_to_f32(unsigned short h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ unsigned short f32_to_f16(float f) { return __builtin_bit_cast(unsigned short, (_Float16)f); }
 
-// Reducer<DT, OP>::one() combines two elements given as raw storage; ::vec() combines 16 bytes.
-template <int DT, int OP> struct Reducer;
-
-#define MSCCLX_INT_REDUCER(DT, T)                                                                  \
-  template <int OP> struct Reducer<DT, OP> {                                                       \
-    typedef T elem;                                                                                \
-    static __device__ __forceinline__ T one(T a, T b) { return red_scalar<OP, T>(a, b); }          \
-    static __device__ __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {                                \
-      typedef T vt __attribute__((ext_vector_type(16 / sizeof(T))));                               \
-      vt x = __builtin_bit_cast(vt, a), y = __builtin_bit_cast(vt, b), r;                          \
-      _Pragma("unroll") for (int i = 0; i < (int)(16 / sizeof(T)); ++i) r[i] = red_scalar<OP, T>(x[i], y[i]); \
-      return __builtin_bit_cast(u32x4, r);                                                         \
-    }                                                                                              \
-  };
-MSCCLX_INT_REDUCER(MSCCLX_U8, unsigned char)
-MSCCLX_INT_REDUCER(MSCCLX_I8, signed char)
-MSCCLX_INT_REDUCER(MSCCLX_I32, int)
-MSCCLX_INT_REDUCER(MSCCLX_U32, unsigned int)
-MSCCLX_INT_REDUCER(MSCCLX_I64, long long)
-MSCCLX_INT_REDUCER(MSCCLX_U64, unsigned long long)
-
-template <int OP> struct Reducer<MSCCLX_F32, OP> {
-  typedef float elem;
-  static __device__ __forceinline__ float one(float a, float b) { return red_float<OP>(a, b); }
-  static __device__ __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
-    u32x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(red_float<OP>(__uint_as_float(a[i]), __uint_as_float(b[i])));
-    return r;
-  }
-};
-template <int OP> struct Reducer<MSCCLX_F64, OP> {
-  typedef double elem;
-  static __device__ __forceinline__ double one(double a, double b) { return red_double<OP>(a, b); }
-  static __device__ __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
-    typedef double d2 __attribute__((ext_vector_type(2)));
-    d2 x = __builtin_bit_cast(d2, a), y = __builtin_bit_cast(d2, b), r;
-    r[0] = red_double<OP>(x[0], y[0]);
-    r[1] = red_double<OP>(x[1], y[1]);
-    return __builtin_bit_cast(u32x4, r);
-  }
-};
+// Element arithmetic per dtype on raw element storage E (unsigned type of the element's size).
 // 16-bit floats: widen to fp32, operate, round to nearest even once.  For sum this equals the
 // correctly rounded 16-bit result (24 >= 2p+2 for p = 11 and p = 8); products of two 16-bit values
 // are exact in fp32, so they too are rounded once.
-template <int OP> struct Reducer<MSCCLX_F16, OP> {
-  typedef unsigned short elem;
-  static __device__ __forceinline__ unsigned short one(unsigned short a, unsigned short b) {
-    return f32_to_f16(red_float<OP>(f16_to_f32(a), f16_to_f32(b)));
-  }
-  static __device__ __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
-    u32x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      unsigned lo = one((unsigned short)(a[i] & 0xffffu), (unsigned short)(b[i] & 0xffffu));
-      unsigned hi = one((unsigned short)(a[i] >> 16), (unsigned short)(b[i] >> 16));
-      r[i] = lo | (hi << 16);
-    }
-    return r;
+template <int DT, int OP> struct ElemOp;
+#define MSCCLX_INT_ELEM(DT, T, E)                                                                  \
+  template <int OP> struct ElemOp<DT, OP> {                                                        \
+    typedef E store;                                                                               \
+    static __device__ __forceinline__ E op(E a, E b) { return (E)red_int<OP, T>((T)a, (T)b); }     \
+  };
+MSCCLX_INT_ELEM(MSCCLX_U8, unsigned char, unsigned char)
+MSCCLX_INT_ELEM(MSCCLX_I8, signed char, unsigned char)
+MSCCLX_INT_ELEM(MSCCLX_I32, int, unsigned int)
+MSCCLX_INT_ELEM(MSCCLX_U32, unsigned int, unsigned int)
+MSCCLX_INT_ELEM(MSCCLX_I64, long long, unsigned long long)
+MSCCLX_INT_ELEM(MSCCLX_U64, unsigned long long, unsigned long long)
+template <int OP> struct ElemOp<MSCCLX_F16, OP> {
+  typedef unsigned short store;
+  static __device__ __forceinline__ unsigned short op(unsigned short a, unsigned short b) { return f32_to_f16(red_float<OP>(f16_to_f32(a), f16_to_f32(b))); }
+};
+template <int OP> struct ElemOp<MSCCLX_BF16, OP> {
+  typedef unsigned short store;
+  static __device__ __forceinline__ unsigned short op(unsigned short a, unsigned short b) { return f32_to_bf16(red_float<OP>(bf16_to_f32(a), bf16_to_f32(b))); }
+};
+template <int OP> struct ElemOp<MSCCLX_F32, OP> {
+  typedef unsigned int store;
+  static __device__ __forceinline__ unsigned int op(unsigned int a, unsigned int b) { return __float_as_uint(red_float<OP>(__uint_as_float(a), __uint_as_float(b))); }
+};
+template <int OP> struct ElemOp<MSCCLX_F64, OP> {
+  typedef unsigned long long store;
+  static __device__ __forceinline__ unsigned long long op(unsigned long long a, unsigned long long b) {
+    return __builtin_bit_cast(unsigned long long, red_double<OP>(__builtin_bit_cast(double, a), __builtin_bit_cast(double, b)));
   }
 };
-template <int OP> struct Reducer<MSCCLX_BF16, OP> {
-  typedef unsigned short elem;
-  static __device__ __forceinline__ unsigned short one(unsigned short a, unsigned short b) {
-    return f32_to_bf16(red_float<OP>(bf16_to_f32(a), bf16_to_f32(b)));
-  }
-  static __device__ __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
-    u32x4 r;
+
+template <int DT, int OP> struct Reducer {
+  typedef ElemOp<DT, OP> E;
+  typedef typename E::store store;
+  static constexpr int kElemBytes = sizeof(store);
+  // 16 bytes of elements
+  static __device__ __forceinline__ u32x4 combine(u32x4 a, u32x4 b) {
+    typedef store vt __attribute__((ext_vector_type(16 / sizeof(store))));
+    vt x = __builtin_bit_cast(vt, a), y = __builtin_bit_cast(vt, b), r;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      unsigned lo = one((unsigned short)(a[i] & 0xffffu), (unsigned short)(b[i] & 0xffffu));
-      unsigned hi = one((unsigned short)(a[i] >> 16), (unsigned short)(b[i] >> 16));
-      r[i] = lo | (hi << 16);
-    }
-    return r;
+    for (int i = 0; i < (int)(16 / sizeof(store)); ++i) r[i] = E::op(x[i], y[i]);
+    return __builtin_bit_cast(u32x4, r);
+  }
+  // one element held in the word a buffer access of its size returns
+  static __device__ __forceinline__ unsigned char combine(unsigned char a, unsigned char b) { return (unsigned char)E::op((store)a, (store)b); }
+  static __device__ __forceinline__ unsigned short combine(unsigned short a, unsigned short b) { return (unsigned short)E::op((store)a, (store)b); }
+  static __device__ __forceinline__ unsigned int combine(unsigned int a, unsigned int b) { return (unsigned int)E::op((store)a, (store)b); }
+  static __device__ __forceinline__ u32x2 combine(u32x2 a, u32x2 b) {
+    return __builtin_bit_cast(u32x2, (unsigned long long)E::op((store)__builtin_bit_cast(unsigned long long, a), (store)__builtin_bit_cast(unsigned long long, b)));
   }
 };
 
 // ------------------------------------------------------------------------------------------------
-// data movement: out1[, out2] = a [(+) b] over n units.  STREAM_* marks operands that live in a rank
-// buffer (touched once: non-temporal) as opposed to a FIFO slot (re-read soon: cached).
+// memory access.  Every load and store of payload goes through a raw buffer descriptor with the
+// device-scope cache policy (sc1): stores are written through this XCD's L2 and loads do not hit
+// lines the L2 may hold from before, so data handed from one workgroup to another (possibly on
+// another XCD, with its own L2) needs no cache-wide write-back or invalidate -- only
+// "my stores are acknowledged" (s_waitcnt vmcnt(0)) before the counter that announces them.
+// The descriptor also bounds every access: lanes past the end of a piece load 0 and store nothing.
 // ------------------------------------------------------------------------------------------------
-template <bool STREAM> __device__ __forceinline__ u32x4 ld(const u32x4* p) {
-  return STREAM ? __builtin_nontemporal_load(p) : *p;
-}
-template <bool STREAM> __device__ __forceinline__ void st(u32x4* p, u32x4 v) {
-  if (STREAM) __builtin_nontemporal_store(v, p); else *p = v;
+#ifndef MSCCLX_AUX_STREAM
+#define MSCCLX_AUX_STREAM 16 /* sc1: rank buffers */
+#endif
+#ifndef MSCCLX_AUX_FIFO
+#define MSCCLX_AUX_FIFO 16 /* sc1: FIFO slots */
+#endif
+constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family dword 3)
+
+template <int W> struct Access;
+template <> struct Access<16> {
+  typedef u32x4 word;
+  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, AUX); }
+};
+template <> struct Access<8> {
+  typedef u32x2 word;
+  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, AUX); }
+};
+template <> struct Access<4> {
+  typedef unsigned int word;
+  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, AUX); }
+};
+template <> struct Access<2> {
+  typedef unsigned short word;
+  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b16(v, r, off, 0, AUX); }
+};
+template <> struct Access<1> {
+  typedef unsigned char word;
+  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b8(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b8(v, r, off, 0, AUX); }
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kBufferFlags);
 }
 
 constexpr int kUnroll = 4;
 
-template <class R, bool HAS_B, bool HAS_O2, bool SA, bool SB, bool SO1, bool SO2>
-__device__ __forceinline__ void move_vec(u32x4* o1, u32x4* o2, const u32x4* a, const u32x4* b, uint32_t n) {
+// out1[, out2] = a [(+) b] over n units of W bytes.  S* says which operands are rank buffers.
+template <class R, int W, bool HAS_B, bool HAS_O2, bool SA, bool SB, bool SO1, bool SO2>
+__device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n) {
+  typedef Access<W> A;
+  typedef typename A::word word;
+  constexpr int XA = SA ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO, XB = SB ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO;
+  constexpr int X1 = SO1 ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO, X2 = SO2 ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO;
+  const uint32_t bytes = n * W;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
   const uint32_t T = blockDim.x;
-  uint32_t i = threadIdx.x;
-  for (; i + (kUnroll - 1) * T < n; i += kUnroll * T) {
-    u32x4 x[kUnroll], y[kUnroll];
+  for (uint32_t i = threadIdx.x; i < n; i += kUnroll * T) {
+    word x[kUnroll], y[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) x[u] = ld<SA>(a + i + u * T);
+    for (int u = 0; u < kUnroll; ++u) x[u] = A::template ld<XA>(ra, (int)((i + u * T) * W));
     if (HAS_B) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) y[u] = ld<SB>(b + i + u * T);
+      for (int u = 0; u < kUnroll; ++u) y[u] = A::template ld<XB>(rb, (int)((i + u * T) * W));
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) x[u] = R::vec(y[u], x[u]);
+      for (int u = 0; u < kUnroll; ++u) x[u] = R::combine(y[u], x[u]);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) st<SO1>(o1 + i + u * T, x[u]);
+    for (int u = 0; u < kUnroll; ++u) A::template st<X1>(r1, (int)((i + u * T) * W), x[u]);
     if (HAS_O2) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) st<SO2>(o2 + i + u * T, x[u]);
+      for (int u = 0; u < kUnroll; ++u) A::template st<X2>(r2, (int)((i + u * T) * W), x[u]);
     }
-  }
-  for (; i < n; i += T) {
-    u32x4 x = ld<SA>(a + i);
-    if (HAS_B) x = R::vec(ld<SB>(b + i), x);
-    st<SO1>(o1 + i, x);
-    if (HAS_O2) st<SO2>(o2 + i, x);
-  }
-}
-
-template <class R, bool HAS_B, bool HAS_O2>
-__device__ __forceinline__ void move_elem(typename R::elem* o1, typename R::elem* o2,
-                                          const typename R::elem* a, const typename R::elem* b, uint32_t n) {
-  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
-    typename R::elem x = a[i];
-    if (HAS_B) x = R::one(b[i], x);
-    o1[i] = x;
-    if (HAS_O2) o2[i] = x;
   }
 }
 
@@ -207,17 +216,11 @@ __device__ __forceinline__ void move_elem(typename R::elem* o1, typename R::elem
 template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool SA, bool SB, bool SO1, bool SO2>
 __device__ __forceinline__ void move_rows(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b,
                                           int rows, uint32_t n, uint64_t stride) {
-  constexpr uint64_t UB = VEC ? 16 : sizeof(typename R::elem);
+  constexpr int W = VEC ? 16 : R::kElemBytes;
   for (int r = 0; r < rows; ++r) {
-    const uint64_t so = (uint64_t)r * stride * UB, fo = (uint64_t)r * n * UB;
-    unsigned char* p1 = o1 + (SO1 ? so : fo);
-    unsigned char* p2 = HAS_O2 ? o2 + (SO2 ? so : fo) : nullptr;
-    const unsigned char* pa = a + (SA ? so : fo);
-    const unsigned char* pb = HAS_B ? b + (SB ? so : fo) : nullptr;
-    if (VEC)
-      move_vec<R, HAS_B, HAS_O2, SA, SB, SO1, SO2>((u32x4*)p1, (u32x4*)p2, (const u32x4*)pa, (const u32x4*)pb, n);
-    else
-      move_elem<R, HAS_B, HAS_O2>((typename R::elem*)p1, (typename R::elem*)p2, (const typename R::elem*)pa, (const typename R::elem*)pb, n);
+    const uint64_t so = (uint64_t)r * stride * W, fo = (uint64_t)r * n * W;
+    move_units<R, W, HAS_B, HAS_O2, SA, SB, SO1, SO2>(o1 + (SO1 ? so : fo), HAS_O2 ? o2 + (SO2 ? so : fo) : nullptr,
+                                                      a + (SA ? so : fo), HAS_B ? b + (SB ? so : fo) : nullptr, n);
   }
 }
 
@@ -225,9 +228,6 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, unsigned char* o2, 
 // waiting
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ u64 load_counter(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-// Agent-scope release, spelled out: write this XCD's dirty L2 lines back and wait for the write-back
-// before any counter store that follows can be issued.
-__device__ __forceinline__ void release_agent() { asm volatile("buffer_wbl2 sc1\n\ts_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Called by the 64 lanes of wave 0.  Lane l < 3 waits for *addr[l] >= target[l] (null = nothing to
@@ -264,7 +264,7 @@ __device__ __forceinline__ int wait_conditions(const u64* a0, u64 t0, const u64*
 // ------------------------------------------------------------------------------------------------
 template <class R, bool VEC>
 __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
-  constexpr uint64_t UB = VEC ? 16 : sizeof(typename R::elem);
+  constexpr uint64_t UB = VEC ? 16 : R::kElemBytes;
   __shared__ int sh_fail;
   const int tbi = blockIdx.x / p.slices;
   const int j = blockIdx.x % p.slices;
@@ -336,9 +336,6 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
         }
         __syncthreads();
         if (sh_fail) return;
-        // every wave invalidates stale cache lines itself: the producer's data was written back
-        // before the counter wave 0 just saw
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
       }
 
       // ---- move data ----
@@ -368,12 +365,11 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
 
       // ---- publish ----
       if (rcv || snd || op.hasdep) {
-        // each wave waits until its own stores are acknowledged by L2, so that thread 0's release
-        // (L2 write-back + flag store) below covers the stores of every wave of the workgroup
+        // each wave waits until its own device-scope stores are acknowledged; after the barrier
+        // thread 0 may therefore announce the whole workgroup's data with plain counter stores
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (threadIdx.x == 0) {
-          release_agent();
           if (snd) publish(my_head, sseq + 1);
           if (rcv) publish(my_tail, rseq + 1);
           if (op.hasdep) publish(my_flag, pass * (u64)tb.nops + (u64)s + 1);
