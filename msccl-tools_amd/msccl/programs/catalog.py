@@ -1,0 +1,82 @@
+"""Complete programs: name -> XML, for the benchmark configurations and the tests.
+
+Each builder opens an MSCCLProgram with the collective, replication and threadblock policy the
+corresponding msccl-tools program is meant to run with, traces the algorithm, checks the
+collective's post-condition symbolically and returns the MSCCL-IR XML.
+"""
+from __future__ import annotations
+
+from msccl.language import MSCCLProgram, ThreadblockPolicy
+from msccl.language.collectives import AllGather, AllReduce, AllToAll
+from msccl.topologies import fully_connected
+
+
+def _finish(prog):
+    if not prog.check():
+        raise RuntimeError(f"program {prog.name} does not implement its collective")
+    return prog.generate_xml()
+
+
+def ring_allreduce(num_ranks, channels=1, instances=1, protocol="Simple"):
+    """msccl/programs/allreduce_a100_ring.py as registered in autosynth/ndv4_plans.py:24-32:
+    AllReduce(n, n, inplace), manual threadblocks."""
+    from msccl.programs.allreduce_a100_ring import allreduce_ring
+    prog = MSCCLProgram(f"allreduce_ring_{channels}channelsperring", fully_connected(num_ranks), AllReduce(num_ranks, num_ranks, True),
+                        instances, protocol=protocol, threadblock_policy=ThreadblockPolicy.manual)
+    with prog:
+        allreduce_ring(num_ranks, channels)
+    return _finish(prog)
+
+
+def ring_allgather(num_ranks, channels=1, instances=1, protocol="Simple"):
+    """examples/mscclang/allgather_ring.py:13-26: AllGather(n, 1, inplace), manual threadblocks."""
+    from msccl.programs.allgather_ring import allgather_ring
+    prog = MSCCLProgram(f"allgather_ring_{channels}channelsperring", fully_connected(num_ranks), AllGather(num_ranks, 1, True),
+                        instances, protocol=protocol, threadblock_policy=ThreadblockPolicy.manual)
+    with prog:
+        allgather_ring(num_ranks, channels)
+    return _finish(prog)
+
+
+def hierarchical_alltoall(num_nodes, gpus_per_node, instances=1, protocol="Simple"):
+    """examples/mscclang/alltoall_a100_two_step.py:8-48: AllToAll(n, 1, out of place), automatic
+    threadblocks."""
+    from msccl.programs.alltoall_a100_yifan import alltoall_hierarchical
+    n = num_nodes * gpus_per_node
+    prog = MSCCLProgram("hierarchical_all_to_all", fully_connected(n), AllToAll(n, 1, False), instances, protocol=protocol)
+    with prog:
+        alltoall_hierarchical(num_nodes, gpus_per_node)
+    return _finish(prog)
+
+
+def two_level_allreduce(num_local_gpus, num_nodes, instances=1, protocol="Simple", schedule="auto"):
+    """examples/mscclang/hierarchical_allreduce.py:26-77: AllReduce(n, n, inplace), batched
+    replication, automatic or manual channels."""
+    from msccl.programs.hierarchical_allreduce import hierarchical_allreduce
+    n = num_local_gpus * num_nodes
+    prog = MSCCLProgram("hierarchical_allreduce", fully_connected(n), AllReduce(n, n, True), instances, protocol=protocol,
+                        interleaved_replication=False)
+    with prog:
+        hierarchical_allreduce(num_local_gpus, num_nodes, schedule)
+    return _finish(prog)
+
+
+def allpairs_allreduce(num_ranks, instances=1, protocol="Simple", dependence_nop=True):
+    """msccl/programs/allreduce_allpairs.py as registered in autosynth/ndv4_plans.py:14-22."""
+    from msccl.programs.allreduce_allpairs import allreduce_allpairs
+    prog = MSCCLProgram("allreduce_allpairs", fully_connected(num_ranks), AllReduce(num_ranks, num_ranks * num_ranks, True), instances,
+                        protocol=protocol, threadblock_policy=ThreadblockPolicy.manual, interleaved_replication=False,
+                        dependence_nop=dependence_nop)
+    with prog:
+        allreduce_allpairs(num_ranks)
+    return _finish(prog)
+
+
+def three_step_alltoall(num_nodes, gpus_per_node, instances=1, protocol="Simple"):
+    """msccl/programs/alltoall_a100_8kp1.py: AllToAll(n, 1, out of place), automatic threadblocks."""
+    from msccl.programs.alltoall_a100_8kp1 import alltoall_three_step
+    n = num_nodes * gpus_per_node
+    prog = MSCCLProgram("alltoall_three_step", fully_connected(n), AllToAll(n, 1, False), 1, protocol=protocol)
+    with prog:
+        alltoall_three_step(num_nodes, gpus_per_node, instances=instances)
+    return _finish(prog)

@@ -110,3 +110,29 @@ def ring_allreduce_orders(n, nchunks=None, instances=1):
         base = [(index + k) % n for k in range(n)]
         orders.extend([base] * instances)
     return orders
+
+
+def two_level_allreduce_orders(num_local, num_nodes, instances=1):
+    """Fold order of msccl-tools' examples/mscclang/hierarchical_allreduce.py:13-19,38-44 with
+    num_local*num_nodes chunks: chunk q (b = q // num_nodes, j = q % num_nodes) is first summed
+    inside every node over local gpus b+1, b+2, ..., b (mod num_local), left to right, then the node
+    partials are summed over nodes j+1, j+2, ..., j (mod num_nodes), left to right.  Replication is
+    batched (rank_dag.py:339-340): chunk len*i + q of instance i follows chunk q."""
+    n = num_local * num_nodes
+    orders = []
+    for q in range(n):
+        b, j = q // num_nodes, q % num_nodes
+        nodes = [(j + 1 + m) % num_nodes for m in range(num_nodes)]
+        orders.append([[node * num_local + (b + 1 + k) % num_local for k in range(num_local)] for node in nodes])
+    return orders * instances
+
+
+def allpairs_allreduce_orders(n, instances=1):
+    """msccl-tools' msccl/programs/allreduce_allpairs.py:6-28 with n*n chunks: chunk r*n + lane is
+    folded on rank r as own value, then the peers' copies in ascending peer order (the order in
+    which they were appended to rank r's scratch).  Batched replication."""
+    orders = []
+    for c in range(n * n):
+        r = c // n
+        orders.append([r] + [p for p in range(n) if p != r])
+    return orders * instances

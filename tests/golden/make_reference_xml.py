@@ -1,0 +1,135 @@
+"""Writes tests/golden/reference_xml/*.xml.gz: MSCCL-IR emitted by msccl-tools' own MSCCLang compiler.
+
+Runs ONLY in the development container, where the msccl-tools checkout is mounted read-only at
+/root/reference; the GPU box has no such checkout and only ever sees the committed XML files.
+The fixtures are data (compiler output), used for two things no test of msccl-tools pins:
+  * the executor is fed IR the real compiler produced (not only IR from this package's compiler);
+  * this package's scheduler is compared, structurally, with the real one on auto-scheduled programs.
+
+msccl-tools imports lxml, z3 and humanfriendly at package import time; none is installed here.
+Only msccl.language and msccl.topologies are needed, so the top-level package is entered through an
+empty stand-in module object (its __init__ is not executed) and `lxml.etree` is served by the
+standard library's ElementTree, of which the emitter uses Element/SubElement/set/indent/tostring.
+
+usage: python tests/golden/make_reference_xml.py [/root/reference]
+"""
+import contextlib
+import gzip
+import io
+import os
+import runpy
+import sys
+import types
+import xml.etree.ElementTree as ET
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_xml")
+sys.dont_write_bytecode = True
+
+
+def install_entry_points():
+    pkg = types.ModuleType("msccl")
+    pkg.__path__ = [os.path.join(REF, "msccl")]
+    sys.modules["msccl"] = pkg
+    lxml = types.ModuleType("lxml")
+    lxml.etree = ET
+    sys.modules["lxml"] = lxml
+    sys.modules["lxml.etree"] = ET
+    sys.path.insert(0, REF)
+
+
+def normalise(xml):
+    return xml.replace(" />", "/>").strip() + "\n"
+
+
+def from_example(script, argv):
+    """Run an examples/mscclang script as __main__ and capture the XML it prints."""
+    old = sys.argv
+    sys.argv = [script] + [str(a) for a in argv]
+    buf = io.StringIO()
+    try:
+        with contextlib.redirect_stdout(buf):
+            runpy.run_path(os.path.join(REF, "examples", "mscclang", script), run_name="__main__")
+    finally:
+        sys.argv = old
+    text = buf.getvalue()
+    return normalise(text[text.index("<algo"):text.index("</algo>") + len("</algo>")])
+
+
+def from_program(build):
+    buf = io.StringIO()
+    with contextlib.redirect_stdout(buf):
+        build()
+    text = buf.getvalue()
+    return normalise(text[text.index("<algo"):text.index("</algo>") + len("</algo>")])
+
+
+def main():
+    install_entry_points()
+    from msccl.language import MSCCLProgram, XML, Check, ThreadblockPolicy
+    from msccl.language.collectives import AllReduce, AllToAll
+    from msccl.topologies import fully_connected
+
+    def ring(n, channels, instances):
+        from msccl.programs.allreduce_a100_ring import allreduce_ring
+        with MSCCLProgram("allreduce_ring", fully_connected(n), AllReduce(n, n, True), instances,
+                          threadblock_policy=ThreadblockPolicy.manual):
+            allreduce_ring(n, channels)
+            assert Check()
+            XML()
+
+    def allpairs(n, instances):
+        from msccl.programs.allreduce_allpairs import allreduce_allpairs
+        with MSCCLProgram("allreduce_allpairs", fully_connected(n), AllReduce(n, n * n, True), instances, protocol="LL",
+                          threadblock_policy=ThreadblockPolicy.manual, interleaved_replication=False, dependence_nop=True):
+            allreduce_allpairs(n)
+            assert Check()
+            XML()
+
+    def three_step(nodes, gpus):
+        from msccl.programs.alltoall_a100_8kp1 import alltoall_three_step
+        n = nodes * gpus
+        with MSCCLProgram("alltoall_three_step", fully_connected(n), AllToAll(n, 1, False), 1):
+            alltoall_three_step(nodes, gpus)
+            assert Check()
+            XML()
+
+    def registered_hierarchical(nodes):
+        from msccl.programs.alltoall_a100_yifan import alltoall_hierarchical
+        n = nodes * 8
+        with MSCCLProgram("hierarchical_all_to_all", fully_connected(n), AllToAll(n, 1, False), 1):
+            alltoall_hierarchical(nodes, 8)
+            assert Check()
+            XML()
+
+    jobs = {
+        "c1_allreduce_ring_8r_1ch_1inst": lambda: from_program(lambda: ring(8, 1, 1)),
+        "c2_allgather_ring_8r_1ch_4inst": lambda: from_example("allgather_ring.py", [8, 1, 4, "--protocol", "Simple"]),
+        "c3_alltoall_two_step_2x8": lambda: from_example("alltoall_a100_two_step.py", [2, 8]),
+        "c3_alltoall_registered_2x8": lambda: from_program(lambda: registered_hierarchical(2)),
+        "c4_hierarchical_allreduce_8x4_2inst_auto": lambda: from_example("hierarchical_allreduce.py", [8, 4, 2]),
+        "c4_hierarchical_allreduce_4x2_1inst_manual": lambda: from_example("hierarchical_allreduce.py", [4, 2, 1, "--schedule", "manual"]),
+        "c5_allreduce_ring_64r_1ch_1inst": lambda: from_program(lambda: ring(64, 1, 1)),
+        "allreduce_ring_8r_4ch_8inst": lambda: from_program(lambda: ring(8, 4, 8)),
+        "allreduce_allpairs_8r_2inst": lambda: from_program(lambda: allpairs(8, 2)),
+        "alltoall_three_step_3x4": lambda: from_program(lambda: three_step(3, 4)),
+        "allgather_recursive_doubling_8r": lambda: from_example("allgather_recursive_doubling.py", [8, 1]),
+        "allreduce_recursive_doubling_halving_8r": lambda: from_example("allreduce_recursive_doubling_halving.py", [8, 1]),
+        "allgather_allpairs_8r": lambda: from_example("allgather_allpairs.py", [8, 1]),
+        "allreduce_a100_allpairs_8r": lambda: from_example("allreduce_a100_allpairs.py", [8, 1]),
+        "alltoall_allpairs_4r": lambda: from_example("alltoall_allpairs.py", [4, 1]),
+    }
+    os.makedirs(OUT, exist_ok=True)
+    for name, job in jobs.items():
+        try:
+            xml = job()
+        except (SystemExit, Exception) as e:  # some examples are written against an older DSL and fail upstream too
+            print(f"{name}: skipped ({type(e).__name__}: {e})")
+            continue
+        with open(os.path.join(OUT, name + ".xml.gz"), "wb") as f:
+            f.write(gzip.compress(xml.encode(), 9, mtime=0))
+        print(f"{name}: {len(xml)} bytes")
+
+
+if __name__ == "__main__":
+    main()

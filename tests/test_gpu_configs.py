@@ -1,0 +1,120 @@
+"""The five benchmark configurations and every reference-emitted program on the GPU.
+
+Reduced sizes: HIP executor vs the NumPy interpreter, bit for bit, on IR from msccl-tools' compiler
+and from this package's compiler.  Full sizes: properties that need no CPU pass over the data --
+all-gather = concatenation, all-to-all = block transpose, all-reduce = the closed-form fold evaluated
+with torch's own bf16/fp16/fp32 arithmetic on the device, all compared bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+import golden_util
+from msccl.executor.workloads import WORKLOADS, numpy_input, torch_input
+from oracle import collectives as oc
+from oracle import ir_interp as oi
+from test_configs_oracle import GOLDEN_OF, OTHERS, fold_orders
+from test_gpu_parity import to_numpy, to_torch
+
+pytestmark = pytest.mark.gpu
+
+REDUCED = {"c1": 8 * 4 * 5000, "c2": 4 * 4 * 30000, "c3": 16 * 70000, "c4": 64 * 2 * 3000, "c5": 64 * 2 * 2048}
+
+
+def device_run(xml, w, inputs_np, **knobs):
+    from msccl.executor import Executor, collective_buffers
+    ex = Executor(xml)
+    print(f"case: {w.key} bytes/rank={w.bytes_per_rank} chunk_bytes={w.chunk_bytes} knobs={knobs}", flush=True)
+    info = ex.setup(w.chunk_bytes, w.dtype, **knobs)
+    ins, outs, res = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, inputs=[to_torch(v, w.dtype) for v in inputs_np])
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    return [to_numpy(r, w.dtype) for r in res], info
+
+
+def oracle_run(xml, w, inputs_np):
+    algo = oi.parse_xml(xml)
+    E = w.chunk_bytes // np.dtype(oi.DTYPES[w.dtype]).itemsize
+    bufs = oc.place_inputs(algo, inputs_np, E, w.dtype)
+    oi.Interpreter(algo).run(bufs, E, w.dtype)
+    return oc.extract_outputs(algo, bufs, E)
+
+
+@pytest.mark.parametrize("source", ["msccl-tools", "this-package"])
+@pytest.mark.parametrize("key", sorted(WORKLOADS))
+def test_config_reduced_size_vs_oracle(key, source):
+    w = WORKLOADS[key].scaled(REDUCED[key])
+    xml = golden_util.load(GOLDEN_OF[key]) if source == "msccl-tools" else WORKLOADS[key].build()
+    x = [numpy_input(w, r) for r in range(w.ranks)]
+    got, _ = device_run(xml, w, x)
+    want = oracle_run(xml, w, x)
+    for r in range(w.ranks):
+        assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
+
+
+@pytest.mark.parametrize("name", sorted(OTHERS))
+def test_reference_emitted_programs_vs_oracle(name):
+    from msccl.executor import Executor, collective_buffers
+    coll, n, _ = OTHERS[name]
+    xml = golden_util.load(name)
+    algo = oi.parse_xml(xml)
+    E = 3000
+    g0 = algo.gpus[0]
+    in_elems = (g0.o_chunks // n) * E if (coll == "allgather" and algo.inplace) else g0.i_chunks * E
+    rng = np.random.default_rng(5)
+    x = [(rng.random(in_elems, dtype=np.float32) * 2 - 1) for _ in range(n)]
+    bufs = oc.place_inputs(algo, x, E, "float32")
+    oi.Interpreter(algo).run(bufs, E, "float32")
+    want = oc.extract_outputs(algo, bufs, E)
+    ex = Executor(xml)
+    print(f"case: {name}", flush=True)
+    ex.setup(E * 4, "float32")
+    ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+    ex.run(ins, outs)
+    for r in range(n):
+        assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), (name, r)
+
+
+def torch_fold(order, operands):
+    if isinstance(order, int):
+        return operands[order]
+    acc = None
+    for item in order:
+        v = torch_fold(item, operands)
+        acc = v if acc is None else acc + v   # torch adds bf16/fp16 in fp32 and rounds to nearest even
+    return acc
+
+
+@pytest.mark.parametrize("key", sorted(WORKLOADS))
+def test_config_full_size_properties(key):
+    from msccl.executor import Executor, collective_buffers
+    w = WORKLOADS[key]
+    dev = "cuda:0"
+    xml = w.build()
+    ex = Executor(xml)
+    print(f"case: full-size {key}", flush=True)
+    info = ex.setup(w.chunk_bytes, w.dtype)
+    x = [torch_input(w, r, dev) for r in range(w.ranks)]
+    ins, outs, res = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, device=dev, inputs=x)
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    n = w.ranks
+    if w.coll == "allgather":
+        want = torch.cat(x)
+        for r in range(n):
+            assert torch.equal(res[r], want), r
+    elif w.coll == "alltoall":
+        blk = x[0].numel() // n
+        for r in range(n):
+            want = torch.cat([x[i][r * blk:(r + 1) * blk] for i in range(n)])
+            assert torch.equal(res[r], want), r
+    else:
+        E = x[0].numel() // w.nchunks
+        orders = fold_orders(key)
+        itype = torch.int32 if x[0].element_size() == 4 else torch.int16
+        for c in range(w.nchunks):
+            want = torch_fold(orders[c], [x[i][c * E:(c + 1) * E] for i in range(n)])
+            for r in range(n):
+                assert torch.equal(res[r][c * E:(c + 1) * E].view(itype), want.view(itype)), (c, r)
+    del x, ins, outs, res
+    torch.cuda.empty_cache()
