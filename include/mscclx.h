@@ -92,7 +92,8 @@ typedef struct {
   int32_t threads;     /* threads per workgroup: 64, 128, 256 or 512                             */
   int32_t timeout_ms;  /* in-kernel watchdog; default 10000                                      */
   int32_t max_workgroups; /* cap on resident workgroups assumed when no device is queried (tests) */
-  int32_t reserved[2];
+  int32_t staging;     /* 0: a receiver reads a payload in place where that is provably safe; 1: always stage in FIFO slots */
+  int32_t reserved[1];
 } mscclx_config;
 
 typedef struct {
@@ -104,6 +105,8 @@ typedef struct {
   int32_t passes;      /* passes of the step list the longest slice makes          */
   int32_t connections;
   int32_t vector_path; /* 1: 16-byte vector path, 0: element path                  */
+  int32_t zero_copy_messages; /* messages per pass read in place instead of staged  */
+  int32_t staged_messages;
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

@@ -21,8 +21,10 @@
 // word, all other workgroups see it in their own waits, and every wave leaves the kernel.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <utility>
 #include <string>
 #include <vector>
 
@@ -141,11 +143,8 @@ template <int DT, int OP> struct Reducer {
 // "my stores are acknowledged" (s_waitcnt vmcnt(0)) before the counter that announces them.
 // The descriptor also bounds every access: lanes past the end of a piece load 0 and store nothing.
 // ------------------------------------------------------------------------------------------------
-#ifndef MSCCLX_AUX_STREAM
-#define MSCCLX_AUX_STREAM 16 /* sc1: rank buffers */
-#endif
-#ifndef MSCCLX_AUX_FIFO
-#define MSCCLX_AUX_FIFO 16 /* sc1: FIFO slots */
+#ifndef MSCCLX_AUX
+#define MSCCLX_AUX 16 /* sc1 = device scope */
 #endif
 constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family dword 3)
 
@@ -180,15 +179,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kBufferFlags);
 }
 
-constexpr int kUnroll = 4;
+#ifndef MSCCLX_UNROLL
+#define MSCCLX_UNROLL 4
+#endif
+constexpr int kUnroll = MSCCLX_UNROLL;
 
-// out1[, out2] = a [(+) b] over n units of W bytes.  S* says which operands are rank buffers.
-template <class R, int W, bool HAS_B, bool HAS_O2, bool SA, bool SB, bool SO1, bool SO2>
+// out1[, out2] = a [(+) b] over n units of W bytes.
+template <class R, int W, bool HAS_B, bool HAS_O2>
 __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n) {
   typedef Access<W> A;
   typedef typename A::word word;
-  constexpr int XA = SA ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO, XB = SB ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO;
-  constexpr int X1 = SO1 ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO, X2 = SO2 ? MSCCLX_AUX_STREAM : MSCCLX_AUX_FIFO;
+  constexpr int X = MSCCLX_AUX;
   const uint32_t bytes = n * W;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
@@ -196,32 +197,32 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
   for (uint32_t i = threadIdx.x; i < n; i += kUnroll * T) {
     word x[kUnroll], y[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) x[u] = A::template ld<XA>(ra, (int)((i + u * T) * W));
+    for (int u = 0; u < kUnroll; ++u) x[u] = A::template ld<X>(ra, (int)((i + u * T) * W));
     if (HAS_B) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) y[u] = A::template ld<XB>(rb, (int)((i + u * T) * W));
+      for (int u = 0; u < kUnroll; ++u) y[u] = A::template ld<X>(rb, (int)((i + u * T) * W));
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) x[u] = R::combine(y[u], x[u]);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) A::template st<X1>(r1, (int)((i + u * T) * W), x[u]);
+    for (int u = 0; u < kUnroll; ++u) A::template st<X>(r1, (int)((i + u * T) * W), x[u]);
     if (HAS_O2) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) A::template st<X2>(r2, (int)((i + u * T) * W), x[u]);
+      for (int u = 0; u < kUnroll; ++u) A::template st<X>(r2, (int)((i + u * T) * W), x[u]);
     }
   }
 }
 
-// rows x n units; row r of a rank buffer is `stride` units further, row r of a FIFO slot is n units further.
-template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool SA, bool SB, bool SO1, bool SO2>
-__device__ __forceinline__ void move_rows(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b,
-                                          int rows, uint32_t n, uint64_t stride) {
+// rows x n units.  Consecutive rows of an operand are `stride_*` units apart: a chunk for rank
+// buffers, n for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
+// buffer, o2 (the forwarded copy) always a FIFO slot.
+template <class R, bool VEC, bool HAS_B, bool HAS_O2>
+__device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
+                                          const unsigned char* b, uint64_t stride_b, int rows, uint32_t n) {
   constexpr int W = VEC ? 16 : R::kElemBytes;
-  for (int r = 0; r < rows; ++r) {
-    const uint64_t so = (uint64_t)r * stride * W, fo = (uint64_t)r * n * W;
-    move_units<R, W, HAS_B, HAS_O2, SA, SB, SO1, SO2>(o1 + (SO1 ? so : fo), HAS_O2 ? o2 + (SO2 ? so : fo) : nullptr,
-                                                      a + (SA ? so : fo), HAS_B ? b + (SB ? so : fo) : nullptr, n);
-  }
+  for (int r = 0; r < rows; ++r)
+    move_units<R, W, HAS_B, HAS_O2>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
+                                    a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -339,26 +340,45 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
       }
 
       // ---- move data ----
+      // in: the incoming payload -- packed in a FIFO slot, or still where the sender has it (then
+      // rows are a chunk apart, like any rank buffer).  out: the FIFO slot to fill, or null when the
+      // receiver will read this step's payload in place.
       if (t != MSCCLX_OP_NOP) {
-        unsigned char* lsrc = nullptr;
+        const uint64_t cs = p.chunk_units;
+        const unsigned char* lsrc = nullptr;
         unsigned char* ldst = nullptr;
         if (t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE)
-          lsrc = (unsigned char*)p.bufs[op.src_slot] + ((uint64_t)op.srcoff * p.chunk_units + off) * UB;
+          lsrc = (const unsigned char*)p.bufs[op.src_slot] + ((uint64_t)op.srcoff * cs + off) * UB;
         if (t != MSCCLX_OP_SEND)
-          ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * p.chunk_units + off) * UB;
-        unsigned char* out = snd ? fifo_out + (sseq % (u64)p.depth) * slot_out * UB : nullptr;
-        const unsigned char* in = rcv ? fifo_in + (rseq % (u64)p.depth) * slot_in * UB : nullptr;
-        const uint64_t cs = p.chunk_units;
+          ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * cs + off) * UB;
+        unsigned char* out = (snd && op.out_staged) ? fifo_out + (sseq % (u64)p.depth) * slot_out * UB : nullptr;
+        const unsigned char* in = nullptr;
+        uint64_t in_stride = n;
+        if (rcv) {
+          if (op.in_slot >= 0) {
+            in = (const unsigned char*)p.bufs[op.in_slot] + ((uint64_t)op.in_off * cs + off) * UB;
+            in_stride = cs;
+          } else {
+            in = fifo_in + (rseq % (u64)p.depth) * slot_in * UB;
+          }
+        }
         switch (t) {
-          //                          R  VEC  HAS_B HAS_O2 SA     SB     SO1    SO2
-          case MSCCLX_OP_SEND:   move_rows<R, VEC, false, false, true,  false, false, false>(out, nullptr, lsrc, nullptr, op.cnt, n, cs); break;
-          case MSCCLX_OP_RECV:   move_rows<R, VEC, false, false, false, false, true,  false>(ldst, nullptr, in, nullptr, op.cnt, n, cs); break;
-          case MSCCLX_OP_RCS:    move_rows<R, VEC, false, true,  false, false, true,  false>(ldst, out, in, nullptr, op.cnt, n, cs); break;
-          case MSCCLX_OP_RRC:    move_rows<R, VEC, true,  false, false, true,  true,  false>(ldst, nullptr, in, ldst, op.cnt, n, cs); break;
-          case MSCCLX_OP_RRS:    move_rows<R, VEC, true,  false, false, true,  false, false>(out, nullptr, in, ldst, op.cnt, n, cs); break;
-          case MSCCLX_OP_RRCS:   move_rows<R, VEC, true,  true,  false, true,  true,  false>(ldst, out, in, ldst, op.cnt, n, cs); break;
-          case MSCCLX_OP_COPY:   move_rows<R, VEC, false, false, true,  false, true,  false>(ldst, nullptr, lsrc, nullptr, op.cnt, n, cs); break;
-          case MSCCLX_OP_REDUCE: move_rows<R, VEC, true,  false, true,  true,  true,  false>(ldst, nullptr, lsrc, ldst, op.cnt, n, cs); break;
+          case MSCCLX_OP_SEND:
+            if (out) move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
+            break;
+          case MSCCLX_OP_RECV: move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n); break;
+          case MSCCLX_OP_RCS:
+            if (out) move_rows<R, VEC, false, true>(ldst, cs, out, in, in_stride, nullptr, 0, op.cnt, n);
+            else     move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
+            break;
+          case MSCCLX_OP_RRC: move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
+          case MSCCLX_OP_RRS: move_rows<R, VEC, true, false>(out, n, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
+          case MSCCLX_OP_RRCS:
+            if (out) move_rows<R, VEC, true, true>(ldst, cs, out, in, in_stride, ldst, cs, op.cnt, n);
+            else     move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n);
+            break;
+          case MSCCLX_OP_COPY:   move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
+          case MSCCLX_OP_REDUCE: move_rows<R, VEC, true, false>(ldst, cs, nullptr, lsrc, cs, ldst, cs, op.cnt, n); break;
           default: break;
         }
       }
@@ -498,6 +518,10 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     info->passes = g.passes;
     info->connections = (int32_t)plan->conns.size();
     info->vector_path = g.vector_path;
+    info->zero_copy_messages = 0;
+    info->staged_messages = 0;
+    for (const Op& op : plan->ops)
+      if (is_send_type(op.type)) ((!g.staging && op.zero_copy) ? info->zero_copy_messages : info->staged_messages)++;
     info->workspace_bytes = g.workspace_bytes;
     info->algorithmic_units = plan->algorithmic_units;
   }
@@ -524,6 +548,19 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
       bufs[(size_t)r * 3 + b] = ptr;
     }
 
+  if (!g.staging) {
+    // reading payloads in place assumes that distinct buffers are distinct memory
+    std::vector<std::pair<uintptr_t, uintptr_t>> spans;
+    for (int r = 0; r < plan->nranks; ++r)
+      for (int b = 0; b < 3; ++b) {
+        const size_t len = (size_t)plan->rank_chunks[(size_t)r * 3 + b] * plan->chunk_bytes;
+        if (len) spans.push_back({(uintptr_t)bufs[(size_t)r * 3 + b], (uintptr_t)bufs[(size_t)r * 3 + b] + len});
+      }
+    std::sort(spans.begin(), spans.end());
+    for (size_t k = 1; k < spans.size(); ++k)
+      if (spans[k].first < spans[k - 1].second)
+        return fail(MSCCLX_ERR_INVALID_ARG, "rank buffers overlap in memory; configure the plan with staging=1 for aliased buffers");
+  }
   if (plan->dev) { destroy_device_state(plan->dev); plan->dev = nullptr; }
   DeviceState* d = new DeviceState();
   plan->dev = d;
@@ -538,7 +575,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   uint64_t fifo_off = 0;
   for (size_t c = 0; c < ncn; ++c) {
     hcn[c].fifo_off = fifo_off;
-    hcn[c].slot_units = (uint32_t)plan->conns[c].max_cnt * g.piece_units;
+    hcn[c].slot_units = (uint32_t)(g.staging ? plan->conns[c].max_cnt : plan->conns[c].max_staged_cnt) * g.piece_units;
     hcn[c].pad = 0;
     fifo_off += (uint64_t)g.depth * hcn[c].slot_units;
   }
@@ -558,6 +595,17 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
         dv.dep_nops = plan->tbs[dv.dep_tb].op_end - plan->tbs[dv.dep_tb].op_begin;
       }
       dv.hasdep = op.hasdep; dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
+      dv.in_slot = -1; dv.in_off = -1; dv.pad = 0;
+      dv.out_staged = is_send_type(op.type) && (g.staging || !op.zero_copy) ? 1 : 0;
+      if (is_recv_type(op.type) && !g.staging) {
+        const Op& sender = plan->ops[op.match_send];
+        if (sender.zero_copy) {  // read the payload where the sending rank keeps it
+          const int sender_rank = plan->tbs[plan->conns[tb.recv_conn].send_tb].rank;
+          const bool from_src = sender.type == MSCCLX_OP_SEND;
+          dv.in_slot = sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf);
+          dv.in_off = from_src ? sender.srcoff : sender.dstoff;
+        }
+      }
     }
   }
   HIP_TRY(hipMalloc((void**)&d->tbs, sizeof(DevTb) * (ntb ? ntb : 1)));

@@ -96,6 +96,80 @@ int simulate(const mscclx_plan& plan, int depth) {
   return MSCCLX_OK;
 }
 
+// Which messages need no FIFO slot.  The payload of a send-type step already sits at a fixed place on
+// the sending rank: the source chunks of an 's', or the local destination an 'rcs'/'rrcs' has just
+// written ('rrs' keeps no local copy, so its payload exists only in the slot).  The receiver may
+// read it from there if no step of the sending rank can overwrite those chunks before the matching
+// receive has run.  That is decided on the program's happens-before graph -- step order inside a
+// threadblock, depid/deps waits, and send -> matching receive -- which holds in every execution:
+// every later writer W of the chunks must be reachable from the matching receive R (then W cannot
+// start before R has finished), and every other writer must be an ancestor of the send.
+static void find_zero_copy_messages(mscclx_plan* p) {
+  const int n = (int)p->ops.size();
+  std::vector<int> tb_of(n), rank_of(n);
+  for (int t = 0; t < (int)p->tbs.size(); ++t)
+    for (int o = p->tbs[t].op_begin; o < p->tbs[t].op_end; ++o) { tb_of[o] = t; rank_of[o] = p->tbs[t].rank; }
+  std::vector<std::vector<int>> succ(n), pred(n);
+  auto edge = [&](int a, int b) { succ[a].push_back(b); pred[b].push_back(a); };
+  for (int t = 0; t < (int)p->tbs.size(); ++t) {
+    const Tb& tb = p->tbs[t];
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      if (o + 1 < tb.op_end) edge(o, o + 1);
+      const Op& op = p->ops[o];
+      if (op.depid >= 0) edge(p->tbs[p->rank_tb_begin[tb.rank] + op.depid].op_begin + op.deps, o);
+      if (is_send_type(op.type)) edge(o, op.match_recv);
+    }
+  }
+  // local writers per (rank, buffer)
+  struct Writer { int op, lo, hi; };
+  std::vector<std::vector<Writer>> writers((size_t)p->nranks * 3);
+  for (int o = 0; o < n; ++o) {
+    const Op& op = p->ops[o];
+    if (touches_local_dst(op.type) && op.type != MSCCLX_OP_RRS)
+      writers[(size_t)rank_of[o] * 3 + op.dstbuf].push_back({o, op.dstoff, op.dstoff + op.cnt});
+  }
+  std::vector<uint32_t> mark_back(n, 0), mark_fwd(n, 0);
+  uint32_t epoch = 0;
+  std::vector<int> stack;
+  auto reach = [&](int from, const std::vector<std::vector<int>>& adj, std::vector<uint32_t>& mark) {
+    stack.assign(1, from);
+    mark[from] = epoch;
+    while (!stack.empty()) {
+      int v = stack.back();
+      stack.pop_back();
+      for (int w : adj[v])
+        if (mark[w] != epoch) { mark[w] = epoch; stack.push_back(w); }
+    }
+  };
+  std::vector<int> later;
+  for (int s = 0; s < n; ++s) {
+    Op& op = p->ops[s];
+    if (!is_send_type(op.type) || op.type == MSCCLX_OP_RRS) continue;
+    const bool from_src = op.type == MSCCLX_OP_SEND;
+    const int buf = from_src ? op.srcbuf : op.dstbuf;
+    const int lo = from_src ? op.srcoff : op.dstoff, hi = lo + op.cnt;
+    later.clear();
+    for (const Writer& w : writers[(size_t)rank_of[s] * 3 + buf])
+      if (w.op != s && w.lo < hi && lo < w.hi) later.push_back(w.op);
+    if (!later.empty()) {
+      ++epoch;
+      reach(s, pred, mark_back);  // ancestors of the send wrote before it read
+      size_t k = 0;
+      for (int w : later)
+        if (mark_back[w] != epoch) later[k++] = w;
+      later.resize(k);
+    }
+    if (!later.empty()) {
+      reach(op.match_recv, succ, mark_fwd);
+      bool safe = true;
+      for (int w : later)
+        if (mark_fwd[w] != epoch) { safe = false; break; }
+      if (!safe) continue;
+    }
+    op.zero_copy = 1;
+  }
+}
+
 static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
   if (d->nranks <= 0 || d->ntbs < 0 || d->nops < 0) return fail(MSCCLX_ERR_INVALID_ARG, "negative table size");
   if (!d->rank_chunks || (d->ntbs && !d->tbs) || (d->nops && !d->ops)) return fail(MSCCLX_ERR_INVALID_ARG, "null table pointer");
@@ -229,8 +303,16 @@ static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
         return fail(MSCCLX_ERR_BAD_IR, name.str() + ": message " + std::to_string(p->ops[so].send_seq) + " is sent with cnt " + std::to_string(p->ops[so].cnt) +
                                            " but received with cnt " + std::to_string(p->ops[ro].cnt));
       cn.max_cnt = std::max(cn.max_cnt, p->ops[so].cnt);
+      p->ops[so].match_recv = ro;
+      p->ops[ro].match_send = so;
       ++ro;
     }
+  }
+  find_zero_copy_messages(p);
+  for (Conn& cn : p->conns) {
+    const Tb& s = p->tbs[cn.send_tb];
+    for (int so = s.op_begin; so < s.op_end; ++so)
+      if (is_send_type(p->ops[so].type) && !p->ops[so].zero_copy) cn.max_staged_cnt = std::max(cn.max_staged_cnt, p->ops[so].cnt);
   }
   return MSCCLX_OK;
 }
@@ -305,8 +387,9 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   }
   g.depth = depth;
 
+  g.staging = cfg.staging ? 1 : 0;
   uint64_t fifo_units = 0;
-  for (const Conn& c : plan.conns) fifo_units += (uint64_t)depth * c.max_cnt * g.piece_units;
+  for (const Conn& c : plan.conns) fifo_units += (uint64_t)depth * (g.staging ? c.max_cnt : c.max_staged_cnt) * g.piece_units;
   g.slice_fifo_units = fifo_units;
   g.sync_slice_words = (uint64_t)(plan.tbs.size() + 2 * plan.conns.size()) * kSyncStrideWords;
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;

@@ -13,6 +13,12 @@ struct Op {
   int32_t type, srcbuf, srcoff, dstbuf, dstoff, cnt, depid, deps, hasdep;
   int32_t send_seq = -1;  // position among this threadblock's send-type steps
   int32_t recv_seq = -1;  // position among this threadblock's recv-type steps
+  int32_t match_recv = -1;  // send-type steps: op row of the receive that takes this step's message
+  int32_t match_send = -1;  // recv-type steps: op row of the send whose message this step takes
+  // Send-type steps whose payload stays readable where it already is (the source of an 's', the
+  // local destination an 'rcs'/'rrcs' has just written) until the matching receive has consumed it:
+  // the receiver reads it from there and no FIFO slot is filled.
+  int32_t zero_copy = 0;
 };
 
 struct Tb {
@@ -29,6 +35,7 @@ struct Conn {
   int32_t send_tb = -1, recv_tb = -1;  // global threadblock rows
   int32_t nmsg = 0;                    // messages per pass
   int32_t max_cnt = 0;                 // largest message, in chunks
+  int32_t max_staged_cnt = 0;          // largest message that must go through a FIFO slot
 };
 
 inline bool is_send_type(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
@@ -46,6 +53,9 @@ struct DevOp {
   int32_t dep_nops;          // number of steps of the threadblock depended on
   int32_t hasdep;
   int32_t send_seq, recv_seq;
+  int32_t in_slot, in_off;   // recv-type: buffer-table index / chunk offset of the sender's payload, or -1: FIFO slot
+  int32_t out_staged;        // send-type: 1 = copy the payload into a FIFO slot, 0 = the receiver reads it in place
+  int32_t pad;
 };
 
 struct DevTb {
@@ -66,6 +76,7 @@ struct Geometry {
   uint32_t unit_bytes = 0;
   uint32_t piece_units = 0;
   int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
+  int32_t staging = 0;            // 1: every message goes through a FIFO slot
   int32_t passes = 0;
   uint64_t slice_fifo_units = 0;  // FIFO units one slice needs (all connections)
   uint64_t sync_words = 0;        // uint64 words of ONE synchronisation area (there are two)

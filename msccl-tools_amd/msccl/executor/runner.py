@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from .binding import DTYPE_SIZES, Plan
+from .binding import DTYPE_SIZES, MscclxError, Plan
 from .ir_tables import AlgoTables, parse_algo_xml
 
 _TORCH_NAMES = {torch.uint8: "uint8", torch.int8: "int8", torch.int32: "int32", torch.int64: "int64",
@@ -51,6 +51,7 @@ class Executor:
             raise RuntimeError("the MSCCL-IR executor needs a GPU; there is no CPU path")
         self.dtype = dtype_name(dtype)
         self.chunk_bytes = int(chunk_bytes)
+        self._setup_args = (chunk_bytes, dtype, redop, dict(knobs))
         with torch.cuda.device(self.device):
             self.info = self.plan.configure(self.chunk_bytes, self.dtype, redop, **knobs)
             t = self.tables
@@ -90,8 +91,20 @@ class Executor:
         ins = self._check_buffers(inputs, 0, "input")
         outs = self._check_buffers(outputs, 1, "output")
         scr = [0 if s is None else s.data_ptr() for s in self._scratch]
-        with torch.cuda.device(self.device):
-            self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
+        try:
+            with torch.cuda.device(self.device):
+                self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
+        except MscclxError as e:
+            if "overlap" not in e.message:
+                raise
+            # the caller aliases buffers the IR names separately (an in-place call): payloads can no
+            # longer be read in place, so every message goes through a FIFO slot
+            chunk_bytes, dtype, redop, knobs = self._setup_args
+            knobs["staging"] = 1
+            self.setup(chunk_bytes, dtype, redop, **knobs)
+            scr = [0 if t is None else t.data_ptr() for t in self._scratch]
+            with torch.cuda.device(self.device):
+                self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
         self._bound = key
         self._keepalive = (inputs, outputs)
 

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
 
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(binding.Config) == 32
-    assert ctypes.sizeof(binding.Info) == 48
+    assert ctypes.sizeof(binding.Info) == 56
     assert ctypes.sizeof(binding.Status) == 32
 
 
@@ -110,8 +110,14 @@ def test_geometry_without_a_device(mscclx_lib):
     assert info.passes == (8 << 20) // 16 // (64 * 1024)
     assert info.connections == 32
     assert info.algorithmic_units * (8 << 20) == 2 * 7 * 8 * (32 << 20)   # 2(n-1) n S_in
-    # FIFO: 32 connections x 16 slices x 4 slots x 64 KiB
-    assert info.workspace_bytes >= 32 * 16 * 4 * 64 * 1024
+    # every message of an all-gather can be read where the sender keeps it: no FIFO memory at all
+    assert (info.zero_copy_messages, info.staged_messages) == (7 * 32, 0)
+    assert info.workspace_bytes < 1 << 20
+    # with staging forced: 32 connections x 16 slices x 4 slots x 64 KiB of FIFO
+    staged = p.configure(8 << 20, "int32", max_workgroups=2048, staging=1)
+    assert (staged.zero_copy_messages, staged.staged_messages) == (0, 7 * 32)
+    assert staged.workspace_bytes >= 32 * 16 * 4 * 64 * 1024
+    info = p.configure(8 << 20, "int32", max_workgroups=2048)
     # element path when the chunk is not a multiple of 16 bytes
     info = p.configure(1000 * 4 + 4, "int32", max_workgroups=2048)
     assert info.vector_path == 0
@@ -130,3 +136,25 @@ def test_launch_before_bind_is_a_state_error(mscclx_lib):
     with pytest.raises(MscclxError) as e:
         p.launch()
     assert e.value.code == binding.ERR_STATE
+
+
+def test_zero_copy_analysis(mscclx_lib):
+    """Which payloads may be read in place (plan.cpp: find_zero_copy_messages)."""
+    def counts(xml):
+        info = Plan(parse_algo_xml(xml)).configure(1 << 20, "float32", max_workgroups=4096)
+        return info.zero_copy_messages, info.staged_messages
+    n = 8
+    # ring all-reduce: per chunk the first 's' (its source is overwritten only by the final value,
+    # which is causally after the receive), the 'rrcs' and the n-2 'rcs' keep their payload in
+    # place; the n-2 'rrs' results exist nowhere but in the slot
+    assert counts(ir_samples.ring_allreduce_xml(n)) == (n * (1 + 1 + (n - 2)), n * (n - 2))
+    # the fusion chain: s, rrcs, rcs in place; rrs staged
+    assert counts(ir_samples.FUSION_CHAIN_XML) == (3, 1)
+    # a sender that overwrites its source right after sending, with nothing ordering the overwrite
+    # after the receive, must stage
+    xml = ir_samples.RRC_CPY_NOP_XML.replace(
+        '<tb id="0" send="1" recv="-1" chan="0">\n' + ir_samples._step(0, "s", "i", 0, "i", 0, 1),
+        '<tb id="0" send="1" recv="-1" chan="0">\n' + ir_samples._step(0, "s", "i", 0, "i", 0, 1) + "\n" +
+        ir_samples._step(1, "cpy", "o", 0, "i", 0, 1)).replace('<gpu id="0" i_chunks="1" o_chunks="0"', '<gpu id="0" i_chunks="1" o_chunks="1"')
+    assert counts(ir_samples.RRC_CPY_NOP_XML) == (1, 0)
+    assert counts(xml) == (0, 1)

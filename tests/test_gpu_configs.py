@@ -40,13 +40,17 @@ def oracle_run(xml, w, inputs_np):
     return oc.extract_outputs(algo, bufs, E)
 
 
+@pytest.mark.parametrize("staging", [0, 1])
 @pytest.mark.parametrize("source", ["msccl-tools", "this-package"])
 @pytest.mark.parametrize("key", sorted(WORKLOADS))
-def test_config_reduced_size_vs_oracle(key, source):
+def test_config_reduced_size_vs_oracle(key, source, staging):
+    """staging=0: payloads are read in place where the plan proved that safe; staging=1: every
+    message is copied through a FIFO slot.  Both must give the interpreter's bits."""
     w = WORKLOADS[key].scaled(REDUCED[key])
     xml = golden_util.load(GOLDEN_OF[key]) if source == "msccl-tools" else WORKLOADS[key].build()
     x = [numpy_input(w, r) for r in range(w.ranks)]
-    got, _ = device_run(xml, w, x)
+    got, info = device_run(xml, w, x, staging=staging)
+    assert (info.zero_copy_messages == 0) == bool(staging)
     want = oracle_run(xml, w, x)
     for r in range(w.ranks):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
@@ -66,13 +70,14 @@ def test_reference_emitted_programs_vs_oracle(name):
     bufs = oc.place_inputs(algo, x, E, "float32")
     oi.Interpreter(algo).run(bufs, E, "float32")
     want = oc.extract_outputs(algo, bufs, E)
-    ex = Executor(xml)
-    print(f"case: {name}", flush=True)
-    ex.setup(E * 4, "float32")
-    ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
-    ex.run(ins, outs)
-    for r in range(n):
-        assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), (name, r)
+    for staging in (0, 1):
+        ex = Executor(xml)
+        print(f"case: {name} staging={staging}", flush=True)
+        ex.setup(E * 4, "float32", staging=staging)
+        ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+        ex.run(ins, outs)
+        for r in range(n):
+            assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), (name, r, staging)
 
 
 def torch_fold(order, operands):
@@ -118,3 +123,23 @@ def test_config_full_size_properties(key):
                 assert torch.equal(res[r][c * E:(c + 1) * E].view(itype), want.view(itype)), (c, r)
     del x, ins, outs, res
     torch.cuda.empty_cache()
+
+
+def test_aliased_buffers_fall_back_to_staging():
+    """An in-place call aliases the 'i' and 'o' buffers the IR names separately; reading payloads in
+    place is then unsound, bind refuses it and the runner re-plans with staging."""
+    from msccl.executor import Executor
+    xml = golden_util.load("alltoall_allpairs_4r")
+    E = 1024
+    ex = Executor(xml)
+    ex.setup(E * 4, "int32")
+    assert ex.info.zero_copy_messages > 0
+    n = 4
+    bufs = [torch.arange(n * E, dtype=torch.int32, device="cuda:0") + 100000 * r for r in range(n)]
+    shadow = [b.clone() for b in bufs]
+    outs = [torch.zeros(n * E, dtype=torch.int32, device="cuda:0") for _ in range(n)]
+    ex.run(shadow, outs)                       # out of place: the reference result
+    ex2 = Executor(xml)
+    ex2.setup(E * 4, "int32")
+    ex2.bind(bufs, [b[: n * E] for b in bufs])  # same memory for 'i' and 'o'
+    assert ex2.info.zero_copy_messages == 0 and ex2.info.staged_messages > 0
