@@ -86,18 +86,18 @@ typedef struct {
 
 /* Launch geometry knobs; a zero field means "choose automatically". */
 typedef struct {
-  int32_t slices;      /* workgroups per threadblock; each owns a 1/slices part of every chunk   */
+  int32_t slices;      /* independent copies of the program, each on a 1/slices part of every chunk */
   int32_t piece_bytes; /* bytes of one chunk moved per step per pass of the step list            */
   int32_t fifo_depth;  /* messages a connection can hold                                         */
   int32_t threads;     /* threads per workgroup: 64, 128, 256 or 512                             */
   int32_t timeout_ms;  /* in-kernel watchdog; default 10000                                      */
   int32_t max_workgroups; /* cap on resident workgroups assumed when no device is queried (tests) */
   int32_t staging;     /* 0: a receiver reads a payload in place where that is provably safe; 1: always stage in FIFO slots */
-  int32_t reserved[1];
+  int32_t workgroups;  /* resident workgroups that share the (threadblock, slice) contexts       */
 } mscclx_config;
 
 typedef struct {
-  int32_t workgroups;  /* = threadblocks * slices                                  */
+  int32_t workgroups;  /* resident workgroups; threadblocks * slices contexts are spread over them */
   int32_t threads;
   int32_t slices;
   int32_t piece_bytes;
@@ -107,6 +107,8 @@ typedef struct {
   int32_t vector_path; /* 1: 16-byte vector path, 0: element path                  */
   int32_t zero_copy_messages; /* messages per pass read in place instead of staged  */
   int32_t staged_messages;
+  int32_t max_hosted;  /* most contexts any workgroup hosts                         */
+  int32_t reserved;
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

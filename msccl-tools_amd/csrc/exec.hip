@@ -194,21 +194,23 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
   const uint32_t T = blockDim.x;
-  for (uint32_t i = threadIdx.x; i < n; i += kUnroll * T) {
-    word x[kUnroll], y[kUnroll];
+  // kUnroll loads are in flight per thread either way: all of a, or half of a and half of b
+  constexpr int UA = HAS_B ? (kUnroll / 2 > 0 ? kUnroll / 2 : 1) : kUnroll;
+  for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
+    word x[UA], y[UA];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) x[u] = A::template ld<X>(ra, (int)((i + u * T) * W));
+    for (int u = 0; u < UA; ++u) x[u] = A::template ld<X>(ra, (int)((i + u * T) * W));
     if (HAS_B) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) y[u] = A::template ld<X>(rb, (int)((i + u * T) * W));
+      for (int u = 0; u < UA; ++u) y[u] = A::template ld<X>(rb, (int)((i + u * T) * W));
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) x[u] = R::combine(y[u], x[u]);
+      for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) A::template st<X>(r1, (int)((i + u * T) * W), x[u]);
+    for (int u = 0; u < UA; ++u) A::template st<X>(r1, (int)((i + u * T) * W), x[u]);
     if (HAS_O2) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) A::template st<X>(r2, (int)((i + u * T) * W), x[u]);
+      for (int u = 0; u < UA; ++u) A::template st<X>(r2, (int)((i + u * T) * W), x[u]);
     }
   }
 }
@@ -226,179 +228,252 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
 }
 
 // ------------------------------------------------------------------------------------------------
-// waiting
+// the executor kernel
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ u64 load_counter(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-// Called by the 64 lanes of wave 0.  Lane l < 3 waits for *addr[l] >= target[l] (null = nothing to
-// wait for).  Returns -1 when all conditions hold, else the index of a condition that timed out (or 3
-// when another workgroup raised the abort word).
-__device__ __forceinline__ int wait_conditions(const u64* a0, u64 t0, const u64* a1, u64 t1, const u64* a2, u64 t2,
-                                               const u64* abort_word, u64 deadline) {
-  const int lane = threadIdx.x;
-  const u64* addr = lane == 0 ? a0 : lane == 1 ? a1 : lane == 2 ? a2 : nullptr;
-  const u64 target = lane == 0 ? t0 : lane == 1 ? t1 : t2;
-  int result = -1;
-  unsigned spins = 0;
-  for (;;) {
-    bool ok = true;
-    if (addr) ok = load_counter(addr) >= target;
-    if (__all(ok)) break;
-    __builtin_amdgcn_s_sleep(1);
-    if ((++spins & 0xffu) == 0) {
-      bool stop = false;
-      if (lane == 0) stop = load_counter(abort_word) != 0;
-      if (__any(stop)) { result = 3; break; }
-      if (wall_clock64() > deadline) {
-        const u64 bad = __ballot(!ok);
-        result = bad ? __ffsll((long long)bad) - 1 : 3;
-        break;
-      }
-    }
-  }
-  return result;
+__device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
+__device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
+
+// One hosted context = (threadblock, slice): the state of one lane of wave 0.
+struct Context {
+  int tb, slice, step, nops, op_begin, send_conn, recv_conn, nsend, nrecv;
+  unsigned pass, npasses;
+  bool active;
+  // the step the context stands at
+  bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
+  int type, hasdep;
+  u64 sseq, rseq;
+  const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
+  u64 t0, t1, t2;           // ... until they reach these values
+};
+
+__device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int slice) {
+  return base + kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words;
 }
 
-// ------------------------------------------------------------------------------------------------
-// the executor kernel
-// ------------------------------------------------------------------------------------------------
+// Describe the step `c` stands at: what it must wait for, and whether it moves data.
+__device__ __forceinline__ void describe_step(Context& c, const KernelParams& p) {
+  const DevOp* op = p.ops + c.op_begin + c.step;
+  u64* area = slice_area(p.sync_cur, p, c.slice);
+  const u64* flags = area;
+  const u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
+  const u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
+  c.type = op->type;
+  c.hasdep = op->hasdep;
+  const bool rcv = is_recv(c.type), snd = is_send(c.type);
+  c.sseq = snd ? (u64)c.pass * (u64)c.nsend + (u64)op->send_seq : 0;
+  c.rseq = rcv ? (u64)c.pass * (u64)c.nrecv + (u64)op->recv_seq : 0;
+  c.w0 = c.w1 = c.w2 = nullptr;
+  c.t0 = c.t1 = c.t2 = 0;
+  if (op->dep_tb >= 0) { c.w0 = flags + (uint64_t)op->dep_tb * kSyncStrideWords; c.t0 = (u64)c.pass * (u64)op->dep_nops + (u64)op->dep_step + 1; }
+  if (rcv) { c.w1 = heads + (uint64_t)c.recv_conn * kSyncStrideWords; c.t1 = c.rseq + 1; }
+  if (snd && c.sseq >= (u64)p.depth) { c.w2 = tails + (uint64_t)c.send_conn * kSyncStrideWords; c.t2 = c.sseq + 1 - (u64)p.depth; }
+  c.moves = !(c.type == MSCCLX_OP_NOP || (c.type == MSCCLX_OP_SEND && !op->out_staged));
+}
+
+// Announce the completed step and move the context to its next one.
+__device__ __forceinline__ void finish_step(Context& c, const KernelParams& p) {
+  u64* area = slice_area(p.sync_cur, p, c.slice);
+  u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
+  u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
+  if (is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, c.sseq + 1);
+  if (is_recv(c.type)) publish(tails + (uint64_t)c.recv_conn * kSyncStrideWords, c.rseq + 1);
+  if (c.hasdep) publish(area + (uint64_t)c.tb * kSyncStrideWords, (u64)c.pass * (u64)c.nops + (u64)c.step + 1);
+  if (++c.step == c.nops) { c.step = 0; ++c.pass; }
+  if (c.pass >= c.npasses) c.active = false;
+  else describe_step(c, p);
+}
+
+// A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
+// active context waits for (one round of loads covers all of them), finishes steps that move no data
+// on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
+// reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
+// share the resident workgroups without deadlock.
 template <class R, bool VEC>
 __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
   constexpr uint64_t UB = VEC ? 16 : R::kElemBytes;
-  __shared__ int sh_fail;
-  const int tbi = blockIdx.x / p.slices;
-  const int j = blockIdx.x % p.slices;
-  const DevTb tb = p.tbs[tbi];
-
-  u64* const area = p.sync_cur + kSyncHeaderWords + (uint64_t)j * p.sync_slice_words;
-  u64* const flags = area;
-  u64* const heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
-  u64* const tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
+  __shared__ int sh_choice, sh_tb, sh_slice, sh_step;
+  __shared__ unsigned sh_pass;
   const u64* const abort_word = p.sync_cur;
+  const int lane = threadIdx.x;
+  const bool poller = threadIdx.x < 64;
+  const int ctx_begin = p.wg_begin[blockIdx.x], hosted = p.wg_begin[blockIdx.x + 1] - ctx_begin;
 
-  if (threadIdx.x == 0) {
-    sh_fail = 0;
-    // clear, for the next launch, the counters this workgroup is the only writer of
-    u64* nxt = p.sync_nxt + kSyncHeaderWords + (uint64_t)j * p.sync_slice_words;
-    nxt[(uint64_t)tbi * kSyncStrideWords] = 0;
-    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
-    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
-    if (blockIdx.x == 0) p.sync_nxt[0] = 0;
+  Context c;
+  c.active = false;
+  if (poller && lane < hosted) {
+    c.tb = p.ctx_tb[ctx_begin + lane];
+    c.slice = p.ctx_slice[ctx_begin + lane];
+    const DevTb tb = p.tbs[c.tb];
+    c.nops = tb.nops; c.op_begin = tb.op_begin; c.send_conn = tb.send_conn; c.recv_conn = tb.recv_conn;
+    c.nsend = tb.nsend; c.nrecv = tb.nrecv;
+    c.step = 0; c.pass = 0;
+    const uint64_t u0 = p.chunk_units * (uint64_t)c.slice / p.slices, u1 = p.chunk_units * (uint64_t)(c.slice + 1) / p.slices;
+    c.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
+    c.active = c.nops > 0 && c.npasses > 0;
+    // clear, for the next launch, the counters this context is the only writer of
+    u64* nxt = slice_area(p.sync_nxt, p, c.slice);
+    nxt[(uint64_t)c.tb * kSyncStrideWords] = 0;
+    if (c.send_conn >= 0) nxt[((uint64_t)p.ntbs + c.send_conn) * kSyncStrideWords] = 0;
+    if (c.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + c.recv_conn) * kSyncStrideWords] = 0;
+    if (c.active) describe_step(c, p);
   }
-  __syncthreads();
+  if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
+  u64 deadline = wall_clock64() + p.timeout_ticks;  // pushed back whenever this workgroup makes progress
+  int cursor = 0;
+#ifdef MSCCLX_PROFILE
+  u64 prof_wait = 0, prof_move = 0;
+  const u64 prof_start = wall_clock64();
+#endif
 
-  // this slice's part of every chunk: units [u0, u1)
-  const uint64_t u0 = p.chunk_units * (uint64_t)j / p.slices;
-  const uint64_t u1 = p.chunk_units * (uint64_t)(j + 1) / p.slices;
-  unsigned char* const fifo_slice = p.fifo + (uint64_t)j * p.slice_fifo_units * UB;
-  unsigned char* fifo_out = nullptr;
-  const unsigned char* fifo_in = nullptr;
-  uint32_t slot_out = 0, slot_in = 0;
-  if (tb.send_conn >= 0) { fifo_out = fifo_slice + p.conns[tb.send_conn].fifo_off * UB; slot_out = p.conns[tb.send_conn].slot_units; }
-  if (tb.recv_conn >= 0) { fifo_in = fifo_slice + p.conns[tb.recv_conn].fifo_off * UB; slot_in = p.conns[tb.recv_conn].slot_units; }
-  u64* const my_flag = flags + (uint64_t)tbi * kSyncStrideWords;
-  u64* const my_head = tb.send_conn >= 0 ? heads + (uint64_t)tb.send_conn * kSyncStrideWords : nullptr;
-  u64* const my_tail = tb.recv_conn >= 0 ? tails + (uint64_t)tb.recv_conn * kSyncStrideWords : nullptr;
-  const u64* const peer_tail = tb.send_conn >= 0 ? tails + (uint64_t)tb.send_conn * kSyncStrideWords : nullptr;
-  const u64* const peer_head = tb.recv_conn >= 0 ? heads + (uint64_t)tb.recv_conn * kSyncStrideWords : nullptr;
-  const u64 deadline = wall_clock64() + p.timeout_ticks;
-
-  u64 pass = 0;
-  for (uint64_t off = u0; off < u1; off += p.piece_units, ++pass) {
-    const uint32_t n = (uint32_t)((u1 - off) < (uint64_t)p.piece_units ? (u1 - off) : (uint64_t)p.piece_units);
-    for (int s = 0; s < tb.nops; ++s) {
-      const DevOp op = p.ops[tb.op_begin + s];
-      const int t = op.type;
-      const bool rcv = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS;
-      const bool snd = t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS;
-      const u64 sseq = snd ? pass * (u64)tb.nsend + (u64)op.send_seq : 0;
-      const u64 rseq = rcv ? pass * (u64)tb.nrecv + (u64)op.recv_seq : 0;
-
-      // ---- wait: dependency, incoming message, free outgoing slot ----
-      const u64* a0 = nullptr; u64 t0 = 0;
-      const u64* a1 = nullptr; u64 t1 = 0;
-      const u64* a2 = nullptr; u64 t2 = 0;
-      if (op.dep_tb >= 0) { a0 = flags + (uint64_t)op.dep_tb * kSyncStrideWords; t0 = pass * (u64)op.dep_nops + (u64)op.dep_step + 1; }
-      if (rcv) { a1 = peer_head; t1 = rseq + 1; }
-      if (snd && sseq >= (u64)p.depth) { a2 = peer_tail; t2 = sseq + 1 - (u64)p.depth; }
-      if (a0 || a1 || a2) {
-        if (threadIdx.x < 64) {
-          const int w = wait_conditions(a0, t0, a1, t1, a2, t2, abort_word, deadline);
-          if (w >= 0 && threadIdx.x == 0) {
-            sh_fail = 1;
-            if (w < 3 && atomicCAS((u64*)abort_word, 0ull, 1ull) == 0ull) {
-              mscclx_status* hs = p.host_status;
-              hs->tb = tbi; hs->step = s; hs->slice = j; hs->pass = (int64_t)pass; hs->waiting_on = w;
-              __threadfence_system();
-              __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  for (;;) {
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t0 = wall_clock64();
+#endif
+    if (poller) {
+      int choice = -2;
+      unsigned spins = 0;
+      while (choice == -2) {
+        bool ready = false;
+        if (c.active) {
+          ready = true;
+          if (c.w0) ready = load_counter(c.w0) >= c.t0;
+          if (ready && c.w1) ready = load_counter(c.w1) >= c.t1;
+          if (ready && c.w2) ready = load_counter(c.w2) >= c.t2;
+        }
+        bool progressed = false;
+        if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
+          finish_step(c, p);
+          progressed = true;
+        }
+        const u64 movers = __ballot(ready && c.moves && c.active);
+        if (movers) {
+          const u64 from_cursor = movers & ~((cursor >= 64) ? ~0ull : ((1ull << cursor) - 1ull));
+          choice = __ffsll((long long)(from_cursor ? from_cursor : movers)) - 1;
+        } else if (!__any(c.active)) {
+          choice = -1;  // every hosted context has run to its end
+        } else if (__any(progressed)) {
+          deadline = wall_clock64() + p.timeout_ticks;
+        } else {
+          __builtin_amdgcn_s_sleep(1);
+          if ((++spins & 0x3fu) == 0) {
+            bool stop = false;
+            if (lane == 0) stop = load_counter(abort_word) != 0;
+            if (__any(stop)) { choice = -3; }
+            else if (wall_clock64() > deadline) {
+              // report the first context that is still waiting
+              const u64 stuck = __ballot(c.active);
+              const int who = __ffsll((long long)stuck) - 1;
+              if (lane == who && atomicCAS((u64*)abort_word, 0ull, 1ull) == 0ull) {
+                int what = 3;
+                if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
+                else if (c.w1 && load_counter(c.w1) < c.t1) what = 1;
+                else if (c.w2 && load_counter(c.w2) < c.t2) what = 2;
+                mscclx_status* hs = p.host_status;
+                hs->tb = c.tb; hs->step = c.step; hs->slice = c.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
+                __threadfence_system();
+                __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+              }
+              choice = -3;
             }
           }
         }
-        __syncthreads();
-        if (sh_fail) return;
       }
+      if (choice >= 0 && lane == choice) { sh_tb = c.tb; sh_slice = c.slice; sh_step = c.step; sh_pass = c.pass; }
+      if (lane == 0) sh_choice = choice;
+      cursor = choice >= 0 ? (choice + 1) & 63 : cursor;
+    }
+    __syncthreads();
+    const int choice = sh_choice;
+    if (choice < 0) break;  // done (-1) or giving up (-3); uniform for the workgroup
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t1 = wall_clock64();
+#endif
 
-      // ---- move data ----
+    // ---- the chosen context's step: move one piece ----
+    {
+      const int tbi = sh_tb, j = sh_slice;
+      const u64 pass = sh_pass;
+      const DevTb tb = p.tbs[tbi];
+      const DevOp op = p.ops[tb.op_begin + sh_step];
+      const int t = op.type;
+      const bool rcv = is_recv(t), snd = is_send(t);
+      const uint64_t cs = p.chunk_units;
+      const uint64_t u0 = cs * (uint64_t)j / p.slices, u1 = cs * (uint64_t)(j + 1) / p.slices;
+      const uint64_t off = u0 + pass * (uint64_t)p.piece_units;
+      const uint32_t n = (uint32_t)((u1 - off) < (uint64_t)p.piece_units ? (u1 - off) : (uint64_t)p.piece_units);
+      unsigned char* const fifo_slice = p.fifo + (uint64_t)j * p.slice_fifo_units * UB;
+      const unsigned char* lsrc = nullptr;
+      unsigned char* ldst = nullptr;
+      if (t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE)
+        lsrc = (const unsigned char*)p.bufs[op.src_slot] + ((uint64_t)op.srcoff * cs + off) * UB;
+      if (t != MSCCLX_OP_SEND)
+        ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * cs + off) * UB;
+      // out: the FIFO slot to fill, or null when the receiver will read this step's payload in place
+      unsigned char* out = nullptr;
+      if (snd && op.out_staged) {
+        const DevConn cn = p.conns[tb.send_conn];
+        const u64 sseq = pass * (u64)tb.nsend + (u64)op.send_seq;
+        out = fifo_slice + (cn.fifo_off + (sseq % (u64)p.depth) * cn.slot_units) * UB;
+      }
       // in: the incoming payload -- packed in a FIFO slot, or still where the sender has it (then
-      // rows are a chunk apart, like any rank buffer).  out: the FIFO slot to fill, or null when the
-      // receiver will read this step's payload in place.
-      if (t != MSCCLX_OP_NOP) {
-        const uint64_t cs = p.chunk_units;
-        const unsigned char* lsrc = nullptr;
-        unsigned char* ldst = nullptr;
-        if (t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE)
-          lsrc = (const unsigned char*)p.bufs[op.src_slot] + ((uint64_t)op.srcoff * cs + off) * UB;
-        if (t != MSCCLX_OP_SEND)
-          ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * cs + off) * UB;
-        unsigned char* out = (snd && op.out_staged) ? fifo_out + (sseq % (u64)p.depth) * slot_out * UB : nullptr;
-        const unsigned char* in = nullptr;
-        uint64_t in_stride = n;
-        if (rcv) {
-          if (op.in_slot >= 0) {
-            in = (const unsigned char*)p.bufs[op.in_slot] + ((uint64_t)op.in_off * cs + off) * UB;
-            in_stride = cs;
-          } else {
-            in = fifo_in + (rseq % (u64)p.depth) * slot_in * UB;
-          }
-        }
-        switch (t) {
-          case MSCCLX_OP_SEND:
-            if (out) move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
-            break;
-          case MSCCLX_OP_RECV: move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n); break;
-          case MSCCLX_OP_RCS:
-            if (out) move_rows<R, VEC, false, true>(ldst, cs, out, in, in_stride, nullptr, 0, op.cnt, n);
-            else     move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
-            break;
-          case MSCCLX_OP_RRC: move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
-          case MSCCLX_OP_RRS: move_rows<R, VEC, true, false>(out, n, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
-          case MSCCLX_OP_RRCS:
-            if (out) move_rows<R, VEC, true, true>(ldst, cs, out, in, in_stride, ldst, cs, op.cnt, n);
-            else     move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n);
-            break;
-          case MSCCLX_OP_COPY:   move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
-          case MSCCLX_OP_REDUCE: move_rows<R, VEC, true, false>(ldst, cs, nullptr, lsrc, cs, ldst, cs, op.cnt, n); break;
-          default: break;
+      // its rows are a chunk apart, like any rank buffer)
+      const unsigned char* in = nullptr;
+      uint64_t in_stride = n;
+      if (rcv) {
+        if (op.in_slot >= 0) {
+          in = (const unsigned char*)p.bufs[op.in_slot] + ((uint64_t)op.in_off * cs + off) * UB;
+          in_stride = cs;
+        } else {
+          const DevConn cn = p.conns[tb.recv_conn];
+          const u64 rseq = pass * (u64)tb.nrecv + (u64)op.recv_seq;
+          in = fifo_slice + (cn.fifo_off + (rseq % (u64)p.depth) * cn.slot_units) * UB;
         }
       }
-
-      // ---- publish ----
-      if (rcv || snd || op.hasdep) {
-        // each wave waits until its own device-scope stores are acknowledged; after the barrier
-        // thread 0 may therefore announce the whole workgroup's data with plain counter stores
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (threadIdx.x == 0) {
-          if (snd) publish(my_head, sseq + 1);
-          if (rcv) publish(my_tail, rseq + 1);
-          if (op.hasdep) publish(my_flag, pass * (u64)tb.nops + (u64)s + 1);
-        }
-      } else if (t != MSCCLX_OP_NOP) {
-        __syncthreads();  // a later step of this threadblock may read what this one wrote
+      switch (t) {
+        case MSCCLX_OP_SEND: move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
+        case MSCCLX_OP_RECV: move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n); break;
+        case MSCCLX_OP_RCS:
+          if (out) move_rows<R, VEC, false, true>(ldst, cs, out, in, in_stride, nullptr, 0, op.cnt, n);
+          else     move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
+          break;
+        case MSCCLX_OP_RRC: move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
+        case MSCCLX_OP_RRS: move_rows<R, VEC, true, false>(out, n, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
+        case MSCCLX_OP_RRCS:
+          if (out) move_rows<R, VEC, true, true>(ldst, cs, out, in, in_stride, ldst, cs, op.cnt, n);
+          else     move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n);
+          break;
+        case MSCCLX_OP_COPY:   move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
+        case MSCCLX_OP_REDUCE: move_rows<R, VEC, true, false>(ldst, cs, nullptr, lsrc, cs, ldst, cs, op.cnt, n); break;
+        default: break;
       }
     }
+    // every wave waits until its own device-scope stores are acknowledged; after the barrier the
+    // polling wave may announce the whole workgroup's data with plain counter stores
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (poller) {
+      if (lane == choice) finish_step(c, p);
+      deadline = wall_clock64() + p.timeout_ticks;
+    }
+#ifdef MSCCLX_PROFILE
+    if (threadIdx.x == 0) {
+      const u64 prof_t2 = wall_clock64();
+      prof_wait += prof_t1 - prof_t0;
+      prof_move += prof_t2 - prof_t1;
+    }
+#endif
   }
+#ifdef MSCCLX_PROFILE
+  if (threadIdx.x == 0 && p.prof) {
+    p.prof[(size_t)blockIdx.x * 4 + 0] = prof_wait;
+    p.prof[(size_t)blockIdx.x * 4 + 1] = prof_move;
+    p.prof[(size_t)blockIdx.x * 4 + 2] = wall_clock64() - prof_start;
+    p.prof[(size_t)blockIdx.x * 4 + 3] = prof_start;
+  }
+#endif
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -440,12 +515,14 @@ struct DeviceState {
   DevOp* ops = nullptr;
   DevConn* conns = nullptr;
   void** bufs = nullptr;
+  int32_t* hosting = nullptr;            // wg_begin | ctx_tb | ctx_slice
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
   kernel_fn kernel = nullptr;
   unsigned launches = 0;
   bool dirty = false;  // counters must be cleared before the next launch (after a failed launch)
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: 4 words per workgroup
 };
 
 void destroy_device_state(DeviceState* d) {
@@ -454,6 +531,7 @@ void destroy_device_state(DeviceState* d) {
   if (d->ops) (void)hipFree(d->ops);
   if (d->conns) (void)hipFree(d->conns);
   if (d->bufs) (void)hipFree(d->bufs);
+  if (d->hosting) (void)hipFree(d->hosting);
   if (d->host_status) (void)hipHostFree(d->host_status);
   if (d->ev0) (void)hipEventDestroy(d->ev0);
   if (d->ev1) (void)hipEventDestroy(d->ev1);
@@ -500,9 +578,11 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     if (rc) return rc;
   }
   Geometry g;
-  int rc = decide_geometry(*plan, chunk_bytes, dtype, cfg, num_cus, capacity, &g);
+  const uint64_t fifo_budget = 2ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes
+  int rc = decide_geometry(*plan, chunk_bytes, dtype, cfg, num_cus, capacity, fifo_budget, &g);
   if (rc) return rc;
-  plan->geo = g;
+  plan->geo = std::move(g);
+  const Geometry& gg = plan->geo;
   plan->chunk_bytes = chunk_bytes;
   plan->dtype = dtype;
   plan->redop = redop;
@@ -510,7 +590,10 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   plan->configured = true;
   if (plan->dev) { destroy_device_state(plan->dev); plan->dev = nullptr; }
   if (info) {
-    info->workgroups = (int32_t)plan->tbs.size() * g.slices;
+    const Geometry& g = gg;
+    info->workgroups = g.workgroups;
+    info->max_hosted = g.max_hosted;
+    info->reserved = 0;
     info->threads = g.threads;
     info->slices = g.slices;
     info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);
@@ -616,6 +699,13 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipMemcpy(d->ops, hop.data(), sizeof(DevOp) * nop, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d->conns, hcn.data(), sizeof(DevConn) * hcn.size(), hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d->bufs, bufs.data(), sizeof(void*) * bufs.size(), hipMemcpyHostToDevice));
+  {
+    std::vector<int32_t> table(g.wg_begin);
+    table.insert(table.end(), g.ctx_tb.begin(), g.ctx_tb.end());
+    table.insert(table.end(), g.ctx_slice.begin(), g.ctx_slice.end());
+    HIP_TRY(hipMalloc((void**)&d->hosting, sizeof(int32_t) * table.size()));
+    HIP_TRY(hipMemcpy(d->hosting, table.data(), sizeof(int32_t) * table.size(), hipMemcpyHostToDevice));
+  }
   HIP_TRY(hipHostMalloc((void**)&d->host_status, sizeof(mscclx_status), hipHostMallocDefault));
   std::memset(d->host_status, 0, sizeof(mscclx_status));
   d->workspace = (unsigned char*)workspace;
@@ -623,6 +713,9 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipDeviceSynchronize());
   HIP_TRY(hipEventCreate(&d->ev0));
   HIP_TRY(hipEventCreate(&d->ev1));
+#ifdef MSCCLX_PROFILE
+  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * 4 * g.workgroups));
+#endif
   return MSCCLX_OK;
 }
 
@@ -646,13 +739,17 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
   kp.sync_nxt = sync + (uint64_t)(parity ^ 1u) * g.sync_words;
   kp.fifo = d->workspace + g.fifo_byte_off;
   kp.host_status = d->host_status;
+  kp.prof = d->prof;
   kp.chunk_units = g.chunk_units;
   kp.slice_fifo_units = g.slice_fifo_units;
   kp.sync_slice_words = g.sync_slice_words;
   kp.timeout_ticks = (uint64_t)plan->timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan->tbs.size(); kp.nconns = (int)plan->conns.size();
-  const unsigned grid = (unsigned)plan->tbs.size() * (unsigned)g.slices;
+  kp.wg_begin = d->hosting;
+  kp.ctx_tb = d->hosting + g.wg_begin.size();
+  kp.ctx_slice = kp.ctx_tb + g.ctx_tb.size();
+  const unsigned grid = (unsigned)g.workgroups;
   hipLaunchKernelGGL(d->kernel, dim3(grid), dim3(g.threads), 0, s, kp);
   HIP_TRY(hipGetLastError());
   d->launches++;
@@ -669,6 +766,23 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
   }
   mscclx_status st = *d->host_status;
   if (status) *status = st;
+#ifdef MSCCLX_PROFILE
+  if (d->prof && getenv("MSCCLX_PROFILE_DUMP")) {
+    const size_t nwg = plan->geo.workgroups;
+    std::vector<unsigned long long> h(nwg * 4);
+    (void)hipMemcpy(h.data(), d->prof, h.size() * 8, hipMemcpyDeviceToHost);
+    double sw = 0, sm = 0, st_ = 0; unsigned long long first = ~0ull, last = 0; size_t worst = 0;
+    for (size_t w = 0; w < nwg; ++w) {
+      sw += h[w * 4]; sm += h[w * 4 + 1]; st_ += h[w * 4 + 2];
+      if (h[w * 4 + 3] < first) first = h[w * 4 + 3];
+      if (h[w * 4 + 3] + h[w * 4 + 2] > last) last = h[w * 4 + 3] + h[w * 4 + 2];
+      if (h[w * 4 + 1] > h[worst * 4 + 1]) worst = w;
+    }
+    fprintf(stderr, "[prof] wgs=%zu span=%.1f us  mean per wg: wait %.1f us move %.1f us total %.1f us | busiest wg %zu (tb %zu): wait %.1f move %.1f total %.1f us\n",
+            nwg, (last - first) / 100.0, sw / nwg / 100, sm / nwg / 100, st_ / nwg / 100, worst, (size_t)0,
+            h[worst * 4] / 100.0, h[worst * 4 + 1] / 100.0, h[worst * 4 + 2] / 100.0);
+  }
+#endif
   if (st.code != MSCCLX_OK) {
     d->dirty = true;
     const Tb& tb = plan->tbs[st.tb];

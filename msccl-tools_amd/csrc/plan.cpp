@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <queue>
 #include <sstream>
 #include <tuple>
 
@@ -321,82 +322,164 @@ static int thread_index(int threads) {
   switch (threads) { case 64: return 0; case 128: return 1; case 256: return 2; case 512: return 3; default: return -1; }
 }
 
+// bytes a threadblock moves per chunk-sized unit of its steps, given which payloads are staged
+static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
+  uint64_t w = 0;
+  for (int o = tb.op_begin; o < tb.op_end; ++o) {
+    const Op& op = plan.ops[o];
+    const bool staged_out = is_send_type(op.type) && (staging || !op.zero_copy);
+    int units = 0;
+    switch (op.type) {
+      case MSCCLX_OP_SEND: units = staged_out ? 2 : 0; break;
+      case MSCCLX_OP_RECV: case MSCCLX_OP_COPY: units = 2; break;
+      case MSCCLX_OP_RCS: units = staged_out ? 3 : 2; break;
+      case MSCCLX_OP_RRC: case MSCCLX_OP_RRS: case MSCCLX_OP_REDUCE: units = 3; break;
+      case MSCCLX_OP_RRCS: units = staged_out ? 4 : 3; break;
+      default: break;
+    }
+    w += (uint64_t)units * op.cnt;
+  }
+  return w;
+}
+
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
-                    int num_cus, const int capacity_by_threads[4], Geometry* out) {
+                    int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);
   if (!elem) return fail(MSCCLX_ERR_INVALID_ARG, "unknown dtype " + std::to_string(dtype));
   if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
+  if (cfg.slices < 0 || cfg.piece_bytes < 0 || cfg.fifo_depth < 0 || cfg.workgroups < 0 || cfg.threads < 0)
+    return fail(MSCCLX_ERR_INVALID_ARG, "geometry knobs must be >= 0");
   Geometry g;
   g.vector_path = (chunk_bytes % 16 == 0) ? 1 : 0;
   g.unit_bytes = g.vector_path ? 16 : elem;
   g.chunk_units = chunk_bytes / g.unit_bytes;
-  const int ntbs = (int)plan.tbs.size();
+  g.staging = cfg.staging ? 1 : 0;
+  const int64_t ntbs = (int64_t)plan.tbs.size();
   if (ntbs == 0) return fail(MSCCLX_ERR_BAD_IR, "the algorithm has no threadblocks");
 
-  // threads per workgroup: as asked, else the largest of 256/128/64 with which every threadblock is resident
-  int threads = cfg.threads;
-  if (threads) {
-    if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
-  } else {
-    threads = 256;
-    while (threads > 64 && capacity_by_threads[thread_index(threads)] < ntbs) threads /= 2;
-  }
-  const int capacity = capacity_by_threads[thread_index(threads)];
-  if (capacity < ntbs)
-    return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks must be resident at once but only " + std::to_string(capacity) +
-                                         " workgroups of " + std::to_string(threads) + " threads fit on the device");
-  g.threads = threads;
-
-  // slices: enough workgroups to cover the chip a few times, never cutting a chunk below 2 KiB
-  const uint64_t min_slice_units = std::max<uint64_t>(1, 2048 / g.unit_bytes);
-  const int64_t max_by_size = (int64_t)std::max<uint64_t>(1, g.chunk_units / min_slice_units);
-  int64_t slices = cfg.slices;
-  if (slices < 0) return fail(MSCCLX_ERR_INVALID_ARG, "slices must be >= 0");
-  if (!slices) {
-    const int64_t target = std::min<int64_t>(capacity, (int64_t)2 * num_cus);
-    slices = std::max<int64_t>(1, target / ntbs);
-    slices = std::min(slices, max_by_size);
-    if (slices >= 8) slices -= slices % 8;
-  }
-  if ((uint64_t)slices > g.chunk_units) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");
-  if (slices * (int64_t)ntbs > capacity)
-    return fail(MSCCLX_ERR_CAPACITY, std::to_string(slices * (int64_t)ntbs) + " workgroups requested but only " + std::to_string(capacity) + " can be resident");
-  g.slices = (int)slices;
-
-  const uint64_t longest_slice = (g.chunk_units + slices - 1) / slices;
-  int64_t piece_bytes = cfg.piece_bytes;
-  if (piece_bytes < 0) return fail(MSCCLX_ERR_INVALID_ARG, "piece_bytes must be >= 0");
-  if (!piece_bytes) piece_bytes = 64 * 1024;
-  uint64_t piece_units = std::max<uint64_t>(1, (uint64_t)piece_bytes / g.unit_bytes);
-  piece_units = std::min(piece_units, longest_slice);
-  if (piece_units > 0x7fffffffu / 64) return fail(MSCCLX_ERR_INVALID_ARG, "piece too large");
-  g.piece_units = (uint32_t)piece_units;
-  g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
-
+  // connection depth: as asked (must not deadlock), else the smallest that works, at least 2
   int depth = cfg.fifo_depth;
-  if (depth < 0) return fail(MSCCLX_ERR_INVALID_ARG, "fifo_depth must be >= 0");
   if (depth) {
     int rc = simulate(plan, depth);
     if (rc) return rc;
   } else {
     depth = 1;
-    while (simulate(plan, depth) != MSCCLX_OK) {
+    while (simulate(plan, depth) != MSCCLX_OK)
       if (++depth > 4096) return fail(MSCCLX_ERR_DEADLOCK, "the program does not finish with any connection depth up to 4096");
-    }
-    depth = std::max(depth, 4);
+    depth = std::max(depth, 2);
   }
   g.depth = depth;
 
-  g.staging = cfg.staging ? 1 : 0;
-  uint64_t fifo_units = 0;
-  for (const Conn& c : plan.conns) fifo_units += (uint64_t)depth * (g.staging ? c.max_cnt : c.max_staged_cnt) * g.piece_units;
-  g.slice_fifo_units = fifo_units;
+  // Slices are independent copies of the program on 1/slices of every chunk; they are what keeps
+  // the chip busy while one copy waits on its dependency chain.  Aim at pieces of about 256 KiB,
+  // bounded by what the resident workgroups can host.
+  const int most_threads_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
+  const int64_t host_limit = (int64_t)most_threads_capacity * kMaxHosted;
+  if (ntbs > host_limit)
+    return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
+  int64_t slices = cfg.slices;
+  if (!slices) {
+    const uint64_t target_piece = 256 * 1024;
+    slices = (int64_t)std::max<uint64_t>(1, chunk_bytes / target_piece);
+    // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~16
+    const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 16) / ntbs);
+    slices = std::min(slices, comfortable);
+    slices = std::min<int64_t>(slices, 64);
+  }
+  slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
+  if (slices < 1 || (cfg.slices && (uint64_t)cfg.slices > g.chunk_units)) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");
+  if (slices * ntbs > host_limit) {
+    if (cfg.slices) return fail(MSCCLX_ERR_CAPACITY, std::to_string(slices * ntbs) + " contexts requested but the device can host only " + std::to_string(host_limit));
+    slices = std::max<int64_t>(1, host_limit / ntbs);
+  }
+  g.slices = (int)slices;
+
+  // piece: the whole slice in one pass unless the FIFO slots of staged messages would not fit the budget
+  const uint64_t longest_slice = (g.chunk_units + slices - 1) / slices;
+  uint64_t piece_units = cfg.piece_bytes ? std::max<uint64_t>(1, (uint64_t)cfg.piece_bytes / g.unit_bytes) : longest_slice;
+  piece_units = std::min(piece_units, longest_slice);
+  uint64_t slot_chunks = 0;  // FIFO units per slice per unit of piece
+  for (const Conn& c : plan.conns) slot_chunks += (uint64_t)depth * (g.staging ? c.max_cnt : c.max_staged_cnt);
+  if (!cfg.piece_bytes && slot_chunks) {
+    const uint64_t cap = fifo_budget_bytes / (slot_chunks * (uint64_t)slices * g.unit_bytes);
+    const uint64_t floor_units = std::max<uint64_t>(1, 16384 / g.unit_bytes);
+    piece_units = std::min(piece_units, std::max(cap, std::min(floor_units, longest_slice)));
+  }
+  if (piece_units > 0x3fffffffu / 16) piece_units = 0x3fffffffu / 16;
+  g.piece_units = (uint32_t)piece_units;
+  g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
+
+  // threads: enough to cover a piece with 8 16-byte loads per thread
+  int threads = cfg.threads;
+  if (threads) {
+    if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
+  } else {
+    const uint64_t piece_bytes = piece_units * g.unit_bytes;
+    threads = piece_bytes >= 64 * 1024 ? 512 : piece_bytes >= 32 * 1024 ? 256 : piece_bytes >= 16 * 1024 ? 128 : 64;
+    while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
+  }
+  const int capacity = capacity_by_threads[thread_index(threads)];
+  if (capacity < 1) return fail(MSCCLX_ERR_CAPACITY, "no workgroup of " + std::to_string(threads) + " threads fits on the device");
+  g.threads = threads;
+
+  // resident workgroups: about 16 waves per compute unit, never more than contexts or capacity
+  const int64_t contexts = slices * ntbs;
+  int64_t wgs = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
+  wgs = std::min<int64_t>(wgs, contexts);
+  if (wgs > capacity) {
+    if (cfg.workgroups) return fail(MSCCLX_ERR_CAPACITY, std::to_string(wgs) + " workgroups requested but only " + std::to_string(capacity) + " can be resident");
+    wgs = capacity;
+  }
+  if (wgs * kMaxHosted < contexts) {
+    if (cfg.workgroups || cfg.slices)
+      return fail(MSCCLX_ERR_CAPACITY, std::to_string(contexts) + " contexts cannot be hosted by " + std::to_string(wgs) + " workgroups of " +
+                                           std::to_string(kMaxHosted) + " contexts each");
+    wgs = std::min<int64_t>(capacity, (contexts + kMaxHosted - 1) / kMaxHosted);
+    if (wgs * kMaxHosted < contexts) return fail(MSCCLX_ERR_CAPACITY, "too many contexts for the resident workgroups");
+  }
+  g.workgroups = (int)wgs;
+
+  // Hosting table: longest-processing-time first -- contexts by decreasing work onto the least
+  // loaded workgroup that still has a free lane.
+  struct Ctx { uint64_t work; int tb, slice; };
+  std::vector<Ctx> ctxs;
+  ctxs.reserve((size_t)contexts);
+  for (int t = 0; t < (int)ntbs; ++t) {
+    const uint64_t w = tb_work(plan, plan.tbs[t], g.staging != 0);
+    for (int j = 0; j < (int)slices; ++j) ctxs.push_back({w, t, j});
+  }
+  std::stable_sort(ctxs.begin(), ctxs.end(), [](const Ctx& a, const Ctx& b) { return a.work > b.work; });
+  std::vector<std::vector<int>> hosted((size_t)wgs);
+  typedef std::pair<uint64_t, int> Load;  // (work so far, workgroup)
+  std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+  for (int w = 0; w < (int)wgs; ++w) heap.push({0, w});
+  for (size_t k = 0; k < ctxs.size(); ++k) {
+    Load l = heap.top();
+    heap.pop();
+    hosted[l.second].push_back((int)k);
+    // +1 so that contexts without data movement are spread too
+    if ((int)hosted[l.second].size() < kMaxHosted) heap.push({l.first + ctxs[k].work + 1, l.second});
+    if (heap.empty() && k + 1 < ctxs.size()) return fail(MSCCLX_ERR_CAPACITY, "hosting table overflow");
+  }
+  g.wg_begin.assign(1, 0);
+  g.max_hosted = 0;
+  for (int w = 0; w < (int)wgs; ++w) {
+    // a workgroup polls its contexts lane by lane; keep slices of one threadblock in slice order
+    std::sort(hosted[w].begin(), hosted[w].end(), [&](int a, int b) {
+      return ctxs[a].slice != ctxs[b].slice ? ctxs[a].slice < ctxs[b].slice : ctxs[a].tb < ctxs[b].tb;
+    });
+    for (int k : hosted[w]) { g.ctx_tb.push_back(ctxs[k].tb); g.ctx_slice.push_back(ctxs[k].slice); }
+    g.wg_begin.push_back((int32_t)g.ctx_tb.size());
+    g.max_hosted = std::max<int32_t>(g.max_hosted, (int32_t)hosted[w].size());
+  }
+
+  g.slice_fifo_units = slot_chunks * g.piece_units;
   g.sync_slice_words = (uint64_t)(plan.tbs.size() + 2 * plan.conns.size()) * kSyncStrideWords;
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
   const uint64_t sync_bytes = (2 * g.sync_words * 8 + 255) / 256 * 256;
   g.fifo_byte_off = sync_bytes;
-  g.workspace_bytes = sync_bytes + fifo_units * g.slices * g.unit_bytes + 256;
-  *out = g;
+  g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * g.unit_bytes + 256;
+  *out = std::move(g);
   return MSCCLX_OK;
 }
 

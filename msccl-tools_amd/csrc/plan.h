@@ -77,6 +77,9 @@ struct Geometry {
   uint32_t piece_units = 0;
   int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
   int32_t staging = 0;            // 1: every message goes through a FIFO slot
+  int32_t workgroups = 0;         // resident workgroups; each hosts up to kMaxHosted (threadblock, slice) contexts
+  int32_t max_hosted = 0;
+  std::vector<int32_t> wg_begin, ctx_tb, ctx_slice;  // the hosting table
   int32_t passes = 0;
   uint64_t slice_fifo_units = 0;  // FIFO units one slice needs (all connections)
   uint64_t sync_words = 0;        // uint64 words of ONE synchronisation area (there are two)
@@ -94,14 +97,19 @@ struct KernelParams {
   unsigned long long* sync_nxt; // next launch's counters (cleared by this launch)
   unsigned char* fifo;
   mscclx_status* host_status;   // pinned host memory
+  unsigned long long* prof;     // per-workgroup tick counters of MSCCLX_PROFILE builds, else null
   uint64_t chunk_units;
   uint64_t slice_fifo_units;
   uint64_t sync_slice_words;
   uint64_t timeout_ticks;
   uint32_t piece_units;
   int32_t slices, depth, ntbs, nconns;
+  const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
+  const int32_t* ctx_tb;        // hosted contexts, grouped by workgroup: threadblock row ...
+  const int32_t* ctx_slice;     // ... and slice
 };
 
+constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
 
@@ -138,6 +146,6 @@ int dtype_size(int dtype);
 int simulate(const mscclx_plan& plan, int depth);
 // Pure geometry decision (no HIP): max_wgs = resident workgroup capacity per thread count.
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
-                    int num_cus, const int capacity_by_threads[4], Geometry* out);
+                    int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out);
 void destroy_device_state(DeviceState* d);
 }  // namespace mscclx

@@ -53,7 +53,7 @@ class PlanDesc(ctypes.Structure):
 class Config(ctypes.Structure):
     _fields_ = [("slices", ctypes.c_int32), ("piece_bytes", ctypes.c_int32), ("fifo_depth", ctypes.c_int32),
                 ("threads", ctypes.c_int32), ("timeout_ms", ctypes.c_int32), ("max_workgroups", ctypes.c_int32),
-                ("staging", ctypes.c_int32), ("reserved", ctypes.c_int32 * 1)]
+                ("staging", ctypes.c_int32), ("workgroups", ctypes.c_int32)]
 
 
 class Info(ctypes.Structure):
@@ -61,6 +61,7 @@ class Info(ctypes.Structure):
                 ("piece_bytes", ctypes.c_int32), ("fifo_depth", ctypes.c_int32), ("passes", ctypes.c_int32),
                 ("connections", ctypes.c_int32), ("vector_path", ctypes.c_int32),
                 ("zero_copy_messages", ctypes.c_int32), ("staged_messages", ctypes.c_int32),
+                ("max_hosted", ctypes.c_int32), ("reserved", ctypes.c_int32),
                 ("workspace_bytes", ctypes.c_uint64), ("algorithmic_units", ctypes.c_uint64)]
 
     def as_dict(self):

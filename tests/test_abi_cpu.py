@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
 
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(binding.Config) == 32
-    assert ctypes.sizeof(binding.Info) == 56
+    assert ctypes.sizeof(binding.Info) == 64
     assert ctypes.sizeof(binding.Status) == 32
 
 
@@ -104,27 +104,37 @@ def test_dependency_cycle_is_a_deadlock(mscclx_lib):
 def test_geometry_without_a_device(mscclx_lib):
     p = Plan(parse_algo_xml(ir_samples.ring_allgather_xml(8, 4)))  # 32 threadblocks
     info = p.configure(8 << 20, "int32", max_workgroups=2048)
-    assert info.vector_path == 1 and info.threads == 256
-    assert info.slices == 16 and info.workgroups == 512          # 2 workgroups per CU of a 256-CU part
-    assert info.piece_bytes == 64 * 1024 and info.fifo_depth == 4
-    assert info.passes == (8 << 20) // 16 // (64 * 1024)
-    assert info.connections == 32
+    assert info.vector_path == 1
+    # 256 KiB pieces: 32 slices of every 8 MiB chunk, each done in one pass by a 512-thread workgroup
+    assert (info.slices, info.piece_bytes, info.passes, info.threads) == (32, 256 * 1024, 1, 512)
+    # 32 x 32 contexts shared by 16 waves per CU of a 256-CU part
+    assert (info.workgroups, info.max_hosted) == (512, 2)
+    assert info.fifo_depth == 2 and info.connections == 32
     assert info.algorithmic_units * (8 << 20) == 2 * 7 * 8 * (32 << 20)   # 2(n-1) n S_in
     # every message of an all-gather can be read where the sender keeps it: no FIFO memory at all
     assert (info.zero_copy_messages, info.staged_messages) == (7 * 32, 0)
-    assert info.workspace_bytes < 1 << 20
-    # with staging forced: 32 connections x 16 slices x 4 slots x 64 KiB of FIFO
+    assert info.workspace_bytes < 2 << 20
+    # with staging forced: 32 connections x 32 slices x 2 slots x 256 KiB of FIFO
     staged = p.configure(8 << 20, "int32", max_workgroups=2048, staging=1)
     assert (staged.zero_copy_messages, staged.staged_messages) == (0, 7 * 32)
-    assert staged.workspace_bytes >= 32 * 16 * 4 * 64 * 1024
-    info = p.configure(8 << 20, "int32", max_workgroups=2048)
+    assert staged.workspace_bytes >= 32 * 32 * 2 * 256 * 1024
+    # a FIFO budget of 2 GiB splits bigger pieces into passes
+    big = p.configure(512 << 20, "int32", max_workgroups=2048, staging=1)
+    assert big.passes > 1 and big.workspace_bytes <= (2 << 30) + (8 << 20)
+    # explicit knobs
+    k = p.configure(8 << 20, "int32", max_workgroups=2048, slices=16, piece_bytes=65536, fifo_depth=4, threads=256, workgroups=128)
+    assert (k.slices, k.piece_bytes, k.passes, k.fifo_depth, k.threads, k.workgroups, k.max_hosted) == (16, 65536, 8, 4, 256, 128, 4)
     # element path when the chunk is not a multiple of 16 bytes
     info = p.configure(1000 * 4 + 4, "int32", max_workgroups=2048)
-    assert info.vector_path == 0
+    assert info.vector_path == 0 and info.slices == 1
     with pytest.raises(MscclxError):
         p.configure(6, "int32", max_workgroups=2048)              # not a multiple of the element
+    # more threadblocks than workgroups is fine: a workgroup hosts up to 64 contexts ...
+    few = p.configure(8 << 20, "int32", max_workgroups=16)
+    assert few.workgroups == 16 and few.max_hosted * 16 >= few.slices * 32
+    # ... but not more than that
     with pytest.raises(MscclxError) as e:
-        p.configure(8 << 20, "int32", max_workgroups=16)          # 32 threadblocks cannot be resident
+        p.configure(8 << 20, "int32", max_workgroups=16, slices=64)
     assert e.value.code == binding.ERR_CAPACITY
     with pytest.raises(MscclxError) as e:
         p.configure(8 << 20, "int32", max_workgroups=2048, fifo_depth=1)
