@@ -1,24 +1,27 @@
 // MI355X (gfx950) executor kernels for MSCCL-IR and the device half of the C ABI.
 //
 // Execution model.  All ranks of the algorithm are virtual ranks whose buffers live in this GPU's
-// HBM.  Every <tb> of every rank is run by `slices` persistent workgroups; workgroup (tb, j) owns
-// the j-th 1/slices part of EVERY chunk, which is legal because every IR step is element-wise, and
-// makes the parts fully independent (own FIFOs, own counters).  A workgroup walks its step list once
-// per "pass"; a pass moves one piece (piece_units) of each chunk its steps name, so a connection's
-// message is cnt pieces and fits a bounded FIFO slot in HBM whatever the chunk size.
+// HBM.  The program is run as `slices` independent copies, copy j on the j-th 1/slices part of
+// EVERY chunk -- legal because every IR step is element-wise -- each with its own FIFOs and counters.
+// A context is one <tb> in one slice; it walks its step list once per "pass", a pass moving one piece
+// (piece_units) of each chunk its steps name.  Contexts are spread over a fixed number of resident
+// workgroups; a workgroup hosts up to 64 of them, polls what all of them wait for in one round of
+// loads (one lane of wave 0 per context), and runs whichever is ready, so it never blocks on one
+// context and the number of threadblocks is not tied to what fits on the chip.
 //
-// Synchronisation (all counters monotone, 64-bit, one per 64 bytes, agent scope):
+// Synchronisation (all counters monotone, 64-bit, one per 64 bytes, agent scope, per slice):
 //   flag[tb]   = pass*nsteps + step + 1 of the last finished step with hasdep=1     (depid/deps wait)
 //   head[conn] = messages produced;  tail[conn] = messages consumed                  (FIFO hand-off)
-// Wave 0 polls up to three conditions at once, one per lane; a barrier releases the other waves.
 // Payload is read and written with device-scope (sc1) accesses only, so a producer publishes by
 // waiting for its stores to be acknowledged, a workgroup barrier, and a counter store; a consumer
 // reads the payload after its poll succeeds.  No cache-wide write-back or invalidate is issued.
+// A receiver reads a payload where the sender keeps it when the plan proved that safe; only the
+// other messages are copied through FIFO slots in HBM.
 // Two counter areas alternate between launches: a launch clears the area the next launch will
 // use, so no memset sits between launches.
 //
-// Every wait is bounded by a wall-clock watchdog; on expiry the workgroup raises the area's abort
-// word, all other workgroups see it in their own waits, and every wave leaves the kernel.
+// A workgroup that makes no progress for the watchdog period raises the area's abort word; all
+// other workgroups see it while they poll, and every wave leaves the kernel.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -180,7 +183,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 }
 
 #ifndef MSCCLX_UNROLL
-#define MSCCLX_UNROLL 4
+#define MSCCLX_UNROLL 8
 #endif
 constexpr int kUnroll = MSCCLX_UNROLL;
 
@@ -347,6 +350,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
           finish_step(c, p);
           progressed = true;
+          ready = false;  // the context now stands at another step, whose conditions are not yet known
         }
         const u64 movers = __ballot(ready && c.moves && c.active);
         if (movers) {
@@ -578,7 +582,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     if (rc) return rc;
   }
   Geometry g;
-  const uint64_t fifo_budget = 2ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes
+  const uint64_t fifo_budget = 4ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes
   int rc = decide_geometry(*plan, chunk_bytes, dtype, cfg, num_cus, capacity, fifo_budget, &g);
   if (rc) return rc;
   plan->geo = std::move(g);

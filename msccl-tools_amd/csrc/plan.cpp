@@ -379,12 +379,15 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
   int64_t slices = cfg.slices;
   if (!slices) {
-    const uint64_t target_piece = 256 * 1024;
-    slices = (int64_t)std::max<uint64_t>(1, chunk_bytes / target_piece);
+    // big chunks: pieces of about 128 KiB amortise the per-step hand-off; small chunks: enough
+    // slices that every compute unit has a context or two, but no piece below 2 KiB
+    const int64_t by_piece = (int64_t)(chunk_bytes / (128 * 1024));
+    const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;
+    slices = std::max<int64_t>(1, std::max(by_piece, to_fill));
+    slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
     // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~16
     const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 16) / ntbs);
     slices = std::min(slices, comfortable);
-    slices = std::min<int64_t>(slices, 64);
   }
   slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
   if (slices < 1 || (cfg.slices && (uint64_t)cfg.slices > g.chunk_units)) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");

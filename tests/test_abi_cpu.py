@@ -105,22 +105,22 @@ def test_geometry_without_a_device(mscclx_lib):
     p = Plan(parse_algo_xml(ir_samples.ring_allgather_xml(8, 4)))  # 32 threadblocks
     info = p.configure(8 << 20, "int32", max_workgroups=2048)
     assert info.vector_path == 1
-    # 256 KiB pieces: 32 slices of every 8 MiB chunk, each done in one pass by a 512-thread workgroup
-    assert (info.slices, info.piece_bytes, info.passes, info.threads) == (32, 256 * 1024, 1, 512)
-    # 32 x 32 contexts shared by 16 waves per CU of a 256-CU part
-    assert (info.workgroups, info.max_hosted) == (512, 2)
+    # 128 KiB pieces: 64 slices of every 8 MiB chunk, each done in one pass by a 512-thread workgroup
+    assert (info.slices, info.piece_bytes, info.passes, info.threads) == (64, 128 * 1024, 1, 512)
+    # 32 x 64 contexts shared by 16 waves per CU of a 256-CU part
+    assert (info.workgroups, info.max_hosted) == (512, 4)
     assert info.fifo_depth == 2 and info.connections == 32
     assert info.algorithmic_units * (8 << 20) == 2 * 7 * 8 * (32 << 20)   # 2(n-1) n S_in
     # every message of an all-gather can be read where the sender keeps it: no FIFO memory at all
     assert (info.zero_copy_messages, info.staged_messages) == (7 * 32, 0)
     assert info.workspace_bytes < 2 << 20
-    # with staging forced: 32 connections x 32 slices x 2 slots x 256 KiB of FIFO
+    # with staging forced: 32 connections x 64 slices x 2 slots x 128 KiB of FIFO
     staged = p.configure(8 << 20, "int32", max_workgroups=2048, staging=1)
     assert (staged.zero_copy_messages, staged.staged_messages) == (0, 7 * 32)
-    assert staged.workspace_bytes >= 32 * 32 * 2 * 256 * 1024
-    # a FIFO budget of 2 GiB splits bigger pieces into passes
-    big = p.configure(512 << 20, "int32", max_workgroups=2048, staging=1)
-    assert big.passes > 1 and big.workspace_bytes <= (2 << 30) + (8 << 20)
+    assert staged.workspace_bytes >= 32 * 64 * 2 * 128 * 1024
+    # a FIFO budget of 4 GiB splits bigger pieces into passes
+    big = p.configure(1 << 30, "int32", max_workgroups=2048, staging=1)
+    assert big.passes > 1 and big.workspace_bytes <= (4 << 30) + (8 << 20)
     # explicit knobs
     k = p.configure(8 << 20, "int32", max_workgroups=2048, slices=16, piece_bytes=65536, fifo_depth=4, threads=256, workgroups=128)
     assert (k.slices, k.piece_bytes, k.passes, k.fifo_depth, k.threads, k.workgroups, k.max_hosted) == (16, 65536, 8, 4, 256, 128, 4)
