@@ -25,10 +25,10 @@ for p in (ROOT, os.path.join(ROOT, "msccl-tools_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/exec_kernel_c2_allgather_pmc.txt), scaled by what the same counters read for a plain
-# copy of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = {"c2": None}
+# HBM-side bytes per launch of the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/exec_kernel_c2_ring_allgather_pmc.txt), each scaled by what the same counter reads for a
+# plain device copy of 1 GiB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Not measured for the others.
+MEASURED_TRAFFIC_BYTES = {"c2": 3766862474}
 
 
 def ensure_built():
@@ -166,6 +166,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run five plain device copies of 1 GiB (known traffic: 1 GiB read + 1 GiB written each), "
+                         "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: every rank of the algorithm is a virtual rank on ONE GPU; run with --gpus 1 "
@@ -177,6 +180,15 @@ def main():
         print("bench.py: no GPU visible; the executor has no CPU path", file=sys.stderr)
         sys.exit(3)
 
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "5 device copies of 1073741824 bytes"}))
+        return
     head = run_workload(args.config, args.steps, args.warmup)
     traffic = MEASURED_TRAFFIC_BYTES.get(args.config)
     line = {

@@ -170,7 +170,7 @@ def test_watchdog_reports_instead_of_hanging():
     xml = ir_samples.slow_producer_xml(24)
     nbytes = 64 << 20
     ex = Executor(xml)
-    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, piece_bytes=65536)
+    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1)  # one pass: the receive waits for all 24 copies
     x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
     ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
     ex.bind(ins, outs)
