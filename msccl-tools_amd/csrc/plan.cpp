@@ -385,8 +385,8 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;
     slices = std::max<int64_t>(1, std::max(by_piece, to_fill));
     slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
-    // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~16
-    const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 16) / ntbs);
+    // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~32
+    const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 32) / ntbs);
     slices = std::min(slices, comfortable);
   }
   slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
