@@ -1,0 +1,92 @@
+"""Registered plans.  `ndv4`: the MSCCLang plans of msccl-tools' msccl/autosynth/ndv4_plans.py:12-48
+(same programs, replication, protocols and size windows).  `mi355x`: plans for algorithms whose ranks
+are all virtual ranks of one MI355X (machines = groups of 8 virtual ranks)."""
+from msccl.autosynth.registry import register_msccl_program
+from msccl.language.ir import ThreadblockPolicy
+from msccl.programs.allgather_ring import allgather_ring
+from msccl.programs.allreduce_a100_ring import allreduce_ring
+from msccl.programs.allreduce_allpairs import allreduce_allpairs
+from msccl.programs.alltoall_a100_8kp1 import alltoall_three_step
+from msccl.programs.alltoall_a100_yifan import alltoall_hierarchical
+from msccl.programs.hierarchical_allreduce import hierarchical_allreduce
+from msccl.topologies import fully_connected
+
+
+def register_ndv4_plans():
+    one = lambda x: x == 1
+    manual = ThreadblockPolicy.manual
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'ndv4', chunk_factor=64, inplace=True, instances=2, protocol='LL',
+                            sizes=('512B', '82944B'), threadblock_policy=manual, interleaved_replication=False,
+                            dependence_nop=True, machines=one)
+    def ndv4_allpairs_allreduce_config1(prog, nodes):
+        allreduce_allpairs(8)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'ndv4', chunk_factor=64, inplace=True, instances=4, protocol='LL',
+                            sizes=('82944B', '458752B'), threadblock_policy=manual, interleaved_replication=False,
+                            dependence_nop=True, machines=one)
+    def ndv4_allpairs_allreduce_config2(prog, nodes):
+        allreduce_allpairs(8)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'ndv4', chunk_factor=8, inplace=True, instances=8, protocol='LL',
+                            sizes=('458752B', '2129920B'), threadblock_policy=manual, machines=one)
+    def ndv4_ring_allreduce_config1(prog, nodes):
+        allreduce_ring(size=8, channels=4)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'ndv4', chunk_factor=8, inplace=True, instances=8, protocol='LL128',
+                            sizes=('2129920B', '22806528B'), threadblock_policy=manual, machines=one)
+    def ndv4_ring_allreduce_config2(prog, nodes):
+        allreduce_ring(size=8, channels=4)
+
+    @register_msccl_program(fully_connected(8), 'alltoall', 'ndv4', protocol='LL128', sizes=('1MB', '32MB'),
+                            machines=lambda x: x in (8, 16, 32, 64))
+    def ndv4_alltoall_hierarchical_config1(prog, nodes):
+        alltoall_hierarchical(num_nodes=nodes, gpus_per_node=8)
+
+    @register_msccl_program(fully_connected(8), 'alltoall', 'ndv4', protocol='Simple', sizes=('32MB', None),
+                            machines=lambda x: x in (8, 16, 32))
+    def ndv4_alltoall_hierarchical_config2(prog, nodes):
+        alltoall_hierarchical(num_nodes=nodes, gpus_per_node=8)
+
+    @register_msccl_program(fully_connected(8), 'alltoall', 'ndv4', protocol='Simple', sizes=('32MB', None), machines=lambda x: x == 64)
+    def ndv4_alltoall_three_step(prog, nodes):
+        alltoall_three_step(num_nodes=nodes, gpus_per_node=8)
+
+    @register_msccl_program(fully_connected(8), 'alltoall', 'ndv4', protocol='Simple', sizes=('1KB', None), machines=lambda x: x in (2, 4))
+    def ndv4_alltoall_hierarchical_config2(prog, nodes):  # noqa: F811 -- same name, other machine counts, as upstream
+        alltoall_hierarchical(num_nodes=nodes, gpus_per_node=8)
+
+
+def register_mi355x_plans():
+    """Virtual-rank plans: `machines` counts groups of 8 virtual ranks held in one GPU's HBM."""
+    one = lambda x: x == 1
+    manual = ThreadblockPolicy.manual
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=8, inplace=True, instances=1,
+                            sizes=(0, '8MB'), threadblock_policy=manual, machines=one)
+    def mi355x_ring_allreduce_small(prog, nodes):
+        allreduce_ring(size=8, channels=1)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=8, inplace=True, instances=4,
+                            sizes=('8MB', None), threadblock_policy=manual, machines=one)
+    def mi355x_ring_allreduce_large(prog, nodes):
+        allreduce_ring(size=8, channels=1)
+
+    @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=4,
+                            threadblock_policy=manual, machines=one)
+    def mi355x_ring_allgather(prog, nodes):
+        allgather_ring(size=8, channels=1)
+
+    @register_msccl_program(fully_connected(8), 'alltoall', 'mi355x', machines=lambda x: 2 <= x <= 8)
+    def mi355x_alltoall_hierarchical(prog, nodes):
+        alltoall_hierarchical(num_nodes=nodes, gpus_per_node=8)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=16, inplace=True, instances=2,
+                            interleaved_replication=False, machines=lambda x: x == 2)
+    def mi355x_two_level_allreduce_2x8(prog, nodes):
+        hierarchical_allreduce(8, 2, "auto")
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=32, inplace=True, instances=2,
+                            interleaved_replication=False, machines=lambda x: x == 4)
+    def mi355x_two_level_allreduce_4x8(prog, nodes):
+        hierarchical_allreduce(8, 4, "auto")

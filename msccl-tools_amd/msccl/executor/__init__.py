@@ -1,5 +1,6 @@
 """MI355X executor for MSCCL-IR: XML -> flat tables -> libmscclx.so (HIP) through ctypes."""
 from .ir_tables import AlgoTables, IRError, load_algo, parse_algo_xml, OP_CODES, BUF_CODES, ALGO_FACTOR
+from .config import LoadedAlgo, load_config, select
 from .binding import (ExecutorUnavailable, MscclxError, Plan, load_library, DTYPE_CODES, DTYPE_SIZES, REDOP_CODES,
                       EXPORTED_SYMBOLS, LIB_PATH)
 

@@ -1,0 +1,123 @@
+"""`msccl.init` and the plan registry: the observable behaviour msccl-tools' own tests assert
+(tests/test_autosynth.py:10-45, tests/test_programs.py:61-86 there), plus the MI355X side reading
+the index back."""
+import math
+import os
+
+import pytest
+
+import msccl
+from msccl.autosynth import _select_plans
+from msccl.autosynth.registry import register_ef_file, register_synthesis_plan, synthesis_plans
+from msccl.autosynth.sizes import format_size, parse_size
+from msccl.executor import load_config, select
+
+
+@pytest.fixture(autouse=True)
+def clean_env(monkeypatch):
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO", "NCCL_IB_AR_THRESHOLD", "NCCL_IB_PCI_RELAXED_ORDERING", "NCCL_TOPO_FILE", "CUDA_VISIBLE_DEVICES"):
+        monkeypatch.delenv(k, raising=False)
+
+
+def test_sizes():
+    assert parse_size("512B") == 512 and parse_size("1KB") == 1000 and parse_size("1MB") == 10 ** 6
+    assert parse_size("1GiB") == 2 ** 30 and parse_size("82944B") == 82944 and parse_size(7) == 7
+    assert format_size(512) == "512 bytes" and format_size(82944) == "82.94 KB" and format_size(math.inf) == "infinity"
+    with pytest.raises(ValueError):
+        parse_size("12 parsecs")
+
+
+def test_msccl_init(capsys):
+    msccl.init('not_a_machine_type', 4, ('alltoall', 0))
+    out, _ = capsys.readouterr()
+    assert 'No plan found' in out
+    assert 'MSCCL_CONFIG' not in os.environ
+    assert 'NCCL_ALGO' not in os.environ
+
+    msccl.init('mi355x', 2, ('alltoall', '1MB'))
+    out, _ = capsys.readouterr()
+    assert 'mi355x_alltoall_hierarchical' in out
+    assert 'MSCCL_CONFIG' in os.environ
+    assert 'NCCL_IB_AR_THRESHOLD' not in os.environ
+    assert os.environ['NCCL_ALGO'] == 'MSCCL,RING,TREE'
+
+    os.environ['NCCL_ALGO'] = 'RING,FAKE_MSCCL'
+    msccl.init('ndv4', 8, (msccl.Collective.alltoall, '2MB'))
+    out, _ = capsys.readouterr()
+    assert 'ndv4_alltoall' in out
+    assert 'NCCL_IB_AR_THRESHOLD' in os.environ
+    assert os.environ['NCCL_ALGO'] == 'MSCCL,RING,FAKE_MSCCL'
+
+    os.environ['NCCL_ALGO'] = 'HELLO,MSCCL,WORLD'
+    msccl.init('ndv4', 16, (msccl.Collective.alltoall, '35MB'))
+    out, _ = capsys.readouterr()
+    assert 'ndv4_alltoall' in out
+    assert os.environ['NCCL_ALGO'] == 'HELLO,MSCCL,WORLD'
+
+
+def test_register_plan():
+    @register_synthesis_plan('allgather', 'fancy_machine', sizes=(0, '4MB'))
+    def dummy_plan(m):
+        return "<algo/>"
+
+    @register_synthesis_plan('allgather', ['m1', 'm2'], sizes=('1GiB', None))
+    def dummy_plan2(m):
+        return "<algo/>"
+    assert synthesis_plans[('allgather', 'fancy_machine')][-1][3] == (0, 4 * 10 ** 6)
+    assert synthesis_plans[('allgather', 'm1')][-1][3] == (2 ** 30, math.inf)
+    assert synthesis_plans[('allgather', 'm2')][-1][0] == 'call dummy_plan2'
+
+
+def test_registered_ndv4_allreduce(capsys):
+    msccl.init('ndv4', 1, (msccl.Collective.allreduce, (512, 1024)))
+    assert 'ndv4_allpairs_allreduce_config1 with LL protocol' in capsys.readouterr().out
+    msccl.init('ndv4', 1, (msccl.Collective.allreduce, (82944, 458752)))
+    assert 'ndv4_allpairs_allreduce_config2 with LL protocol' in capsys.readouterr().out
+    msccl.init('ndv4', 1, (msccl.Collective.allreduce, (458752, 2129920)))
+    assert 'ndv4_ring_allreduce_config1 with LL protocol' in capsys.readouterr().out
+    msccl.init('ndv4', 1, (msccl.Collective.allreduce, (2129920, 22806528)))
+    assert 'ndv4_ring_allreduce_config2 with LL128 protocol' in capsys.readouterr().out
+
+
+def test_registered_ndv4_alltoall(capsys):
+    msccl.init('ndv4', 8, (msccl.Collective.alltoall, ('1MB', '32MB')))
+    assert 'ndv4_alltoall_hierarchical_config1 with LL128 protocol' in capsys.readouterr().out
+    msccl.init('ndv4', 8, (msccl.Collective.alltoall, ('32MB', '64MB')))
+    assert 'ndv4_alltoall_hierarchical_config2 with Simple protocol' in capsys.readouterr().out
+
+
+def test_interval_selection_by_priority(capsys):
+    plan_a, plan_b = (lambda m: "a"), (lambda m: "b")
+    cands = [("A", plan_a, lambda m: True, (0, 1000), "Simple", 0),
+             ("B", plan_b, lambda m: True, (500, 2000), "LL", 1),
+             ("C", plan_a, lambda m: m == 99, (0, math.inf), "Simple", 5)]
+    res = _select_plans("allreduce", cands, 1, (0, 3000))
+    assert [(p, v) for p, v in res] == [(plan_a, [0, 500, "Simple"]), (plan_b, [500, 1000, "LL"]), (plan_b, [1000, 2000, "LL"])]
+    out = capsys.readouterr().out
+    assert "No plan found for allreduce with sizes from 2 KB to infinity" in out
+
+
+def test_index_roundtrip_and_selection(capsys):
+    msccl.init('ndv4', 1, (msccl.Collective.allreduce, (512, 3000000)))
+    capsys.readouterr()
+    algos = load_config()
+    assert [(a.min_bytes, a.max_bytes, a.proto) for a in algos] == [(512, 82944, 'LL'), (82944, 458752, 'LL'), (458752, 2129920, 'LL'),
+                                                                   (2129920, 22806528, 'LL128')]
+    assert all(a.tables.coll == "allreduce" and a.tables.ngpus == 8 for a in algos)
+    assert select(algos, "allreduce", 1024) is algos[0]
+    assert select(algos, "allreduce", 1 << 20) is algos[2]
+    assert select(algos, "allreduce", 100) is None
+    assert select(algos, "alltoall", 1024) is None
+    # ring all-reduce, 8 chunks x 8 instances
+    assert algos[2].tables.nchunksperloop == 64 and algos[2].bytes_per_rank_to_chunk_bytes(1 << 20) == (1 << 20) // 64
+
+
+def test_ef_file_plan(tmp_path, capsys):
+    import ir_samples
+    f = tmp_path / "ring.xml"
+    f.write_text(ir_samples.ring_allgather_xml(4))
+    register_ef_file(str(f), 'allgather', 'testbox', 1, sizes=('1KB', '1MB'))
+    msccl.init('testbox', 1, ('allgather', '64KB'))
+    assert f'load {f}' in capsys.readouterr().out
+    a = select(load_config(), "allgather", 65536)
+    assert a.path == str(f) and a.tables.ngpus == 4 and (a.min_bytes, a.max_bytes) == (1000, 10 ** 6)

@@ -143,3 +143,37 @@ def test_aliased_buffers_fall_back_to_staging():
     ex2.setup(E * 4, "int32")
     ex2.bind(bufs, [b[: n * E] for b in bufs])  # same memory for 'i' and 'o'
     assert ex2.info.zero_copy_messages == 0 and ex2.info.staged_messages > 0
+
+
+def test_init_to_run_flow(capsys):
+    """msccl.init -> MSCCL_CONFIG index -> select by size -> run: the drop-in path end to end."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    nbytes = 8 * 4 * 4 * 2500                                # bytes per rank
+    msccl.init('mi355x', 1, ('allgather', nbytes), ('allreduce', nbytes))
+    algos = load_config()
+    ag = select(algos, "allgather", nbytes)
+    ar = select(algos, "allreduce", nbytes)
+    assert ag is not None and ar is not None and ar.tables.nchunksperloop == 8
+    rng = np.random.default_rng(3)
+    # all-gather
+    x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64).astype(np.int32) for _ in range(8)]
+    cb = ag.bytes_per_rank_to_chunk_bytes(nbytes)
+    ex = Executor(ag.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v) for v in x])
+    ex.run(ins, outs)
+    want = np.concatenate(x)
+    assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(8))
+    # all-reduce (ring order)
+    y = [(rng.random(nbytes // 4, dtype=np.float32) * 2 - 1) for _ in range(8)]
+    cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
+    ex = Executor(ar.tables)
+    ex.setup(cb, "float32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "float32", inputs=[torch.from_numpy(v) for v in y])
+    ex.run(ins, outs)
+    want = oc.expected_allreduce(y, 8, oc.ring_allreduce_orders(8), "float32")
+    assert all(np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)) for r in range(8))
