@@ -118,6 +118,14 @@ def main():
         "allgather_allpairs_8r": lambda: from_example("allgather_allpairs.py", [8, 1]),
         "allreduce_a100_allpairs_8r": lambda: from_example("allreduce_a100_allpairs.py", [8, 1]),
         "alltoall_allpairs_4r": lambda: from_example("alltoall_allpairs.py", [4, 1]),
+        "allreduce_1step_4r": lambda: from_example("allreduce_1step.py", [4, 1]),
+        "allreduce_a100_multinode_allpairs_16r": lambda: from_example("allreduce_a100_multinode_allpairs.py", [16, 1]),
+        "allreduce_a100_ncv4_8r": lambda: from_example("allreduce_a100_ncv4.py", [8, 1]),
+        "allreduce_a100_pcie_hierarchical_8r": lambda: from_example("allreduce_a100_pcie_hierarchical.py", [8, 1]),
+        "alltonext_forward_2x8": lambda: from_example("alltonext_forward.py", [2, 1]),
+        "alltonext_backward_2x8": lambda: from_example("alltonext_backward.py", [2, 1]),
+        "pipeline_a100_allpairs_8r": lambda: from_example("pipeline_a100_allpairs.py", [8, 1]),
+        "pipeline_a100_ring_8r_2ch": lambda: from_example("pipeline_a100_ring.py", [8, 2, 1]),
     }
     os.makedirs(OUT, exist_ok=True)
     for name, job in jobs.items():

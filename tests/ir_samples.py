@@ -135,3 +135,47 @@ def slow_producer_xml(ncopies):
         _gpu(0, 1, 1, 0, [_tb(0, 1, -1, 0, steps)]),
         _gpu(1, 1, 1, 0, [_tb(0, -1, 0, 0, [_step(0, "r", "i", 0, "o", 0, 1)])]),
     ])
+
+
+# ---- documents in the style of msccl-tools' second emitter (msccl/ncclize.py:658-718) ----------
+# inplace="0", only s / r / rrc / cpy / nop, sending and receiving threadblocks separate, one extra
+# threadblock per rank (send=recv=-1, chan 0) holding the pre/post copies, and on r / rrc steps
+# srcbuf/srcoff naming the SENDER's location (ncclize.py:534-535).
+def ncclize_style_allgather_xml(n=3):
+    """Ring all-gather out of place: the copy threadblock puts i[0] into o[r]; chunk k travels
+    k -> k+1 -> ...; forwarding sends wait for the receive that delivered the chunk."""
+    gpus = []
+    for r in range(n):
+        nxt, prv = (r + 1) % n, (r - 1) % n
+        send_steps, recv_steps = [], []
+        for h in range(n - 1):
+            c_out, c_in = (r - h) % n, (r - 1 - h) % n
+            if h == 0:
+                send_steps.append(_step(h, "s", "i", 0, "o", c_out, 1))
+                recv_steps.append(_step(h, "r", "i", 0, "o", c_in, 1, hasdep=1 if n > 2 else 0))
+            else:
+                send_steps.append(_step(h, "s", "o", c_out, "o", c_out, 1, depid=1, deps=h - 1))
+                recv_steps.append(_step(h, "r", "o", c_in, "o", c_in, 1, hasdep=1 if h < n - 2 else 0))
+        gpus.append(_gpu(r, 1, n, 0, [_tb(0, nxt, -1, 0, send_steps), _tb(1, -1, prv, 0, recv_steps),
+                                     _tb(2, -1, -1, 0, [_step(0, "cpy", "i", 0, "o", r, 1)])]))
+    return _algo("ncclize_allgather", "allgather", 0, n, 1, n, gpus)
+
+
+def ncclize_style_allreduce_xml():
+    """3 ranks, 1 chunk, out of place: every rank copies i[0] to o[0]; ranks 1 and 2 send i[0] to rank
+    0, which reduces them into o[0] in that order (rrc, the second waiting for the first); rank 0 then
+    sends o[0] to both, whose receives wait for their own copy.  Result everywhere: (x0 + x1) + x2."""
+    g0 = _gpu(0, 1, 1, 0, [
+        _tb(0, 1, -1, 0, [_step(0, "s", "o", 0, "o", 0, 1, depid=3, deps=0)]),
+        _tb(1, 2, -1, 0, [_step(0, "s", "o", 0, "o", 0, 1, depid=3, deps=0)]),
+        _tb(2, -1, 1, 0, [_step(0, "rrc", "i", 0, "o", 0, 1, depid=4, deps=0, hasdep=1)]),
+        _tb(3, -1, 2, 0, [_step(0, "rrc", "i", 0, "o", 0, 1, depid=2, deps=0, hasdep=1)]),
+        _tb(4, -1, -1, 0, [_step(0, "cpy", "i", 0, "o", 0, 1, hasdep=1)]),
+    ])
+    def leaf(rank):
+        return _gpu(rank, 1, 1, 0, [
+            _tb(0, 0, -1, 0, [_step(0, "s", "i", 0, "o", 0, 1)]),
+            _tb(1, -1, 0, 0, [_step(0, "r", "o", 0, "o", 0, 1, depid=2, deps=0)]),
+            _tb(2, -1, -1, 0, [_step(0, "cpy", "i", 0, "o", 0, 1, hasdep=1)]),
+        ])
+    return _algo("ncclize_allreduce", "allreduce", 0, 3, 1, 1, [g0, leaf(1), leaf(2)])

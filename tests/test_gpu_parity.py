@@ -109,6 +109,17 @@ def test_allpairs_scratch_and_deps(n):
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("staging", [0, 1])
+def test_ncclize_schema(staging):
+    """Documents shaped like msccl-tools' ncclize output: copy threadblocks, inplace=0, sender-side
+    src on receives, rrc chains."""
+    for n in (2, 3, 5):
+        got, want, _, _ = run_both(ir_samples.ncclize_style_allgather_xml(n), 5000, "int32", in_elems=5000, staging=staging)
+        assert_same(got, want)
+    got, want, _, _ = run_both(ir_samples.ncclize_style_allreduce_xml(), 7000, "float32", staging=staging)
+    assert_same(got, want)
+
+
 def test_rrc_cpy_nop():
     got, want, _, _ = run_both(ir_samples.RRC_CPY_NOP_XML, 1000 * 4, "int32")
     assert_same(got, want)

@@ -172,3 +172,21 @@ def test_algorithmic_bytes_closed_forms():
         assert oi.algorithmic_bytes(ar, S // n) * n == 5 * (n - 1) * S * n  # 5(n-1)S over all... per rank S
         ag = oi.parse_xml(ir_samples.ring_allgather_xml(n))
         assert oi.algorithmic_bytes(ag, S) == 2 * (n - 1) * n * S
+
+
+# ---- the second emitter's schema (ncclize) ------------------------------------------------------
+@pytest.mark.parametrize("n", [2, 3, 5])
+def test_ncclize_style_allgather(n):
+    x = _inputs(n, 6, "int32", seed=30)
+    algo, outs = _run(ir_samples.ncclize_style_allgather_xml(n), x, 6, "int32")
+    assert algo.inplace == 0
+    for r in range(n):
+        assert np.array_equal(outs[r], np.concatenate(x))
+
+
+def test_ncclize_style_allreduce():
+    x = _inputs(3, 64, "float32", seed=31)
+    _, outs = _run(ir_samples.ncclize_style_allreduce_xml(), x, 64, "float32")
+    want = (x[0] + x[1]) + x[2]
+    for r in range(3):
+        assert np.array_equal(outs[r].view(np.uint32), want.view(np.uint32))
