@@ -149,6 +149,18 @@ template <int DT, int OP> struct Reducer {
 #ifndef MSCCLX_AUX
 #define MSCCLX_AUX 16 /* sc1 = device scope */
 #endif
+// Loads are marked non-temporal: every payload byte is read exactly once by the step that loads it.
+// Stores stay cacheable (a peer or a later step reads most of them soon, and the memory-side cache
+// then serves that read) except the ones the plan proved are never read again.
+#ifndef MSCCLX_AUX_LD
+#define MSCCLX_AUX_LD (MSCCLX_AUX | 2)
+#endif
+#ifndef MSCCLX_AUX_ST
+#define MSCCLX_AUX_ST MSCCLX_AUX
+#endif
+#ifndef MSCCLX_AUX_ST_FINAL
+#define MSCCLX_AUX_ST_FINAL (MSCCLX_AUX | 2)
+#endif
 constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family dword 3)
 
 template <int W> struct Access;
@@ -188,11 +200,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 constexpr int kUnroll = MSCCLX_UNROLL;
 
 // out1[, out2] = a [(+) b] over n units of W bytes.
-template <class R, int W, bool HAS_B, bool HAS_O2>
+template <class R, int W, bool HAS_B, bool HAS_O2, bool NT1>
 __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n) {
   typedef Access<W> A;
   typedef typename A::word word;
-  constexpr int X = MSCCLX_AUX;
+  constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
   const uint32_t bytes = n * W;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
@@ -202,18 +214,18 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
     word x[UA], y[UA];
 #pragma unroll
-    for (int u = 0; u < UA; ++u) x[u] = A::template ld<X>(ra, (int)((i + u * T) * W));
+    for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * W));
     if (HAS_B) {
 #pragma unroll
-      for (int u = 0; u < UA; ++u) y[u] = A::template ld<X>(rb, (int)((i + u * T) * W));
+      for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * W));
 #pragma unroll
       for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
     }
 #pragma unroll
-    for (int u = 0; u < UA; ++u) A::template st<X>(r1, (int)((i + u * T) * W), x[u]);
+    for (int u = 0; u < UA; ++u) A::template st<X1>(r1, (int)((i + u * T) * W), x[u]);
     if (HAS_O2) {
 #pragma unroll
-      for (int u = 0; u < UA; ++u) A::template st<X>(r2, (int)((i + u * T) * W), x[u]);
+      for (int u = 0; u < UA; ++u) A::template st<XS>(r2, (int)((i + u * T) * W), x[u]);
     }
   }
 }
@@ -221,12 +233,12 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
 // rows x n units.  Consecutive rows of an operand are `stride_*` units apart: a chunk for rank
 // buffers, n for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
 // buffer, o2 (the forwarded copy) always a FIFO slot.
-template <class R, bool VEC, bool HAS_B, bool HAS_O2>
+template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool NT1 = false>
 __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
                                           const unsigned char* b, uint64_t stride_b, int rows, uint32_t n) {
   constexpr int W = VEC ? 16 : R::kElemBytes;
   for (int r = 0; r < rows; ++r)
-    move_units<R, W, HAS_B, HAS_O2>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
+    move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
                                     a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
 }
 
@@ -438,7 +450,10 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
       }
       switch (t) {
         case MSCCLX_OP_SEND: move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
-        case MSCCLX_OP_RECV: move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n); break;
+        case MSCCLX_OP_RECV:
+          if (op.nt_store) move_rows<R, VEC, false, false, true>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
+          else             move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
+          break;
         case MSCCLX_OP_RCS:
           if (out) move_rows<R, VEC, false, true>(ldst, cs, out, in, in_stride, nullptr, 0, op.cnt, n);
           else     move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
@@ -449,7 +464,10 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
           if (out) move_rows<R, VEC, true, true>(ldst, cs, out, in, in_stride, ldst, cs, op.cnt, n);
           else     move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n);
           break;
-        case MSCCLX_OP_COPY:   move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
+        case MSCCLX_OP_COPY:
+          if (op.nt_store) move_rows<R, VEC, false, false, true>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
+          else             move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
+          break;
         case MSCCLX_OP_REDUCE: move_rows<R, VEC, true, false>(ldst, cs, nullptr, lsrc, cs, ldst, cs, op.cnt, n); break;
         default: break;
       }
@@ -682,7 +700,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
         dv.dep_nops = plan->tbs[dv.dep_tb].op_end - plan->tbs[dv.dep_tb].op_begin;
       }
       dv.hasdep = op.hasdep; dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
-      dv.in_slot = -1; dv.in_off = -1; dv.pad = 0;
+      dv.in_slot = -1; dv.in_off = -1; dv.nt_store = op.final_write;
       dv.out_staged = is_send_type(op.type) && (g.staging || !op.zero_copy) ? 1 : 0;
       if (is_recv_type(op.type) && !g.staging) {
         const Op& sender = plan->ops[op.match_send];

@@ -171,6 +171,41 @@ static void find_zero_copy_messages(mscclx_plan* p) {
   }
 }
 
+// Local destinations nobody reads: not as a local source ('s', 'cpy', 're'), not as the accumulator
+// of a reduction, not by a peer reading a forwarded payload in place.  Conservative: a read anywhere
+// in the program, before or after the write, keeps the write cacheable.
+static void find_final_writes(mscclx_plan* p) {
+  typedef std::pair<int, int> Span;  // [lo, hi) in chunks
+  std::vector<std::vector<Span>> reads((size_t)p->nranks * 3);
+  for (const Tb& tb : p->tbs)
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      const Op& op = p->ops[o];
+      if (reads_local_src(op.type)) reads[(size_t)tb.rank * 3 + op.srcbuf].push_back({op.srcoff, op.srcoff + op.cnt});
+      if (is_reduce_type(op.type) || op.type == MSCCLX_OP_RCS) reads[(size_t)tb.rank * 3 + op.dstbuf].push_back({op.dstoff, op.dstoff + op.cnt});
+    }
+  // merge into disjoint sorted spans
+  for (auto& v : reads) {
+    std::sort(v.begin(), v.end());
+    size_t k = 0;
+    for (const Span& s : v) {
+      if (k && s.first <= v[k - 1].second) v[k - 1].second = std::max(v[k - 1].second, s.second);
+      else v[k++] = s;
+    }
+    v.resize(k);
+  }
+  for (const Tb& tb : p->tbs)
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      Op& op = p->ops[o];
+      if (!touches_local_dst(op.type) || op.type == MSCCLX_OP_RRS) continue;
+      const std::vector<Span>& v = reads[(size_t)tb.rank * 3 + op.dstbuf];
+      const int lo = op.dstoff, hi = op.dstoff + op.cnt;
+      auto it = std::upper_bound(v.begin(), v.end(), Span{lo, 0x7fffffff});  // first span starting after lo
+      bool any = it != v.end() && it->first < hi;
+      if (it != v.begin() && std::prev(it)->second > lo) any = true;
+      op.final_write = any ? 0 : 1;
+    }
+}
+
 static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
   if (d->nranks <= 0 || d->ntbs < 0 || d->nops < 0) return fail(MSCCLX_ERR_INVALID_ARG, "negative table size");
   if (!d->rank_chunks || (d->ntbs && !d->tbs) || (d->nops && !d->ops)) return fail(MSCCLX_ERR_INVALID_ARG, "null table pointer");
@@ -310,6 +345,7 @@ static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
     }
   }
   find_zero_copy_messages(p);
+  find_final_writes(p);
   for (Conn& cn : p->conns) {
     const Tb& s = p->tbs[cn.send_tb];
     for (int so = s.op_begin; so < s.op_end; ++so)

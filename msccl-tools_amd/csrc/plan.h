@@ -19,6 +19,9 @@ struct Op {
   // local destination an 'rcs'/'rrcs' has just written) until the matching receive has consumed it:
   // the receiver reads it from there and no FIFO slot is filled.
   int32_t zero_copy = 0;
+  // Steps whose local destination chunks no step of the program ever reads (neither this rank nor,
+  // in place, a peer): their stores are marked non-temporal so they do not displace reusable lines.
+  int32_t final_write = 0;
 };
 
 struct Tb {
@@ -55,7 +58,7 @@ struct DevOp {
   int32_t send_seq, recv_seq;
   int32_t in_slot, in_off;   // recv-type: buffer-table index / chunk offset of the sender's payload, or -1: FIFO slot
   int32_t out_staged;        // send-type: 1 = copy the payload into a FIFO slot, 0 = the receiver reads it in place
-  int32_t pad;
+  int32_t nt_store;          // 1 = the local destination is never read again: store it non-temporally
 };
 
 struct DevTb {
