@@ -307,8 +307,17 @@ __device__ __forceinline__ void finish_step(Context& c, const KernelParams& p) {
 // reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
 // share the resident workgroups without deadlock.
 template <class R, bool VEC>
-__global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
+__global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_params) {
   constexpr uint64_t UB = VEC ? 16 : R::kElemBytes;
+  // Which of the two counter areas this launch uses is kept on the device (control word 0) and is
+  // flipped by the last workgroup to finish, so a launch carries no host-side state and the same
+  // launch can be replayed (stream order guarantees the flip is seen by the next launch).
+  KernelParams p = launch_params;
+  {
+    const u64 parity = load_counter(p.sync_base) & 1ull;
+    p.sync_cur = p.sync_base + kSyncHeaderWords + parity * p.sync_words;
+    p.sync_nxt = p.sync_base + kSyncHeaderWords + (parity ^ 1ull) * p.sync_words;
+  }
   __shared__ int sh_choice, sh_tb, sh_slice, sh_step;
   __shared__ unsigned sh_pass;
   const u64* const abort_word = p.sync_cur;
@@ -488,6 +497,14 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams p) {
     }
 #endif
   }
+  if (threadIdx.x == 0) {
+    // the last workgroup out re-arms the control block: next launch uses the other counter area
+    const u64 finished = __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (finished == (u64)gridDim.x - 1) {
+      publish(p.sync_base + 1, 0);
+      publish(p.sync_base, (load_counter(p.sync_base) & 1ull) ^ 1ull);
+    }
+  }
 #ifdef MSCCLX_PROFILE
   if (threadIdx.x == 0 && p.prof) {
     p.prof[(size_t)blockIdx.x * 4 + 0] = prof_wait;
@@ -541,7 +558,6 @@ struct DeviceState {
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
   kernel_fn kernel = nullptr;
-  unsigned launches = 0;
   bool dirty = false;  // counters must be cleared before the next launch (after a failed launch)
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: 4 words per workgroup
@@ -751,14 +767,13 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
     HIP_TRY(hipMemset(d->workspace, 0, g.fifo_byte_off));
     HIP_TRY(hipDeviceSynchronize());
     d->dirty = false;
-    d->launches = 0;
   }
   KernelParams kp;
   kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns; kp.bufs = d->bufs;
   unsigned long long* sync = (unsigned long long*)d->workspace;
-  const unsigned parity = d->launches & 1u;
-  kp.sync_cur = sync + (uint64_t)parity * g.sync_words;
-  kp.sync_nxt = sync + (uint64_t)(parity ^ 1u) * g.sync_words;
+  kp.sync_base = sync;
+  kp.sync_cur = kp.sync_nxt = nullptr;
+  kp.sync_words = g.sync_words;
   kp.fifo = d->workspace + g.fifo_byte_off;
   kp.host_status = d->host_status;
   kp.prof = d->prof;
@@ -774,7 +789,6 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
   const unsigned grid = (unsigned)g.workgroups;
   hipLaunchKernelGGL(d->kernel, dim3(grid), dim3(g.threads), 0, s, kp);
   HIP_TRY(hipGetLastError());
-  d->launches++;
   return MSCCLX_OK;
 }
 

@@ -515,7 +515,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.slice_fifo_units = slot_chunks * g.piece_units;
   g.sync_slice_words = (uint64_t)(plan.tbs.size() + 2 * plan.conns.size()) * kSyncStrideWords;
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
-  const uint64_t sync_bytes = (2 * g.sync_words * 8 + 255) / 256 * 256;
+  const uint64_t sync_bytes = ((kSyncHeaderWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
   g.fifo_byte_off = sync_bytes;
   g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * g.unit_bytes + 256;
   *out = std::move(g);

@@ -96,14 +96,16 @@ struct KernelParams {
   const DevOp* ops;
   const DevConn* conns;
   void* const* bufs;            // [nranks*3]
-  unsigned long long* sync_cur; // this launch's counters
-  unsigned long long* sync_nxt; // next launch's counters (cleared by this launch)
+  unsigned long long* sync_base; // control block: word 0 = which counter area this launch uses, word 1 = workgroups finished
+  unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
+  unsigned long long* sync_nxt;  // next launch's counters   } from the control block
   unsigned char* fifo;
   mscclx_status* host_status;   // pinned host memory
   unsigned long long* prof;     // per-workgroup tick counters of MSCCLX_PROFILE builds, else null
   uint64_t chunk_units;
   uint64_t slice_fifo_units;
   uint64_t sync_slice_words;
+  uint64_t sync_words;
   uint64_t timeout_ticks;
   uint32_t piece_units;
   int32_t slices, depth, ntbs, nconns;

@@ -173,6 +173,39 @@ def test_relaunch_reuses_counters():
             assert np.array_equal(keep[2][r].cpu().numpy(), want), (it, r)
 
 
+def test_hip_graph_replay():
+    """A launch keeps no host-side state (the counter-area parity lives on the device), so it can be
+    captured once and replayed; every replay, interleaved with eager work, must be right."""
+    from msccl.executor import Executor, collective_buffers
+    xml = ir_samples.ring_allreduce_xml(8, 2)
+    E = 6000
+    ex = Executor(xml)
+    ex.setup(E * 4, "float32")
+    base = make_inputs(8, 16 * E, "float32", seed=70)
+    ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in base])
+    ex.run(ins, outs)                                   # eager launch first (odd number of launches so far)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            ex.launch()
+    algo = oi.parse_xml(xml)
+    for it in range(4):
+        x = make_inputs(8, 16 * E, "float32", seed=80 + it)
+        for r in range(8):
+            ins[r].copy_(torch.from_numpy(x[r]))        # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oc.place_inputs(algo, x, E, "float32")
+        oi.Interpreter(algo).run(want, E, "float32")
+        for r in range(8):
+            assert np.array_equal(ins[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (it, r)
+        if it == 1:                                     # an eager launch in between flips the parity once more
+            ex.run(ins, outs)
+
+
 def test_watchdog_reports_instead_of_hanging():
     """A 1 ms watchdog while a receive legitimately waits for tens of milliseconds: the waiting
     workgroup must give up cleanly (every wave exits, the producer still finishes), the error names
