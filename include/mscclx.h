@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MSCCLX_VERSION 1
+#define MSCCLX_VERSION 2
 
 typedef enum {
   MSCCLX_OK = 0,
@@ -61,6 +61,13 @@ typedef enum {
   MSCCLX_F16 = 6, MSCCLX_BF16 = 7, MSCCLX_F32 = 8, MSCCLX_F64 = 9, MSCCLX_NUM_DTYPES = 10
 } mscclx_dtype;
 
+/* How a message crosses a connection.  SIMPLE: payload, then (after the stores are acknowledged) a
+ * counter; payloads that may be read in place are not copied at all.  LL: every message is written
+ * into its FIFO slot as 16-byte lines of two (data, flag) pairs and the receiver polls the flags in
+ * the data itself -- twice the slot traffic, about half the latency per hop; meant for small pieces
+ * (the trade msccl-tools names with proto="LL", msccl/language/__init__.py:38-39). */
+typedef enum { MSCCLX_PROTO_AUTO = 0, MSCCLX_PROTO_SIMPLE = 1, MSCCLX_PROTO_LL = 2 } mscclx_protocol;
+
 typedef enum { MSCCLX_SUM = 0, MSCCLX_PROD = 1, MSCCLX_MAX = 2, MSCCLX_MIN = 3, MSCCLX_NUM_REDOPS = 4 } mscclx_redop;
 
 #define MSCCLX_TB_COLS 6 /* rank, send, recv, chan, op_begin, op_end */
@@ -94,6 +101,8 @@ typedef struct {
   int32_t max_workgroups; /* cap on resident workgroups assumed when no device is queried (tests) */
   int32_t staging;     /* 0: a receiver reads a payload in place where that is provably safe; 1: always stage in FIFO slots */
   int32_t workgroups;  /* resident workgroups that share the (threadblock, slice) contexts       */
+  int32_t protocol;    /* 0 automatic, MSCCLX_PROTO_SIMPLE, MSCCLX_PROTO_LL                       */
+  int32_t reserved[3];
 } mscclx_config;
 
 typedef struct {
@@ -108,7 +117,7 @@ typedef struct {
   int32_t zero_copy_messages; /* messages per pass read in place instead of staged  */
   int32_t staged_messages;
   int32_t max_hosted;  /* most contexts any workgroup hosts                         */
-  int32_t reserved;
+  int32_t protocol;    /* MSCCLX_PROTO_SIMPLE or MSCCLX_PROTO_LL                    */
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

@@ -20,6 +20,14 @@
 // Two counter areas alternate between launches: a launch clears the area the next launch will
 // use, so no memset sits between launches.
 //
+// LL variant (flag-in-data, for small pieces): every message is written into its FIFO slot as 16-byte
+// lines {d0, flag, d1, flag}, two lines per 16 bytes of payload.  The flag names the launch and the
+// message, so a receiver needs no counter: its threads load the lines and retry the ones whose flags
+// do not match yet.  The sender's "stores acknowledged -> barrier -> counter store" and the receiver's
+// counter poll drop out of the hand-off.  Each 8-byte half of a line carries its own flag, so the
+// scheme only relies on 8-byte accesses being indivisible.  Free slots are still granted through the
+// tail counters.
+//
 // A workgroup that makes no progress for the watchdog period raises the area's abort word; all
 // other workgroups see it while they poll, and every wave leaves the kernel.
 #include <hip/hip_runtime.h>
@@ -251,11 +259,127 @@ __device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v
 __device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
 __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
 
+// ------------------------------------------------------------------------------------------------
+// LL lines.  One unit (16 payload bytes d0..d3) occupies 32 bytes of a slot: {d0,f,d1,f}{d2,f,d3,f}.
+// f = launch number (10 bits) | message number + 1 (22 bits): never 0, so a cleared slot matches
+// nothing, and what an earlier message or launch left in a line cannot be taken for this message.
+// ------------------------------------------------------------------------------------------------
+constexpr int kLLUnitBytes = 32;
+__device__ __forceinline__ uint32_t ll_flag(uint32_t epoch, u64 seq) { return ((epoch & 0x3ffu) << 22) | (uint32_t)((seq + 1) & 0x3fffffu); }
+__device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { return l0.y == f && l0.w == f && l1.y == f && l1.w == f; }
+
+// What a thread needs to give up on a message that never arrives.
+struct LLWatch {
+  u64* abort_word;
+  mscclx_status* host_status;
+  u64 timeout_ticks;
+  int tb, step, slice;
+  u64 pass;
+};
+
+__device__ __noinline__ void ll_give_up(const LLWatch& w) {
+  if (atomicCAS(w.abort_word, 0ull, 1ull) == 0ull) {
+    mscclx_status* hs = w.host_status;
+    hs->tb = w.tb; hs->step = w.step; hs->slice = w.slice; hs->pass = (int64_t)w.pass; hs->waiting_on = 1;
+    __threadfence_system();
+    __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// o1 (rank buffer) [and llo (LL slot)] = a [(+) b] over n units of 16 bytes.  a is an LL slot row when
+// IN_LL (its lines are retried until they carry `fin`), a rank buffer otherwise; b is a rank buffer.
+template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1>
+__device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* llo, const unsigned char* a, const unsigned char* b, uint32_t n,
+                                              uint32_t fin, uint32_t fout, const LLWatch& watch) {
+  typedef Access<16> A;
+  constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, n * (IN_LL ? kLLUnitBytes : 16));
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, n * (HAS_B ? 16 : (IN_LL ? kLLUnitBytes : 16)));
+  const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? n * 16 : 0);
+  const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * kLLUnitBytes : 0);
+  const uint32_t T = blockDim.x;
+  constexpr int UA = 4;
+  for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
+    u32x4 x[UA], y[UA];
+    if (IN_LL) {
+      u32x4 l0[UA], l1[UA];
+#pragma unroll
+      for (int u = 0; u < UA; ++u) {
+        l0[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes));
+        l1[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
+      }
+      if (HAS_B) {
+#pragma unroll
+        for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
+      }
+      unsigned spins = 0;
+      u64 since = 0;
+      for (;;) {
+        bool all = true;
+#pragma unroll
+        for (int u = 0; u < UA; ++u)
+          if (i + u * T < n && !ll_valid(l0[u], l1[u], fin)) {
+            all = false;
+            l0[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes));
+            l1[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
+          }
+        if (all) break;
+        if ((++spins & 0x7fu) == 0) {
+          const u64 now = wall_clock64();
+          if (!since) since = now;
+          const bool expired = now - since > watch.timeout_ticks;
+          if (expired) ll_give_up(watch);
+          if (expired || load_counter(watch.abort_word) != 0) break;  // the launch is lost; leave with what is there
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UA; ++u) x[u] = u32x4{l0[u].x, l0[u].z, l1[u].x, l1[u].z};
+    } else {
+#pragma unroll
+      for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * 16));
+      if (HAS_B) {
+#pragma unroll
+        for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
+      }
+    }
+    if (HAS_B) {
+#pragma unroll
+      for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
+    }
+    if (OUT_LL) {  // the forwarded lines first: the next rank is waiting for them
+#pragma unroll
+      for (int u = 0; u < UA; ++u) {
+        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes), u32x4{x[u].x, fout, x[u].y, fout});
+        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
+      }
+    }
+    if (HAS_O1) {
+#pragma unroll
+      for (int u = 0; u < UA; ++u) A::template st<X1>(r1, (int)((i + u * T) * 16), x[u]);
+    }
+  }
+}
+
+// rows x n units; rank-buffer rows are `stride_*` units apart, slot rows are packed.
+template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1 = false>
+__device__ __forceinline__ void move_rows_ll(unsigned char* o1, uint64_t stride_o1, unsigned char* llo, const unsigned char* a, uint64_t stride_a,
+                                             const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t fin, uint32_t fout,
+                                             const LLWatch& watch) {
+  for (int r = 0; r < rows; ++r)
+    move_units_ll<R, IN_LL, HAS_B, HAS_O1, OUT_LL, NT1>(HAS_O1 ? o1 + (uint64_t)r * stride_o1 * 16 : nullptr,
+                                                       OUT_LL ? llo + (uint64_t)r * n * kLLUnitBytes : nullptr,
+                                                       a + (uint64_t)r * (IN_LL ? (uint64_t)n * kLLUnitBytes : stride_a * 16),
+                                                       HAS_B ? b + (uint64_t)r * stride_b * 16 : nullptr, n, fin, fout, watch);
+}
+
 // One hosted context = (threadblock, slice): the state of one lane of wave 0.
 struct Context {
   int tb, slice, step, nops, op_begin, send_conn, recv_conn, nsend, nrecv;
   unsigned pass, npasses;
   bool active;
+  uint32_t slice_units;          // units of a chunk this slice covers
+  u64 in_fifo_off;               // LL: where the incoming connection's slots start inside the slice's FIFO region ...
+  uint32_t in_slot_units;        // ... and the units of one slot
   // the step the context stands at
   bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
   int type, hasdep;
@@ -269,7 +393,11 @@ __device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int
 }
 
 // Describe the step `c` stands at: what it must wait for, and whether it moves data.
-__device__ __forceinline__ void describe_step(Context& c, const KernelParams& p) {
+// LL: an incoming message is not announced by a counter; the lane watches the flag in the last
+// 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order, so
+// this is a hint that the message is about to be complete; the threads that read it check every line.
+template <bool LL>
+__device__ __forceinline__ void describe_step(Context& c, const KernelParams& p, uint32_t epoch) {
   const DevOp* op = p.ops + c.op_begin + c.step;
   u64* area = slice_area(p.sync_cur, p, c.slice);
   const u64* flags = area;
@@ -283,22 +411,34 @@ __device__ __forceinline__ void describe_step(Context& c, const KernelParams& p)
   c.w0 = c.w1 = c.w2 = nullptr;
   c.t0 = c.t1 = c.t2 = 0;
   if (op->dep_tb >= 0) { c.w0 = flags + (uint64_t)op->dep_tb * kSyncStrideWords; c.t0 = (u64)c.pass * (u64)op->dep_nops + (u64)op->dep_step + 1; }
-  if (rcv) { c.w1 = heads + (uint64_t)c.recv_conn * kSyncStrideWords; c.t1 = c.rseq + 1; }
+  if (rcv) {
+    if (LL) {
+      const uint64_t done = (uint64_t)c.pass * p.piece_units;
+      const uint32_t n = (uint32_t)(c.slice_units - done < (uint64_t)p.piece_units ? c.slice_units - done : (uint64_t)p.piece_units);
+      const unsigned char* slot = p.fifo + ((uint64_t)c.slice * p.slice_fifo_units + c.in_fifo_off + (c.rseq % (u64)p.depth) * c.in_slot_units) * kLLUnitBytes;
+      c.w1 = (const u64*)(slot + ((uint64_t)op->cnt * n - 1) * kLLUnitBytes + 24);
+      c.t1 = ll_flag(epoch, c.rseq);
+    } else {
+      c.w1 = heads + (uint64_t)c.recv_conn * kSyncStrideWords;
+      c.t1 = c.rseq + 1;
+    }
+  }
   if (snd && c.sseq >= (u64)p.depth) { c.w2 = tails + (uint64_t)c.send_conn * kSyncStrideWords; c.t2 = c.sseq + 1 - (u64)p.depth; }
   c.moves = !(c.type == MSCCLX_OP_NOP || (c.type == MSCCLX_OP_SEND && !op->out_staged));
 }
 
 // Announce the completed step and move the context to its next one.
-__device__ __forceinline__ void finish_step(Context& c, const KernelParams& p) {
+template <bool LL>
+__device__ __forceinline__ void finish_step(Context& c, const KernelParams& p, uint32_t epoch) {
   u64* area = slice_area(p.sync_cur, p, c.slice);
   u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
   u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
-  if (is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, c.sseq + 1);
+  if (!LL && is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, c.sseq + 1);  // LL: the lines announce themselves
   if (is_recv(c.type)) publish(tails + (uint64_t)c.recv_conn * kSyncStrideWords, c.rseq + 1);
   if (c.hasdep) publish(area + (uint64_t)c.tb * kSyncStrideWords, (u64)c.pass * (u64)c.nops + (u64)c.step + 1);
   if (++c.step == c.nops) { c.step = 0; ++c.pass; }
   if (c.pass >= c.npasses) c.active = false;
-  else describe_step(c, p);
+  else describe_step<LL>(c, p, epoch);
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -306,15 +446,20 @@ __device__ __forceinline__ void finish_step(Context& c, const KernelParams& p) {
 // on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
 // reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
 // share the resident workgroups without deadlock.
-template <class R, bool VEC>
+template <class R, bool VEC, bool LL>
 __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_params) {
+  static_assert(VEC || !LL, "LL lines carry 16-byte units");
   constexpr uint64_t UB = VEC ? 16 : R::kElemBytes;
-  // Which of the two counter areas this launch uses is kept on the device (control word 0) and is
-  // flipped by the last workgroup to finish, so a launch carries no host-side state and the same
-  // launch can be replayed (stream order guarantees the flip is seen by the next launch).
+  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;  // bytes one unit takes inside a FIFO slot
+  // The number of launches so far is kept on the device (control word 0) and is advanced by the
+  // last workgroup to finish, so a launch carries no host-side state and the same launch can be
+  // replayed (stream order guarantees the next launch sees the new value).  Its lowest bit picks
+  // which of the two counter areas this launch uses; its low 10 bits mark the LL lines.
   KernelParams p = launch_params;
+  const u64 launch_no = load_counter(p.sync_base);
+  const uint32_t epoch = (uint32_t)launch_no & 0x3ffu;
   {
-    const u64 parity = load_counter(p.sync_base) & 1ull;
+    const u64 parity = launch_no & 1ull;
     p.sync_cur = p.sync_base + kSyncHeaderWords + parity * p.sync_words;
     p.sync_nxt = p.sync_base + kSyncHeaderWords + (parity ^ 1ull) * p.sync_words;
   }
@@ -324,6 +469,9 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
   const int lane = threadIdx.x;
   const bool poller = threadIdx.x < 64;
   const int ctx_begin = p.wg_begin[blockIdx.x], hosted = p.wg_begin[blockIdx.x + 1] - ctx_begin;
+  // LL, one hosted context: nothing else could run while it waits for a message, so the lane does not
+  // watch for it; the moving threads go straight to the lines and retry them until they are there.
+  const bool direct = LL && hosted == 1;
 
   Context c;
   c.active = false;
@@ -336,13 +484,16 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     c.step = 0; c.pass = 0;
     const uint64_t u0 = p.chunk_units * (uint64_t)c.slice / p.slices, u1 = p.chunk_units * (uint64_t)(c.slice + 1) / p.slices;
     c.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
+    c.slice_units = (uint32_t)(u1 - u0);
+    c.in_fifo_off = 0; c.in_slot_units = 0;
+    if (LL && c.recv_conn >= 0) { const DevConn cn = p.conns[c.recv_conn]; c.in_fifo_off = cn.fifo_off; c.in_slot_units = cn.slot_units; }
     c.active = c.nops > 0 && c.npasses > 0;
     // clear, for the next launch, the counters this context is the only writer of
     u64* nxt = slice_area(p.sync_nxt, p, c.slice);
     nxt[(uint64_t)c.tb * kSyncStrideWords] = 0;
     if (c.send_conn >= 0) nxt[((uint64_t)p.ntbs + c.send_conn) * kSyncStrideWords] = 0;
     if (c.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + c.recv_conn) * kSyncStrideWords] = 0;
-    if (c.active) describe_step(c, p);
+    if (c.active) describe_step<LL>(c, p, epoch);
   }
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
   u64 deadline = wall_clock64() + p.timeout_ticks;  // pushed back whenever this workgroup makes progress
@@ -362,14 +513,17 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
       while (choice == -2) {
         bool ready = false;
         if (c.active) {
-          ready = true;
-          if (c.w0) ready = load_counter(c.w0) >= c.t0;
-          if (ready && c.w1) ready = load_counter(c.w1) >= c.t1;
-          if (ready && c.w2) ready = load_counter(c.w2) >= c.t2;
+          // the (up to three) counters are loaded together: one round trip to memory, not one each
+          const bool watch1 = c.w1 && !direct;
+          const u64 v0 = c.w0 ? load_counter(c.w0) : 0;
+          const u64 v1 = watch1 ? load_counter(c.w1) : 0;
+          const u64 v2 = c.w2 ? load_counter(c.w2) : 0;
+          ready = (!c.w0 || v0 >= c.t0) && (!c.w2 || v2 >= c.t2) &&
+                  (!watch1 || (LL ? (uint32_t)(v1 >> 32) == (uint32_t)c.t1 : v1 >= c.t1));
         }
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
-          finish_step(c, p);
+          finish_step<LL>(c, p, epoch);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
         }
@@ -394,7 +548,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
               if (lane == who && atomicCAS((u64*)abort_word, 0ull, 1ull) == 0ull) {
                 int what = 3;
                 if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
-                else if (c.w1 && load_counter(c.w1) < c.t1) what = 1;
+                else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
                 else if (c.w2 && load_counter(c.w2) < c.t2) what = 2;
                 mscclx_status* hs = p.host_status;
                 hs->tb = c.tb; hs->step = c.step; hs->slice = c.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
@@ -429,7 +583,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
       const uint64_t u0 = cs * (uint64_t)j / p.slices, u1 = cs * (uint64_t)(j + 1) / p.slices;
       const uint64_t off = u0 + pass * (uint64_t)p.piece_units;
       const uint32_t n = (uint32_t)((u1 - off) < (uint64_t)p.piece_units ? (u1 - off) : (uint64_t)p.piece_units);
-      unsigned char* const fifo_slice = p.fifo + (uint64_t)j * p.slice_fifo_units * UB;
+      unsigned char* const fifo_slice = p.fifo + (uint64_t)j * p.slice_fifo_units * FB;
       const unsigned char* lsrc = nullptr;
       unsigned char* ldst = nullptr;
       if (t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE)
@@ -438,10 +592,11 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
         ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * cs + off) * UB;
       // out: the FIFO slot to fill, or null when the receiver will read this step's payload in place
       unsigned char* out = nullptr;
+      u64 sseq = 0, rseq = 0;
       if (snd && op.out_staged) {
         const DevConn cn = p.conns[tb.send_conn];
-        const u64 sseq = pass * (u64)tb.nsend + (u64)op.send_seq;
-        out = fifo_slice + (cn.fifo_off + (sseq % (u64)p.depth) * cn.slot_units) * UB;
+        sseq = pass * (u64)tb.nsend + (u64)op.send_seq;
+        out = fifo_slice + (cn.fifo_off + (sseq % (u64)p.depth) * cn.slot_units) * FB;
       }
       // in: the incoming payload -- packed in a FIFO slot, or still where the sender has it (then
       // its rows are a chunk apart, like any rank buffer)
@@ -453,10 +608,27 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
           in_stride = cs;
         } else {
           const DevConn cn = p.conns[tb.recv_conn];
-          const u64 rseq = pass * (u64)tb.nrecv + (u64)op.recv_seq;
-          in = fifo_slice + (cn.fifo_off + (rseq % (u64)p.depth) * cn.slot_units) * UB;
+          rseq = pass * (u64)tb.nrecv + (u64)op.recv_seq;
+          in = fifo_slice + (cn.fifo_off + (rseq % (u64)p.depth) * cn.slot_units) * FB;
         }
       }
+      if (LL && (rcv || snd)) {
+        // every message goes through a slot, as lines
+        const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
+        const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tbi, sh_step, j, pass};
+        switch (t) {
+          case MSCCLX_OP_SEND: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, lsrc, cs, nullptr, 0, op.cnt, n, fin, fout, watch); break;
+          case MSCCLX_OP_RECV:
+            if (op.nt_store) move_rows_ll<R, true, false, true, false, true>(ldst, cs, nullptr, in, n, nullptr, 0, op.cnt, n, fin, fout, watch);
+            else             move_rows_ll<R, true, false, true, false>(ldst, cs, nullptr, in, n, nullptr, 0, op.cnt, n, fin, fout, watch);
+            break;
+          case MSCCLX_OP_RCS: move_rows_ll<R, true, false, true, true>(ldst, cs, out, in, n, nullptr, 0, op.cnt, n, fin, fout, watch); break;
+          case MSCCLX_OP_RRC: move_rows_ll<R, true, true, true, false>(ldst, cs, nullptr, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
+          case MSCCLX_OP_RRS: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
+          case MSCCLX_OP_RRCS: move_rows_ll<R, true, true, true, true>(ldst, cs, out, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
+          default: break;
+        }
+      } else
       switch (t) {
         case MSCCLX_OP_SEND: move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
         case MSCCLX_OP_RECV:
@@ -486,7 +658,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (poller) {
-      if (lane == choice) finish_step(c, p);
+      if (lane == choice) finish_step<LL>(c, p, epoch);
       deadline = wall_clock64() + p.timeout_ticks;
     }
 #ifdef MSCCLX_PROFILE
@@ -502,7 +674,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     const u64 finished = __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (finished == (u64)gridDim.x - 1) {
       publish(p.sync_base + 1, 0);
-      publish(p.sync_base, (load_counter(p.sync_base) & 1ull) ^ 1ull);
+      publish(p.sync_base, launch_no + 1);
     }
   }
 #ifdef MSCCLX_PROFILE
@@ -520,30 +692,31 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
 
-template <int DT, int OP> static kernel_fn pick_vec(bool vec) {
-  return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true> : (kernel_fn)exec_kernel<Reducer<DT, OP>, false>;
+template <int DT, int OP> static kernel_fn pick_vec(bool vec, bool ll) {
+  if (ll) return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, true> : nullptr;
+  return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false> : (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false>;
 }
-template <int DT> static kernel_fn pick_op(int op, bool vec) {
+template <int DT> static kernel_fn pick_op(int op, bool vec, bool ll) {
   switch (op) {
-    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec);
-    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec);
-    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec);
-    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec);
+    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec, ll);
+    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec, ll);
+    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec, ll);
+    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec, ll);
     default: return nullptr;
   }
 }
-static kernel_fn pick_kernel(int dtype, int op, bool vec) {
+static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll) {
   switch (dtype) {
-    case MSCCLX_U8: return pick_op<MSCCLX_U8>(op, vec);
-    case MSCCLX_I8: return pick_op<MSCCLX_I8>(op, vec);
-    case MSCCLX_I32: return pick_op<MSCCLX_I32>(op, vec);
-    case MSCCLX_U32: return pick_op<MSCCLX_U32>(op, vec);
-    case MSCCLX_I64: return pick_op<MSCCLX_I64>(op, vec);
-    case MSCCLX_U64: return pick_op<MSCCLX_U64>(op, vec);
-    case MSCCLX_F16: return pick_op<MSCCLX_F16>(op, vec);
-    case MSCCLX_BF16: return pick_op<MSCCLX_BF16>(op, vec);
-    case MSCCLX_F32: return pick_op<MSCCLX_F32>(op, vec);
-    case MSCCLX_F64: return pick_op<MSCCLX_F64>(op, vec);
+    case MSCCLX_U8: return pick_op<MSCCLX_U8>(op, vec, ll);
+    case MSCCLX_I8: return pick_op<MSCCLX_I8>(op, vec, ll);
+    case MSCCLX_I32: return pick_op<MSCCLX_I32>(op, vec, ll);
+    case MSCCLX_U32: return pick_op<MSCCLX_U32>(op, vec, ll);
+    case MSCCLX_I64: return pick_op<MSCCLX_I64>(op, vec, ll);
+    case MSCCLX_U64: return pick_op<MSCCLX_U64>(op, vec, ll);
+    case MSCCLX_F16: return pick_op<MSCCLX_F16>(op, vec, ll);
+    case MSCCLX_BF16: return pick_op<MSCCLX_BF16>(op, vec, ll);
+    case MSCCLX_F32: return pick_op<MSCCLX_F32>(op, vec, ll);
+    case MSCCLX_F64: return pick_op<MSCCLX_F64>(op, vec, ll);
     default: return nullptr;
   }
 }
@@ -611,8 +784,8 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   if (cfg.max_workgroups > 0) {
     for (int i = 0; i < 4; ++i) capacity[i] = cfg.max_workgroups;
   } else {
-    kernel_fn k = pick_kernel(dtype, redop, vec);
-    int rc = query_capacity(k, &num_cus, capacity);
+    const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
+    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll), &num_cus, capacity);
     if (rc) return rc;
   }
   Geometry g;
@@ -631,7 +804,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     const Geometry& g = gg;
     info->workgroups = g.workgroups;
     info->max_hosted = g.max_hosted;
-    info->reserved = 0;
+    info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
     info->threads = g.threads;
     info->slices = g.slices;
     info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);
@@ -686,7 +859,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   DeviceState* d = new DeviceState();
   plan->dev = d;
   HIP_TRY(hipGetDevice(&d->device));
-  d->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0);
+  d->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0);
   if (!d->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
 
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
@@ -747,7 +920,8 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipHostMalloc((void**)&d->host_status, sizeof(mscclx_status), hipHostMallocDefault));
   std::memset(d->host_status, 0, sizeof(mscclx_status));
   d->workspace = (unsigned char*)workspace;
-  HIP_TRY(hipMemset(d->workspace, 0, g.fifo_byte_off));  // both counter areas
+  // both counter areas; LL: the slots too, so that no line of whatever the memory held carries a flag
+  HIP_TRY(hipMemset(d->workspace, 0, g.ll ? g.workspace_bytes : g.fifo_byte_off));
   HIP_TRY(hipDeviceSynchronize());
   HIP_TRY(hipEventCreate(&d->ev0));
   HIP_TRY(hipEventCreate(&d->ev1));
@@ -764,7 +938,7 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
   hipStream_t s = (hipStream_t)stream;
   if (d->dirty) {  // the previous launch gave up half-way: its counters mean nothing
     HIP_TRY(hipStreamSynchronize(s));
-    HIP_TRY(hipMemset(d->workspace, 0, g.fifo_byte_off));
+    HIP_TRY(hipMemset(d->workspace, 0, g.ll ? g.workspace_bytes : g.fifo_byte_off));  // LL: launches count from 0 again, old lines must go
     HIP_TRY(hipDeviceSynchronize());
     d->dirty = false;
   }

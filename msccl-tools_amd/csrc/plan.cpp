@@ -378,6 +378,13 @@ static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
   return w;
 }
 
+static int decide_geometry_simple_retry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg, int num_cus,
+                                        const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
+  mscclx_config simple = cfg;
+  simple.protocol = MSCCLX_PROTO_SIMPLE;
+  return decide_geometry(plan, chunk_bytes, dtype, simple, num_cus, capacity_by_threads, fifo_budget_bytes, out);
+}
+
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);
@@ -389,6 +396,8 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.vector_path = (chunk_bytes % 16 == 0) ? 1 : 0;
   g.unit_bytes = g.vector_path ? 16 : elem;
   g.chunk_units = chunk_bytes / g.unit_bytes;
+  if (cfg.protocol < 0 || cfg.protocol > MSCCLX_PROTO_LL) return fail(MSCCLX_ERR_INVALID_ARG, "unknown protocol");
+  if (cfg.protocol == MSCCLX_PROTO_LL && !g.vector_path) return fail(MSCCLX_ERR_UNSUPPORTED, "the LL protocol needs chunks that are a multiple of 16 bytes");
   g.staging = cfg.staging ? 1 : 0;
   const int64_t ntbs = (int64_t)plan.tbs.size();
   if (ntbs == 0) return fail(MSCCLX_ERR_BAD_IR, "the algorithm has no threadblocks");
@@ -437,16 +446,34 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   const uint64_t longest_slice = (g.chunk_units + slices - 1) / slices;
   uint64_t piece_units = cfg.piece_bytes ? std::max<uint64_t>(1, (uint64_t)cfg.piece_bytes / g.unit_bytes) : longest_slice;
   piece_units = std::min(piece_units, longest_slice);
+  // protocol: flag-in-data lines pay twice the slot traffic and stage every message to take the
+  // counter round trip out of a hand-off.  Chosen only on request: measured on MI355X a hop is bound
+  // as much by the receiving workgroup's own step-to-step time as by the hand-off, and reading
+  // payloads in place (which LL gives up) wins at every piece size tried.
+  g.ll = cfg.protocol == MSCCLX_PROTO_LL ? 1 : 0;
+  if (g.ll) g.staging = 1;
+  const uint64_t fifo_unit_bytes = (uint64_t)g.unit_bytes * (g.ll ? 2 : 1);
   uint64_t slot_chunks = 0;  // FIFO units per slice per unit of piece
   for (const Conn& c : plan.conns) slot_chunks += (uint64_t)depth * (g.staging ? c.max_cnt : c.max_staged_cnt);
   if (!cfg.piece_bytes && slot_chunks) {
-    const uint64_t cap = fifo_budget_bytes / (slot_chunks * (uint64_t)slices * g.unit_bytes);
+    const uint64_t cap = fifo_budget_bytes / (slot_chunks * (uint64_t)slices * fifo_unit_bytes);
     const uint64_t floor_units = std::max<uint64_t>(1, 16384 / g.unit_bytes);
     piece_units = std::min(piece_units, std::max(cap, std::min(floor_units, longest_slice)));
   }
-  if (piece_units > 0x3fffffffu / 16) piece_units = 0x3fffffffu / 16;
+  const uint64_t most_units = 0x3fffffffu / (g.ll ? 32 : 16);  // byte offsets inside a piece (a slot row, in LL lines) stay below 2^30
+  if (piece_units > most_units) piece_units = most_units;
   g.piece_units = (uint32_t)piece_units;
   g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
+  if (g.ll) {  // a message's flag carries its sequence number in 22 bits
+    int64_t most = 0;
+    for (const Conn& c : plan.conns) most = std::max<int64_t>(most, c.nmsg);
+    if (most * g.passes >= (1 << 22) - 1) {
+      if (cfg.protocol == MSCCLX_PROTO_LL) return fail(MSCCLX_ERR_UNSUPPORTED, "too many messages per connection for the LL protocol");
+      g.ll = 0;
+      g.staging = cfg.staging ? 1 : 0;
+      return decide_geometry_simple_retry(plan, chunk_bytes, dtype, cfg, num_cus, capacity_by_threads, fifo_budget_bytes, out);
+    }
+  }
 
   // threads: enough to cover a piece with 8 16-byte loads per thread
   int threads = cfg.threads;
@@ -517,7 +544,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
   const uint64_t sync_bytes = ((kSyncHeaderWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
   g.fifo_byte_off = sync_bytes;
-  g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * g.unit_bytes + 256;
+  g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * fifo_unit_bytes + 256;
   *out = std::move(g);
   return MSCCLX_OK;
 }

@@ -80,6 +80,7 @@ struct Geometry {
   uint32_t piece_units = 0;
   int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
   int32_t staging = 0;            // 1: every message goes through a FIFO slot
+  int32_t ll = 0;                 // 1: flag-in-data lines in the slots (implies staging); FIFO bytes double
   int32_t workgroups = 0;         // resident workgroups; each hosts up to kMaxHosted (threadblock, slice) contexts
   int32_t max_hosted = 0;
   std::vector<int32_t> wg_begin, ctx_tb, ctx_slice;  // the hosting table
@@ -96,7 +97,7 @@ struct KernelParams {
   const DevOp* ops;
   const DevConn* conns;
   void* const* bufs;            // [nranks*3]
-  unsigned long long* sync_base; // control block: word 0 = which counter area this launch uses, word 1 = workgroups finished
+  unsigned long long* sync_base; // control block: word 0 = launches finished so far (its parity picks the counter area), word 1 = workgroups finished
   unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
   unsigned long long* sync_nxt;  // next launch's counters   } from the control block
   unsigned char* fifo;

@@ -24,6 +24,7 @@ DTYPE_CODES = {"uint8": 0, "int8": 1, "int32": 2, "uint32": 3, "int64": 4, "uint
 DTYPE_SIZES = {"uint8": 1, "int8": 1, "int32": 4, "uint32": 4, "int64": 8, "uint64": 8,
                "float16": 2, "bfloat16": 2, "float32": 4, "float64": 8}
 REDOP_CODES = {"sum": 0, "prod": 1, "max": 2, "min": 3}
+PROTOCOL_CODES = {"auto": 0, "simple": 1, "ll": 2, "Simple": 1, "LL": 2}
 
 # every symbol include/mscclx.h declares
 EXPORTED_SYMBOLS = (
@@ -53,7 +54,8 @@ class PlanDesc(ctypes.Structure):
 class Config(ctypes.Structure):
     _fields_ = [("slices", ctypes.c_int32), ("piece_bytes", ctypes.c_int32), ("fifo_depth", ctypes.c_int32),
                 ("threads", ctypes.c_int32), ("timeout_ms", ctypes.c_int32), ("max_workgroups", ctypes.c_int32),
-                ("staging", ctypes.c_int32), ("workgroups", ctypes.c_int32)]
+                ("staging", ctypes.c_int32), ("workgroups", ctypes.c_int32),
+                ("protocol", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
 
 
 class Info(ctypes.Structure):
@@ -61,7 +63,7 @@ class Info(ctypes.Structure):
                 ("piece_bytes", ctypes.c_int32), ("fifo_depth", ctypes.c_int32), ("passes", ctypes.c_int32),
                 ("connections", ctypes.c_int32), ("vector_path", ctypes.c_int32),
                 ("zero_copy_messages", ctypes.c_int32), ("staged_messages", ctypes.c_int32),
-                ("max_hosted", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("max_hosted", ctypes.c_int32), ("protocol", ctypes.c_int32),
                 ("workspace_bytes", ctypes.c_uint64), ("algorithmic_units", ctypes.c_uint64)]
 
     def as_dict(self):
@@ -153,7 +155,7 @@ class Plan:
         for k, v in knobs.items():
             if not hasattr(cfg, k):
                 raise TypeError(f"unknown executor knob {k!r}")
-            setattr(cfg, k, int(v))
+            setattr(cfg, k, PROTOCOL_CODES[v] if k == "protocol" and isinstance(v, str) else int(v))
         info = Info()
         _check(self.lib, self.lib.mscclx_plan_configure(self.handle, chunk_bytes, DTYPE_CODES[dtype], REDOP_CODES[redop],
                                                        ctypes.byref(cfg), ctypes.byref(info)))

@@ -20,11 +20,11 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
     assert declared == set(EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(mscclx_lib, name), name
-    assert mscclx_lib.mscclx_version() == 1
+    assert mscclx_lib.mscclx_version() == 2
 
 
 def test_struct_layouts_match_header():
-    assert ctypes.sizeof(binding.Config) == 32
+    assert ctypes.sizeof(binding.Config) == 48
     assert ctypes.sizeof(binding.Info) == 64
     assert ctypes.sizeof(binding.Status) == 32
 
@@ -151,7 +151,7 @@ def test_launch_before_bind_is_a_state_error(mscclx_lib):
 def test_zero_copy_analysis(mscclx_lib):
     """Which payloads may be read in place (plan.cpp: find_zero_copy_messages)."""
     def counts(xml):
-        info = Plan(parse_algo_xml(xml)).configure(1 << 20, "float32", max_workgroups=4096)
+        info = Plan(parse_algo_xml(xml)).configure(1 << 20, "float32", max_workgroups=4096, protocol="simple")
         return info.zero_copy_messages, info.staged_messages
     n = 8
     # ring all-reduce: per chunk the first 's' (its source is overwritten only by the final value,
@@ -168,3 +168,26 @@ def test_zero_copy_analysis(mscclx_lib):
         ir_samples._step(1, "cpy", "o", 0, "i", 0, 1)).replace('<gpu id="0" i_chunks="1" o_chunks="0"', '<gpu id="0" i_chunks="1" o_chunks="1"')
     assert counts(ir_samples.RRC_CPY_NOP_XML) == (1, 0)
     assert counts(xml) == (0, 1)
+
+
+def test_protocol_choice(mscclx_lib):
+    """Flag-in-data lines are used on request only, double the slot bytes and stage every message."""
+    p = Plan(parse_algo_xml(ir_samples.ring_allreduce_xml(8)))
+    for chunk in (8 << 20, 64 << 10):
+        auto = p.configure(chunk, "float32", max_workgroups=2048)
+        assert auto.protocol == binding.PROTOCOL_CODES["simple"] and auto.zero_copy_messages > 0
+    small = p.configure(64 << 10, "float32", max_workgroups=2048, protocol="ll")
+    assert small.protocol == binding.PROTOCOL_CODES["ll"]
+    assert small.zero_copy_messages == 0 and small.staged_messages == 8 * 14
+    # same geometry, every message staged: the LL workspace holds twice the slot bytes
+    a = p.configure(8 << 20, "float32", max_workgroups=2048, protocol="ll", slices=16, piece_bytes=65536)
+    b = p.configure(8 << 20, "float32", max_workgroups=2048, protocol="simple", staging=1, slices=16, piece_bytes=65536)
+    assert a.protocol == binding.PROTOCOL_CODES["ll"] and a.staged_messages == b.staged_messages == 8 * 14
+    slots = 8 * 2 * 65536 * 16  # connections x depth x piece x slices
+    assert b.workspace_bytes - slots == a.workspace_bytes - 2 * slots  # what is left are the counters
+    with pytest.raises(MscclxError) as e:
+        p.configure(1000 * 4 + 4, "int32", max_workgroups=2048, protocol="ll")  # lines carry 16-byte units
+    assert e.value.code == binding.ERR_UNSUPPORTED
+    with pytest.raises(MscclxError) as e:
+        p.configure(64 << 10, "float32", max_workgroups=2048, protocol=7)
+    assert e.value.code == binding.ERR_INVALID_ARG

@@ -40,17 +40,23 @@ def oracle_run(xml, w, inputs_np):
     return oc.extract_outputs(algo, bufs, E)
 
 
-@pytest.mark.parametrize("staging", [0, 1])
+# the three ways a message can cross a connection
+MODES = {"in-place": dict(protocol="simple", staging=0), "staged": dict(protocol="simple", staging=1), "ll": dict(protocol="ll")}
+
+
+@pytest.mark.parametrize("mode", sorted(MODES))
 @pytest.mark.parametrize("source", ["msccl-tools", "this-package"])
 @pytest.mark.parametrize("key", sorted(WORKLOADS))
-def test_config_reduced_size_vs_oracle(key, source, staging):
-    """staging=0: payloads are read in place where the plan proved that safe; staging=1: every
-    message is copied through a FIFO slot.  Both must give the interpreter's bits."""
+def test_config_reduced_size_vs_oracle(key, source, mode):
+    """in-place: payloads are read where the sender keeps them when the plan proved that safe;
+    staged: every message is copied through a FIFO slot; ll: every message goes through a slot as
+    flag-in-data lines.  All must give the interpreter's bits."""
     w = WORKLOADS[key].scaled(REDUCED[key])
     xml = golden_util.load(GOLDEN_OF[key]) if source == "msccl-tools" else WORKLOADS[key].build()
     x = [numpy_input(w, r) for r in range(w.ranks)]
-    got, info = device_run(xml, w, x, staging=staging)
-    assert (info.zero_copy_messages == 0) == bool(staging)
+    got, info = device_run(xml, w, x, **MODES[mode])
+    assert (info.zero_copy_messages == 0) == (mode != "in-place")
+    assert info.protocol == (2 if mode == "ll" else 1)
     want = oracle_run(xml, w, x)
     for r in range(w.ranks):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
@@ -60,7 +66,7 @@ def test_config_reduced_size_vs_oracle(key, source, staging):
 def test_reference_emitted_programs_vs_oracle(name):
     """Every program msccl-tools' compiler emitted for the fixtures, whatever its collective: all
     three buffers of every rank start from the same random bits on both sides and must end equal,
-    with payloads read in place (staging=0) and with everything staged (staging=1)."""
+    with payloads read in place, with everything staged, and with flag-in-data lines."""
     from msccl.executor import Executor
     xml = golden_util.load(name)
     algo = oi.parse_xml(xml)
@@ -70,10 +76,10 @@ def test_reference_emitted_programs_vs_oracle(name):
             for g in algo.gpus]
     want = [{b: v.copy() for b, v in d.items()} for d in init]
     oi.Interpreter(algo).run(want, E, "float32")
-    for staging in (0, 1):
+    for mode in sorted(MODES):
         ex = Executor(xml)
-        print(f"case: {name} staging={staging}", flush=True)
-        ex.setup(E * 4, "float32", staging=staging)
+        print(f"case: {name} mode={mode}", flush=True)
+        ex.setup(E * 4, "float32", **MODES[mode])
         ins = [torch.from_numpy(d["i"]).cuda() if d["i"].size else None for d in init]
         outs = [torch.from_numpy(d["o"]).cuda() if d["o"].size else None for d in init]
         for r, d in enumerate(init):
@@ -85,7 +91,7 @@ def test_reference_emitted_programs_vs_oracle(name):
             got = {"i": ins[r], "o": outs[r], "s": None if ex._scratch[r] is None else ex._scratch[r].view(torch.float32)}
             for b in "ios":
                 if want[r][b].size:
-                    assert np.array_equal(got[b].cpu().numpy().view(np.uint32), want[r][b].view(np.uint32)), (name, r, b, staging)
+                    assert np.array_equal(got[b].cpu().numpy().view(np.uint32), want[r][b].view(np.uint32)), (name, r, b, mode)
 
 
 def torch_fold(order, operands):
@@ -140,7 +146,7 @@ def test_aliased_buffers_fall_back_to_staging():
     xml = golden_util.load("alltoall_allpairs_4r")
     E = 1024
     ex = Executor(xml)
-    ex.setup(E * 4, "int32")
+    ex.setup(E * 4, "int32", protocol="simple")
     assert ex.info.zero_copy_messages > 0
     n = 4
     bufs = [torch.arange(n * E, dtype=torch.int32, device="cuda:0") + 100000 * r for r in range(n)]
@@ -148,7 +154,7 @@ def test_aliased_buffers_fall_back_to_staging():
     outs = [torch.zeros(n * E, dtype=torch.int32, device="cuda:0") for _ in range(n)]
     ex.run(shadow, outs)                       # out of place: the reference result
     ex2 = Executor(xml)
-    ex2.setup(E * 4, "int32")
+    ex2.setup(E * 4, "int32", protocol="simple")
     ex2.bind(bufs, [b[: n * E] for b in bufs])  # same memory for 'i' and 'o'
     assert ex2.info.zero_copy_messages == 0 and ex2.info.staged_messages > 0
 

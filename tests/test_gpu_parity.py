@@ -79,50 +79,97 @@ def assert_same(got, want, keys=("i", "o")):
                 raise AssertionError(f"rank {r} buffer {k}: {bad.size} bytes differ, first at byte {bad[0]}")
 
 
-def test_fusion_chain_f32():
-    got, want, _, _ = run_both(ir_samples.FUSION_CHAIN_XML, 1024, "float32")
+# How messages cross connections: counters with payloads read in place where that is safe, counters
+# with every payload copied through a slot, flag-in-data lines.
+MODES = {"in-place": dict(protocol="simple", staging=0), "staged": dict(protocol="simple", staging=1), "ll": dict(protocol="ll")}
+PROTOCOLS = ["simple", "ll"]
+
+
+@pytest.mark.parametrize("protocol", PROTOCOLS)
+def test_fusion_chain_f32(protocol):
+    got, want, _, info = run_both(ir_samples.FUSION_CHAIN_XML, 1024, "float32", protocol=protocol)
+    assert info.protocol == PROTOCOLS.index(protocol) + 1
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "int32", "uint8", "float64", "int64", "int8"])
-def test_ring_allreduce_dtypes(dtype):
-    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(8), 4096, dtype)
+def test_ring_allreduce_dtypes(dtype, protocol):
+    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(8), 4096, dtype, protocol=protocol)
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("redop", ["prod", "max", "min"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "int32"])
-def test_ring_allreduce_redops(dtype, redop):
-    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(4), 2048, dtype, redop=redop)
+def test_ring_allreduce_redops(dtype, redop, protocol):
+    got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(4), 2048, dtype, redop=redop, protocol=protocol)
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("n,inst", [(2, 1), (8, 4), (5, 2)])
-def test_ring_allgather(n, inst):
-    got, want, _, _ = run_both(ir_samples.ring_allgather_xml(n, inst), 8192, "int32")
+def test_ring_allgather(n, inst, protocol):
+    got, want, _, _ = run_both(ir_samples.ring_allgather_xml(n, inst), 8192, "int32", protocol=protocol)
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("n", [2, 4, 8])
-def test_allpairs_scratch_and_deps(n):
-    got, want, _, _ = run_both(ir_samples.allpairs_allreduce_xml(n), 4096, "float32")
+def test_allpairs_scratch_and_deps(n, protocol):
+    got, want, _, _ = run_both(ir_samples.allpairs_allreduce_xml(n), 4096, "float32", protocol=protocol)
     assert_same(got, want)
 
 
-@pytest.mark.parametrize("staging", [0, 1])
-def test_ncclize_schema(staging):
+@pytest.mark.parametrize("mode", sorted(MODES))
+def test_ncclize_schema(mode):
     """Documents shaped like msccl-tools' ncclize output: copy threadblocks, inplace=0, sender-side
     src on receives, rrc chains."""
     for n in (2, 3, 5):
-        got, want, _, _ = run_both(ir_samples.ncclize_style_allgather_xml(n), 5000, "int32", in_elems=5000, staging=staging)
+        got, want, _, _ = run_both(ir_samples.ncclize_style_allgather_xml(n), 5000, "int32", in_elems=5000, **MODES[mode])
         assert_same(got, want)
-    got, want, _, _ = run_both(ir_samples.ncclize_style_allreduce_xml(), 7000, "float32", staging=staging)
+    got, want, _, _ = run_both(ir_samples.ncclize_style_allreduce_xml(), 7000, "float32", **MODES[mode])
     assert_same(got, want)
 
 
-def test_rrc_cpy_nop():
-    got, want, _, _ = run_both(ir_samples.RRC_CPY_NOP_XML, 1000 * 4, "int32")
+@pytest.mark.parametrize("protocol", PROTOCOLS)
+def test_rrc_cpy_nop(protocol):
+    got, want, _, _ = run_both(ir_samples.RRC_CPY_NOP_XML, 1000 * 4, "int32", protocol=protocol)
     assert_same(got, want)
+
+
+@pytest.mark.parametrize("knobs", [
+    dict(slices=1, piece_bytes=256, fifo_depth=2),                  # 63 passes: every slot is reused 30 times
+    dict(slices=3, piece_bytes=1024, fifo_depth=3, workgroups=4),   # many contexts per workgroup: the lane watches the last line
+    dict(slices=2, piece_bytes=4096, fifo_depth=2, workgroups=64),  # one context per workgroup: threads go straight to the lines
+    dict(slices=8, threads=64),
+    dict(slices=1, threads=512),                                    # one big piece per step
+])
+def test_ll_geometry_and_relaunch(knobs):
+    """Flag-in-data lines over many passes (slot reuse), both ways of noticing a message, and several
+    launches on one binding: a launch must not take lines the previous launch left for its own."""
+    from msccl.executor import Executor, collective_buffers
+    xml = ir_samples.ring_allreduce_xml(8, 2)
+    algo = oi.parse_xml(xml)
+    E = 4000
+    ex = Executor(xml)
+    print(f"case: ll relaunch knobs={knobs}", flush=True)
+    info = ex.setup(E * 4, "float32", protocol="ll", **knobs)
+    assert info.protocol == 2 and info.zero_copy_messages == 0
+    keep = None
+    for it in range(4):
+        x = make_inputs(8, 16 * E, "float32", seed=300 + it)
+        if keep is None:
+            keep = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+        else:
+            for r in range(8):
+                keep[0][r].copy_(torch.from_numpy(x[r]))
+        ex.run(keep[0], keep[1])
+        torch.cuda.synchronize()
+        want = oc.place_inputs(algo, x, E, "float32")
+        oi.Interpreter(algo).run(want, E, "float32")
+        for r in range(8):
+            assert np.array_equal(keep[0][r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (it, r)
 
 
 @pytest.mark.parametrize("chunk_elems,dtype", [(1, "float32"), (3, "float32"), (4, "float32"), (1001, "float16"),
@@ -144,6 +191,7 @@ def test_ragged_chunk_sizes(chunk_elems, dtype):
     dict(slices=2, staging=1, workgroups=7),
 ])
 def test_geometry_knobs(knobs):
+    knobs = dict(protocol="simple", **knobs)
     got, want, _, info = run_both(ir_samples.ring_allreduce_xml(8, 2), 40000, "float32", **knobs)
     assert info.slices == knobs["slices"] and info.threads == knobs.get("threads", info.threads)
     assert_same(got, want)
@@ -227,6 +275,34 @@ def test_watchdog_reports_instead_of_hanging():
     # same plan, sane limit: completes and delivers
     ex2 = Executor(xml)
     ex2.setup(nbytes, "uint8", slices=4)
+    ins, outs, _ = collective_buffers(ex2.tables, nbytes, "uint8", inputs=x)
+    ex2.run(ins, outs)
+    assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
+
+
+def test_watchdog_in_ll_mode():
+    """Flag-in-data lines, one context per workgroup: the receiving threads themselves wait on the
+    lines, so they carry the watchdog.  Same scenario as above; afterwards the same binding is launched
+    again (the library clears counters and lines after a lost launch) -- it times out the same way,
+    cleanly -- and a fresh plan with the default limit delivers."""
+    from msccl.executor import Executor, MscclxError, collective_buffers
+    xml = ir_samples.slow_producer_xml(24)
+    nbytes = 64 << 20
+    ex = Executor(xml)
+    info = ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, protocol="ll")
+    assert info.protocol == 2
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    for attempt in range(2):
+        print(f"case: ll watchdog launch {attempt}", flush=True)
+        ex.launch()
+        with pytest.raises(MscclxError) as e:
+            ex.wait()
+        assert "watchdog" in str(e.value) and "rank 1 tb 0 step 0" in str(e.value) and "incoming message" in str(e.value)
+        torch.cuda.synchronize()
+    ex2 = Executor(xml)
+    ex2.setup(nbytes, "uint8", slices=4, protocol="ll")
     ins, outs, _ = collective_buffers(ex2.tables, nbytes, "uint8", inputs=x)
     ex2.run(ins, outs)
     assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
