@@ -292,21 +292,22 @@ template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1>
 __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* llo, const unsigned char* a, const unsigned char* b, uint32_t n,
                                               uint32_t fin, uint32_t fout, const LLWatch& watch) {
   typedef Access<16> A;
-  constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
+  // XV: the retried loads must really be issued again each time round the loop (bit 31 = volatile, for the compiler only)
+  constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, XV = (int)(0x80000000u | MSCCLX_AUX), X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, n * (IN_LL ? kLLUnitBytes : 16));
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, n * (HAS_B ? 16 : (IN_LL ? kLLUnitBytes : 16)));
   const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? n * 16 : 0);
   const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * kLLUnitBytes : 0);
   const uint32_t T = blockDim.x;
-  constexpr int UA = 4;
+  constexpr int UA = 2;  // small pieces: few lines per thread, few registers
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
     u32x4 x[UA], y[UA];
     if (IN_LL) {
       u32x4 l0[UA], l1[UA];
 #pragma unroll
       for (int u = 0; u < UA; ++u) {
-        l0[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes));
-        l1[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
+        l0[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes));
+        l1[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
       }
       if (HAS_B) {
 #pragma unroll
@@ -320,8 +321,8 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
         for (int u = 0; u < UA; ++u)
           if (i + u * T < n && !ll_valid(l0[u], l1[u], fin)) {
             all = false;
-            l0[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes));
-            l1[u] = A::template ld<XF>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
+            l0[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes));
+            l1[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
           }
         if (all) break;
         if ((++spins & 0x7fu) == 0) {
@@ -372,73 +373,124 @@ __device__ __forceinline__ void move_rows_ll(unsigned char* o1, uint64_t stride_
                                                        HAS_B ? b + (uint64_t)r * stride_b * 16 : nullptr, n, fin, fout, watch);
 }
 
+// What the workgroup does for one step of one context: operands as byte addresses, filled in by the
+// context's lane when the context arrives at the step and handed to the other threads through LDS.
+struct Move {
+  u64 a;      // source: the incoming payload (slot, or the sender's buffer) or the local source
+  u64 dst;    // local destination, which is also the local operand of a reduction
+  u64 out;    // slot to fill
+  uint32_t n; // units per row
+  int rows, kind;
+};
+// kind: how the operands are used.  Rows of a rank buffer are a chunk apart, rows in a slot are packed.
+enum {
+  kHasB = 1,     // reduce: a (+) dst
+  kHasO2 = 2,    // also forward the result into `out`
+  kNt1 = 4,      // the first destination is never read again
+  kLLKind = 8,   // flag-in-data lines: bits 0-2 then say which movement (kLL* below)
+  kAPacked = 16, // a is a slot
+  kToSlot = 32,  // the first (only) destination is `out` instead of dst
+};
+enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
+
 // One hosted context = (threadblock, slice): the state of one lane of wave 0.
 struct Context {
   int tb, slice, step, nops, op_begin, send_conn, recv_conn, nsend, nrecv;
   unsigned pass, npasses;
   bool active;
-  uint32_t slice_units;          // units of a chunk this slice covers
-  u64 in_fifo_off;               // LL: where the incoming connection's slots start inside the slice's FIFO region ...
-  uint32_t in_slot_units;        // ... and the units of one slot
+  u64 slice_begin;               // first unit of a chunk this slice covers ...
+  uint32_t slice_units;          // ... and how many
+  u64 in_slots, out_slots;       // byte address of the first slot of the incoming / outgoing connection, in this slice
+  uint32_t in_slot_units, out_slot_units;
   // the step the context stands at
   bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
   int type, hasdep;
-  u64 sseq, rseq;
+  uint32_t sseq, rseq;      // number of the message this step sends / receives on its connection (all passes)
   const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
-  u64 t0, t1, t2;           // ... until they reach these values
+  uint32_t t0, t1, t2;      // ... until they reach these values (every counter of a launch stays below 2^32)
+  Move m;
 };
 
 __device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int slice) {
   return base + kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words;
 }
 
-// Describe the step `c` stands at: what it must wait for, and whether it moves data.
-// LL: an incoming message is not announced by a counter; the lane watches the flag in the last
-// 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order, so
-// this is a hint that the message is about to be complete; the threads that read it check every line.
-template <bool LL>
+// Describe the step `c` stands at: what it must wait for, whether it moves data, and from where to
+// where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
+// last 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order,
+// so this is a hint that the message is about to be complete; the threads that read it check every line.
+template <bool VEC, int EB, bool LL>
 __device__ __forceinline__ void describe_step(Context& c, const KernelParams& p, uint32_t epoch) {
-  const DevOp* op = p.ops + c.op_begin + c.step;
+  constexpr uint64_t UB = VEC ? 16 : EB;
+  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;
+  const DevOp op = p.ops[c.op_begin + c.step];
   u64* area = slice_area(p.sync_cur, p, c.slice);
   const u64* flags = area;
   const u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
   const u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
-  c.type = op->type;
-  c.hasdep = op->hasdep;
-  const bool rcv = is_recv(c.type), snd = is_send(c.type);
-  c.sseq = snd ? (u64)c.pass * (u64)c.nsend + (u64)op->send_seq : 0;
-  c.rseq = rcv ? (u64)c.pass * (u64)c.nrecv + (u64)op->recv_seq : 0;
+  const int t = op.type;
+  c.type = t;
+  c.hasdep = op.hasdep;
+  const bool rcv = is_recv(t), snd = is_send(t);
+  c.sseq = snd ? c.pass * (uint32_t)c.nsend + (uint32_t)op.send_seq : 0;
+  c.rseq = rcv ? c.pass * (uint32_t)c.nrecv + (uint32_t)op.recv_seq : 0;
   c.w0 = c.w1 = c.w2 = nullptr;
   c.t0 = c.t1 = c.t2 = 0;
-  if (op->dep_tb >= 0) { c.w0 = flags + (uint64_t)op->dep_tb * kSyncStrideWords; c.t0 = (u64)c.pass * (u64)op->dep_nops + (u64)op->dep_step + 1; }
+  if (op.dep_tb >= 0) { c.w0 = flags + (uint64_t)op.dep_tb * kSyncStrideWords; c.t0 = c.pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1; }
+  if (snd && c.sseq >= (uint32_t)p.depth) { c.w2 = tails + (uint64_t)c.send_conn * kSyncStrideWords; c.t2 = c.sseq + 1 - (uint32_t)p.depth; }
+  c.moves = !(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !op.out_staged));
+
+  const uint64_t done = (uint64_t)c.pass * p.piece_units;
+  const uint32_t n = (uint32_t)(c.slice_units - done < (uint64_t)p.piece_units ? c.slice_units - done : (uint64_t)p.piece_units);
+  const u64 off = (c.slice_begin + done) * UB;  // this piece inside any chunk, in bytes
+  // out: the slot to fill, or 0 when the receiver will read this step's payload in place
+  const u64 out = (snd && op.out_staged) ? c.out_slots + (u64)(c.sseq % (uint32_t)p.depth) * c.out_slot_units * FB : 0;
+  // in: the incoming payload -- packed in a slot, or still where the sender has it (then its rows are
+  // a chunk apart, like any rank buffer)
+  u64 in = 0;
+  int in_packed = kAPacked;
   if (rcv) {
+    if (op.in_place) { in = op.in_addr + off; in_packed = 0; }
+    else in = c.in_slots + (u64)(c.rseq % (uint32_t)p.depth) * c.in_slot_units * FB;
     if (LL) {
-      const uint64_t done = (uint64_t)c.pass * p.piece_units;
-      const uint32_t n = (uint32_t)(c.slice_units - done < (uint64_t)p.piece_units ? c.slice_units - done : (uint64_t)p.piece_units);
-      const unsigned char* slot = p.fifo + ((uint64_t)c.slice * p.slice_fifo_units + c.in_fifo_off + (c.rseq % (u64)p.depth) * c.in_slot_units) * kLLUnitBytes;
-      c.w1 = (const u64*)(slot + ((uint64_t)op->cnt * n - 1) * kLLUnitBytes + 24);
+      c.w1 = (const u64*)(in + ((uint64_t)op.cnt * n - 1) * kLLUnitBytes + 24);
       c.t1 = ll_flag(epoch, c.rseq);
     } else {
       c.w1 = heads + (uint64_t)c.recv_conn * kSyncStrideWords;
       c.t1 = c.rseq + 1;
     }
   }
-  if (snd && c.sseq >= (u64)p.depth) { c.w2 = tails + (uint64_t)c.send_conn * kSyncStrideWords; c.t2 = c.sseq + 1 - (u64)p.depth; }
-  c.moves = !(c.type == MSCCLX_OP_NOP || (c.type == MSCCLX_OP_SEND && !op->out_staged));
+  Move& m = c.m;
+  m.n = n; m.rows = op.cnt;
+  m.a = in; m.dst = op.dst_addr + off; m.out = out;
+  const int nt = op.nt_store ? kNt1 : 0;
+  int kind = 0;
+  switch (t) {
+    case MSCCLX_OP_SEND: m.a = op.src_addr + off; kind = LL ? kLLKind | kLLSend : (int)kToSlot; break;
+    case MSCCLX_OP_RECV: kind = LL ? kLLKind | (nt ? kLLRecvNt : kLLRecv) : in_packed | nt; break;
+    case MSCCLX_OP_RCS: kind = LL ? kLLKind | kLLRcs : in_packed | (out ? (int)kHasO2 : 0); break;
+    case MSCCLX_OP_RRC: kind = LL ? kLLKind | kLLRrc : in_packed | kHasB; break;
+    case MSCCLX_OP_RRS: kind = LL ? kLLKind | kLLRrs : in_packed | kHasB | kToSlot; break;
+    case MSCCLX_OP_RRCS: kind = LL ? kLLKind | kLLRrcs : in_packed | kHasB | (out ? (int)kHasO2 : 0); break;
+    case MSCCLX_OP_COPY: m.a = op.src_addr + off; kind = nt; break;
+    case MSCCLX_OP_REDUCE: m.a = op.src_addr + off; kind = kHasB; break;
+    default: break;
+  }
+  m.kind = kind;
 }
 
 // Announce the completed step and move the context to its next one.
-template <bool LL>
+template <bool VEC, int EB, bool LL>
 __device__ __forceinline__ void finish_step(Context& c, const KernelParams& p, uint32_t epoch) {
   u64* area = slice_area(p.sync_cur, p, c.slice);
   u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
   u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
-  if (!LL && is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, c.sseq + 1);  // LL: the lines announce themselves
-  if (is_recv(c.type)) publish(tails + (uint64_t)c.recv_conn * kSyncStrideWords, c.rseq + 1);
+  if (!LL && is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, (u64)c.sseq + 1);  // LL: the lines announce themselves
+  if (is_recv(c.type)) publish(tails + (uint64_t)c.recv_conn * kSyncStrideWords, (u64)c.rseq + 1);
   if (c.hasdep) publish(area + (uint64_t)c.tb * kSyncStrideWords, (u64)c.pass * (u64)c.nops + (u64)c.step + 1);
   if (++c.step == c.nops) { c.step = 0; ++c.pass; }
   if (c.pass >= c.npasses) c.active = false;
-  else describe_step<LL>(c, p, epoch);
+  else describe_step<VEC, EB, LL>(c, p, epoch);
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -449,7 +501,8 @@ __device__ __forceinline__ void finish_step(Context& c, const KernelParams& p, u
 template <class R, bool VEC, bool LL>
 __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_params) {
   static_assert(VEC || !LL, "LL lines carry 16-byte units");
-  constexpr uint64_t UB = VEC ? 16 : R::kElemBytes;
+  constexpr int EB = R::kElemBytes;
+  constexpr uint64_t UB = VEC ? 16 : EB;
   constexpr uint64_t FB = LL ? kLLUnitBytes : UB;  // bytes one unit takes inside a FIFO slot
   // The number of launches so far is kept on the device (control word 0) and is advanced by the
   // last workgroup to finish, so a launch carries no host-side state and the same launch can be
@@ -463,9 +516,11 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     p.sync_cur = p.sync_base + kSyncHeaderWords + parity * p.sync_words;
     p.sync_nxt = p.sync_base + kSyncHeaderWords + (parity ^ 1ull) * p.sync_words;
   }
-  __shared__ int sh_choice, sh_tb, sh_slice, sh_step;
-  __shared__ unsigned sh_pass;
-  const u64* const abort_word = p.sync_cur;
+  __shared__ int sh_choice;
+  __shared__ Move sh_move;
+  __shared__ uint32_t sh_seq[2];   // LL: numbers of the incoming and the outgoing message
+  __shared__ int sh_who[4];        // LL: threadblock, step, slice, pass of the chosen step, for the watchdog's report
+  u64* const abort_word = p.sync_cur;
   const int lane = threadIdx.x;
   const bool poller = threadIdx.x < 64;
   const int ctx_begin = p.wg_begin[blockIdx.x], hosted = p.wg_begin[blockIdx.x + 1] - ctx_begin;
@@ -484,19 +539,21 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     c.step = 0; c.pass = 0;
     const uint64_t u0 = p.chunk_units * (uint64_t)c.slice / p.slices, u1 = p.chunk_units * (uint64_t)(c.slice + 1) / p.slices;
     c.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
+    c.slice_begin = u0;
     c.slice_units = (uint32_t)(u1 - u0);
-    c.in_fifo_off = 0; c.in_slot_units = 0;
-    if (LL && c.recv_conn >= 0) { const DevConn cn = p.conns[c.recv_conn]; c.in_fifo_off = cn.fifo_off; c.in_slot_units = cn.slot_units; }
+    const u64 slice_fifo = (u64)p.fifo + (uint64_t)c.slice * p.slice_fifo_units * FB;
+    c.in_slots = c.out_slots = 0; c.in_slot_units = c.out_slot_units = 0;
+    if (c.recv_conn >= 0) { const DevConn cn = p.conns[c.recv_conn]; c.in_slots = slice_fifo + cn.fifo_off * FB; c.in_slot_units = cn.slot_units; }
+    if (c.send_conn >= 0) { const DevConn cn = p.conns[c.send_conn]; c.out_slots = slice_fifo + cn.fifo_off * FB; c.out_slot_units = cn.slot_units; }
     c.active = c.nops > 0 && c.npasses > 0;
     // clear, for the next launch, the counters this context is the only writer of
     u64* nxt = slice_area(p.sync_nxt, p, c.slice);
     nxt[(uint64_t)c.tb * kSyncStrideWords] = 0;
     if (c.send_conn >= 0) nxt[((uint64_t)p.ntbs + c.send_conn) * kSyncStrideWords] = 0;
     if (c.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + c.recv_conn) * kSyncStrideWords] = 0;
-    if (c.active) describe_step<LL>(c, p, epoch);
+    if (c.active) describe_step<VEC, EB, LL>(c, p, epoch);
   }
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
-  u64 deadline = wall_clock64() + p.timeout_ticks;  // pushed back whenever this workgroup makes progress
   int cursor = 0;
 #ifdef MSCCLX_PROFILE
   u64 prof_wait = 0, prof_move = 0;
@@ -510,6 +567,10 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
     if (poller) {
       int choice = -2;
       unsigned spins = 0;
+      // The watchdog period starts when this workgroup last made progress.  The clock is only read
+      // while nothing is ready, so a workgroup that keeps finding work never pays for it.
+      u64 deadline = 0;
+      bool armed = false;
       while (choice == -2) {
         bool ready = false;
         if (c.active) {
@@ -523,7 +584,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
         }
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
-          finish_step<LL>(c, p, epoch);
+          finish_step<VEC, EB, LL>(c, p, epoch);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
         }
@@ -534,18 +595,20 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
         } else if (!__any(c.active)) {
           choice = -1;  // every hosted context has run to its end
         } else if (__any(progressed)) {
-          deadline = wall_clock64() + p.timeout_ticks;
+          armed = false;
         } else {
           __builtin_amdgcn_s_sleep(1);
           if ((++spins & 0x3fu) == 0) {
+            const u64 now = wall_clock64();
+            if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
             bool stop = false;
             if (lane == 0) stop = load_counter(abort_word) != 0;
             if (__any(stop)) { choice = -3; }
-            else if (wall_clock64() > deadline) {
+            else if (now > deadline) {
               // report the first context that is still waiting
               const u64 stuck = __ballot(c.active);
               const int who = __ffsll((long long)stuck) - 1;
-              if (lane == who && atomicCAS((u64*)abort_word, 0ull, 1ull) == 0ull) {
+              if (lane == who && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
                 int what = 3;
                 if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
                 else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
@@ -560,7 +623,10 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
           }
         }
       }
-      if (choice >= 0 && lane == choice) { sh_tb = c.tb; sh_slice = c.slice; sh_step = c.step; sh_pass = c.pass; }
+      if (choice >= 0 && lane == choice) {
+        sh_move = c.m;
+        if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = c.tb; sh_who[1] = c.step; sh_who[2] = c.slice; sh_who[3] = (int)c.pass; }
+      }
       if (lane == 0) sh_choice = choice;
       cursor = choice >= 0 ? (choice + 1) & 63 : cursor;
     }
@@ -573,94 +639,43 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
 
     // ---- the chosen context's step: move one piece ----
     {
-      const int tbi = sh_tb, j = sh_slice;
-      const u64 pass = sh_pass;
-      const DevTb tb = p.tbs[tbi];
-      const DevOp op = p.ops[tb.op_begin + sh_step];
-      const int t = op.type;
-      const bool rcv = is_recv(t), snd = is_send(t);
-      const uint64_t cs = p.chunk_units;
-      const uint64_t u0 = cs * (uint64_t)j / p.slices, u1 = cs * (uint64_t)(j + 1) / p.slices;
-      const uint64_t off = u0 + pass * (uint64_t)p.piece_units;
-      const uint32_t n = (uint32_t)((u1 - off) < (uint64_t)p.piece_units ? (u1 - off) : (uint64_t)p.piece_units);
-      unsigned char* const fifo_slice = p.fifo + (uint64_t)j * p.slice_fifo_units * FB;
-      const unsigned char* lsrc = nullptr;
-      unsigned char* ldst = nullptr;
-      if (t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE)
-        lsrc = (const unsigned char*)p.bufs[op.src_slot] + ((uint64_t)op.srcoff * cs + off) * UB;
-      if (t != MSCCLX_OP_SEND)
-        ldst = (unsigned char*)p.bufs[op.dst_slot] + ((uint64_t)op.dstoff * cs + off) * UB;
-      // out: the FIFO slot to fill, or null when the receiver will read this step's payload in place
-      unsigned char* out = nullptr;
-      u64 sseq = 0, rseq = 0;
-      if (snd && op.out_staged) {
-        const DevConn cn = p.conns[tb.send_conn];
-        sseq = pass * (u64)tb.nsend + (u64)op.send_seq;
-        out = fifo_slice + (cn.fifo_off + (sseq % (u64)p.depth) * cn.slot_units) * FB;
-      }
-      // in: the incoming payload -- packed in a FIFO slot, or still where the sender has it (then
-      // its rows are a chunk apart, like any rank buffer)
-      const unsigned char* in = nullptr;
-      uint64_t in_stride = n;
-      if (rcv) {
-        if (op.in_slot >= 0) {
-          in = (const unsigned char*)p.bufs[op.in_slot] + ((uint64_t)op.in_off * cs + off) * UB;
-          in_stride = cs;
-        } else {
-          const DevConn cn = p.conns[tb.recv_conn];
-          rseq = pass * (u64)tb.nrecv + (u64)op.recv_seq;
-          in = fifo_slice + (cn.fifo_off + (rseq % (u64)p.depth) * cn.slot_units) * FB;
-        }
-      }
-      if (LL && (rcv || snd)) {
-        // every message goes through a slot, as lines
-        const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
-        const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tbi, sh_step, j, pass};
-        switch (t) {
-          case MSCCLX_OP_SEND: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, lsrc, cs, nullptr, 0, op.cnt, n, fin, fout, watch); break;
-          case MSCCLX_OP_RECV:
-            if (op.nt_store) move_rows_ll<R, true, false, true, false, true>(ldst, cs, nullptr, in, n, nullptr, 0, op.cnt, n, fin, fout, watch);
-            else             move_rows_ll<R, true, false, true, false>(ldst, cs, nullptr, in, n, nullptr, 0, op.cnt, n, fin, fout, watch);
-            break;
-          case MSCCLX_OP_RCS: move_rows_ll<R, true, false, true, true>(ldst, cs, out, in, n, nullptr, 0, op.cnt, n, fin, fout, watch); break;
-          case MSCCLX_OP_RRC: move_rows_ll<R, true, true, true, false>(ldst, cs, nullptr, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
-          case MSCCLX_OP_RRS: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
-          case MSCCLX_OP_RRCS: move_rows_ll<R, true, true, true, true>(ldst, cs, out, in, n, ldst, cs, op.cnt, n, fin, fout, watch); break;
+      const Move m = sh_move;
+      const u64 cs = p.chunk_units;
+      unsigned char* const dst = (unsigned char*)m.dst;
+      unsigned char* const out = (unsigned char*)m.out;
+      const unsigned char* const a = (const unsigned char*)m.a;
+      if (LL && (m.kind & kLLKind)) {
+        const uint32_t fin = ll_flag(epoch, sh_seq[0]), fout = ll_flag(epoch, sh_seq[1]);
+        const LLWatch watch{abort_word, p.host_status, p.timeout_ticks, sh_who[0], sh_who[1], sh_who[2], (u64)(unsigned)sh_who[3]};
+        switch (m.kind & 7) {
+          case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+          case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+          case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+          case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+          case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+          case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+          case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
           default: break;
         }
-      } else
-      switch (t) {
-        case MSCCLX_OP_SEND: move_rows<R, VEC, false, false>(out, n, nullptr, lsrc, cs, nullptr, 0, op.cnt, n); break;
-        case MSCCLX_OP_RECV:
-          if (op.nt_store) move_rows<R, VEC, false, false, true>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
-          else             move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
-          break;
-        case MSCCLX_OP_RCS:
-          if (out) move_rows<R, VEC, false, true>(ldst, cs, out, in, in_stride, nullptr, 0, op.cnt, n);
-          else     move_rows<R, VEC, false, false>(ldst, cs, nullptr, in, in_stride, nullptr, 0, op.cnt, n);
-          break;
-        case MSCCLX_OP_RRC: move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
-        case MSCCLX_OP_RRS: move_rows<R, VEC, true, false>(out, n, nullptr, in, in_stride, ldst, cs, op.cnt, n); break;
-        case MSCCLX_OP_RRCS:
-          if (out) move_rows<R, VEC, true, true>(ldst, cs, out, in, in_stride, ldst, cs, op.cnt, n);
-          else     move_rows<R, VEC, true, false>(ldst, cs, nullptr, in, in_stride, ldst, cs, op.cnt, n);
-          break;
-        case MSCCLX_OP_COPY:
-          if (op.nt_store) move_rows<R, VEC, false, false, true>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
-          else             move_rows<R, VEC, false, false>(ldst, cs, nullptr, lsrc, cs, nullptr, 0, op.cnt, n);
-          break;
-        case MSCCLX_OP_REDUCE: move_rows<R, VEC, true, false>(ldst, cs, nullptr, lsrc, cs, ldst, cs, op.cnt, n); break;
-        default: break;
+      } else {
+        const u64 stride_a = (m.kind & kAPacked) ? (u64)m.n : cs;
+        unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
+        const u64 stride_o1 = (m.kind & kToSlot) ? (u64)m.n : cs;
+        switch (m.kind & 7) {
+          case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
+          case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
+          case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n); break;
+          case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n); break;
+          case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n); break;
+          default: break;
+        }
       }
     }
     // every wave waits until its own device-scope stores are acknowledged; after the barrier the
     // polling wave may announce the whole workgroup's data with plain counter stores
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (poller) {
-      if (lane == choice) finish_step<LL>(c, p, epoch);
-      deadline = wall_clock64() + p.timeout_ticks;
-    }
+    if (poller && lane == choice) finish_step<VEC, EB, LL>(c, p, epoch);
 #ifdef MSCCLX_PROFILE
     if (threadIdx.x == 0) {
       const u64 prof_t2 = wall_clock64();
@@ -726,7 +741,6 @@ struct DeviceState {
   DevTb* tbs = nullptr;
   DevOp* ops = nullptr;
   DevConn* conns = nullptr;
-  void** bufs = nullptr;
   int32_t* hosting = nullptr;            // wg_begin | ctx_tb | ctx_slice
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
@@ -741,7 +755,6 @@ void destroy_device_state(DeviceState* d) {
   if (d->tbs) (void)hipFree(d->tbs);
   if (d->ops) (void)hipFree(d->ops);
   if (d->conns) (void)hipFree(d->conns);
-  if (d->bufs) (void)hipFree(d->bufs);
   if (d->hosting) (void)hipFree(d->hosting);
   if (d->host_status) (void)hipHostFree(d->host_status);
   if (d->ev0) (void)hipEventDestroy(d->ev0);
@@ -879,9 +892,14 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
     for (int o = tb.op_begin; o < tb.op_end; ++o) {
       const Op& op = plan->ops[o];
       DevOp& dv = hop[o];
+      dv = DevOp{};
       dv.type = op.type; dv.cnt = op.cnt;
-      dv.src_slot = tb.rank * 3 + (op.srcbuf >= 0 && op.srcbuf <= 2 ? op.srcbuf : 0); dv.srcoff = op.srcoff;
-      dv.dst_slot = tb.rank * 3 + (op.dstbuf >= 0 && op.dstbuf <= 2 ? op.dstbuf : 0); dv.dstoff = op.dstoff;
+      auto chunk_addr = [&](int buf, int off) -> uint64_t {
+        if (buf < 0 || buf > 2 || off < 0) return 0;
+        return (uint64_t)(uintptr_t)bufs[(size_t)tb.rank * 3 + buf] + (uint64_t)off * plan->chunk_bytes;
+      };
+      if (reads_local_src(op.type)) dv.src_addr = chunk_addr(op.srcbuf, op.srcoff);
+      if (touches_local_dst(op.type)) dv.dst_addr = chunk_addr(op.dstbuf, op.dstoff);
       dv.dep_tb = -1; dv.dep_step = -1; dv.dep_nops = 0;
       if (op.depid >= 0) {
         dv.dep_tb = plan->rank_tb_begin[tb.rank] + op.depid;
@@ -889,15 +907,16 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
         dv.dep_nops = plan->tbs[dv.dep_tb].op_end - plan->tbs[dv.dep_tb].op_begin;
       }
       dv.hasdep = op.hasdep; dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
-      dv.in_slot = -1; dv.in_off = -1; dv.nt_store = op.final_write;
+      dv.nt_store = op.final_write;
       dv.out_staged = is_send_type(op.type) && (g.staging || !op.zero_copy) ? 1 : 0;
       if (is_recv_type(op.type) && !g.staging) {
         const Op& sender = plan->ops[op.match_send];
         if (sender.zero_copy) {  // read the payload where the sending rank keeps it
           const int sender_rank = plan->tbs[plan->conns[tb.recv_conn].send_tb].rank;
           const bool from_src = sender.type == MSCCLX_OP_SEND;
-          dv.in_slot = sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf);
-          dv.in_off = from_src ? sender.srcoff : sender.dstoff;
+          dv.in_place = 1;
+          dv.in_addr = (uint64_t)(uintptr_t)bufs[(size_t)sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf)] +
+                       (uint64_t)(from_src ? sender.srcoff : sender.dstoff) * plan->chunk_bytes;
         }
       }
     }
@@ -905,11 +924,9 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipMalloc((void**)&d->tbs, sizeof(DevTb) * (ntb ? ntb : 1)));
   HIP_TRY(hipMalloc((void**)&d->ops, sizeof(DevOp) * (nop ? nop : 1)));
   HIP_TRY(hipMalloc((void**)&d->conns, sizeof(DevConn) * hcn.size()));
-  HIP_TRY(hipMalloc((void**)&d->bufs, sizeof(void*) * bufs.size()));
   HIP_TRY(hipMemcpy(d->tbs, htb.data(), sizeof(DevTb) * ntb, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d->ops, hop.data(), sizeof(DevOp) * nop, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d->conns, hcn.data(), sizeof(DevConn) * hcn.size(), hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(d->bufs, bufs.data(), sizeof(void*) * bufs.size(), hipMemcpyHostToDevice));
   {
     std::vector<int32_t> table(g.wg_begin);
     table.insert(table.end(), g.ctx_tb.begin(), g.ctx_tb.end());
@@ -943,7 +960,7 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
     d->dirty = false;
   }
   KernelParams kp;
-  kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns; kp.bufs = d->bufs;
+  kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns;
   unsigned long long* sync = (unsigned long long*)d->workspace;
   kp.sync_base = sync;
   kp.sync_cur = kp.sync_nxt = nullptr;

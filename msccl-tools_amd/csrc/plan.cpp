@@ -464,6 +464,12 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (piece_units > most_units) piece_units = most_units;
   g.piece_units = (uint32_t)piece_units;
   g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
+  {  // the kernel keeps step and message numbers of one launch in 32 bits
+    int64_t longest = 0;
+    for (const Tb& tb : plan.tbs) longest = std::max<int64_t>(longest, tb.op_end - tb.op_begin);
+    if (longest * g.passes >= (int64_t)1 << 31)
+      return fail(MSCCLX_ERR_CAPACITY, "piece_bytes is so small that a threadblock would make more than 2^31 steps");
+  }
   if (g.ll) {  // a message's flag carries its sequence number in 22 bits
     int64_t most = 0;
     for (const Conn& c : plan.conns) most = std::max<int64_t>(most, c.nmsg);

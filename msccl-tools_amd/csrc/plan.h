@@ -50,15 +50,18 @@ inline bool touches_local_dst(int t) { return is_recv_type(t) || t == MSCCLX_OP_
 // ---- device-side images (plain data, uploaded at bind) ----
 struct DevOp {
   int32_t type, cnt;
-  int32_t src_slot, srcoff;  // src_slot = rank*3 + buffer: index into the buffer pointer table
-  int32_t dst_slot, dstoff;
   int32_t dep_tb, dep_step;  // global threadblock row / step, or -1
   int32_t dep_nops;          // number of steps of the threadblock depended on
   int32_t hasdep;
   int32_t send_seq, recv_seq;
-  int32_t in_slot, in_off;   // recv-type: buffer-table index / chunk offset of the sender's payload, or -1: FIFO slot
   int32_t out_staged;        // send-type: 1 = copy the payload into a FIFO slot, 0 = the receiver reads it in place
   int32_t nt_store;          // 1 = the local destination is never read again: store it non-temporally
+  int32_t in_place;          // recv-type: 1 = the payload is read where the sender keeps it (in_addr), 0 = from a FIFO slot
+  int32_t pad;
+  // byte addresses of the first named chunk, resolved when buffers are bound (0 where the step has none)
+  uint64_t src_addr;         // local source of s / cpy / re
+  uint64_t dst_addr;         // local destination (and local reduction operand) of every step but s
+  uint64_t in_addr;          // in_place: the chunk of the sending rank's buffer that holds the payload
 };
 
 struct DevTb {
@@ -96,7 +99,6 @@ struct KernelParams {
   const DevTb* tbs;
   const DevOp* ops;
   const DevConn* conns;
-  void* const* bufs;            // [nranks*3]
   unsigned long long* sync_base; // control block: word 0 = launches finished so far (its parity picks the counter area), word 1 = workgroups finished
   unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
   unsigned long long* sync_nxt;  // next launch's counters   } from the control block
