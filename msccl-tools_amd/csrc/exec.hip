@@ -277,10 +277,10 @@ struct LLWatch {
   u64 pass;
 };
 
-__device__ __noinline__ void ll_give_up(const LLWatch& w) {
-  if (atomicCAS(w.abort_word, 0ull, 1ull) == 0ull) {
-    mscclx_status* hs = w.host_status;
-    hs->tb = w.tb; hs->step = w.step; hs->slice = w.slice; hs->pass = (int64_t)w.pass; hs->waiting_on = 1;
+// (arguments by value: a struct handed to a function that is not inlined would have to live in memory)
+__device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int tb, int step, int slice, u64 pass) {
+  if (atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
+    hs->tb = tb; hs->step = step; hs->slice = slice; hs->pass = (int64_t)pass; hs->waiting_on = 1;
     __threadfence_system();
     __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
@@ -303,12 +303,10 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
     u32x4 x[UA], y[UA];
     if (IN_LL) {
-      u32x4 l0[UA], l1[UA];
-#pragma unroll
-      for (int u = 0; u < UA; ++u) {
-        l0[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes));
-        l1[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
-      }
+      static_assert(UA == 2, "the retry below names its two units");
+      const uint32_t ia = i, ib = i + T;
+      u32x4 a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)), a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16));
+      u32x4 b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)), b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16));
       if (HAS_B) {
 #pragma unroll
         for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
@@ -316,25 +314,20 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
       unsigned spins = 0;
       u64 since = 0;
       for (;;) {
-        bool all = true;
-#pragma unroll
-        for (int u = 0; u < UA; ++u)
-          if (i + u * T < n && !ll_valid(l0[u], l1[u], fin)) {
-            all = false;
-            l0[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes));
-            l1[u] = A::template ld<XV>(ra, (int)((i + u * T) * kLLUnitBytes + 16));
-          }
-        if (all) break;
+        const bool ok_a = ll_valid(a0, a1, fin), ok_b = ib >= n || ll_valid(b0, b1, fin);
+        if (ok_a && ok_b) break;
+        if (!ok_a) { a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)); a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16)); }
+        if (!ok_b) { b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)); b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16)); }
         if ((++spins & 0x7fu) == 0) {
           const u64 now = wall_clock64();
           if (!since) since = now;
           const bool expired = now - since > watch.timeout_ticks;
-          if (expired) ll_give_up(watch);
+          if (expired) ll_give_up(watch.abort_word, watch.host_status, watch.tb, watch.step, watch.slice, watch.pass);
           if (expired || load_counter(watch.abort_word) != 0) break;  // the launch is lost; leave with what is there
         }
       }
-#pragma unroll
-      for (int u = 0; u < UA; ++u) x[u] = u32x4{l0[u].x, l0[u].z, l1[u].x, l1[u].z};
+      x[0] = u32x4{a0.x, a0.z, a1.x, a1.z};
+      x[1] = u32x4{b0.x, b0.z, b1.x, b1.z};
     } else {
 #pragma unroll
       for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * 16));
@@ -393,104 +386,137 @@ enum {
 };
 enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
 
-// One hosted context = (threadblock, slice): the state of one lane of wave 0.
-struct Context {
-  int tb, slice, step, nops, op_begin, send_conn, recv_conn, nsend, nrecv;
-  unsigned pass, npasses;
-  bool active;
-  u64 slice_begin;               // first unit of a chunk this slice covers ...
-  uint32_t slice_units;          // ... and how many
-  u64 in_slots, out_slots;       // byte address of the first slot of the incoming / outgoing connection, in this slice
-  uint32_t in_slot_units, out_slot_units;
-  // the step the context stands at
-  bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
-  int type, hasdep;
-  uint32_t sseq, rseq;      // number of the message this step sends / receives on its connection (all passes)
-  const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
-  uint32_t t0, t1, t2;      // ... until they reach these values (every counter of a launch stays below 2^32)
-  Move m;
+// One hosted context = (threadblock, slice), run by one lane of wave 0.  What never changes while it
+// runs sits in LDS (one entry per lane, touched by that lane only), so that it occupies no registers
+// while the workgroup moves data; what changes from step to step is the lane's Context.
+struct Hosted {
+  int nops, op_begin;
+  unsigned npasses;
+  // Slots: offsets from the start of the FIFO region, in 16-byte steps on the vector path and in bytes otherwise; counters: 64-bit word index
+  // inside this launch's counter area.  32 bits each, so that the lot is read from LDS in one go.
+  uint32_t in_slots, out_slots;    // first slot of the incoming / outgoing connection, in this slice
+  uint32_t in_slot_bytes, out_slot_bytes;
+  uint32_t in_wrap, out_wrap;      // depth * slot bytes: where the ring of slots starts over
+  uint32_t flags;                  // flag of threadblock t of this slice is flags + t * kSyncStrideWords
+  uint32_t my_flag;
+  uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
+  uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
+  int tb, slice;                   // for the watchdog's report only
 };
 
 __device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int slice) {
   return base + kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words;
 }
 
+// The changing part.  Everything that depends on the pass or on how many messages went by is kept
+// as a running value, advanced when a step finishes: the lane's instructions between two moves are
+// on the critical path of a latency-bound program, and multiplications and divisions dominate them.
+struct Context {
+  int step;
+  unsigned pass;
+  bool active;
+  uint32_t count;           // steps finished so far in this launch (all passes)
+  uint32_t sseq, rseq;      // messages sent / received so far = number of the next message on its connection
+  uint32_t sslot, rslot;    // byte offset of that message's slot inside the connection's ring
+  uint32_t left;            // units of the slice not yet covered before this pass
+  u64 off;                  // byte offset of this pass's piece inside any chunk
+  // the step the context stands at
+  bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
+  int type, hasdep;
+  const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
+  uint32_t t0, t1, t2;      // ... until they reach these values (every counter of a launch stays below 2^32)
+  Move m;
+};
+
 // Describe the step `c` stands at: what it must wait for, whether it moves data, and from where to
 // where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
 // last 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order,
 // so this is a hint that the message is about to be complete; the threads that read it check every line.
-template <bool VEC, int EB, bool LL>
-__device__ __forceinline__ void describe_step(Context& c, const KernelParams& p, uint32_t epoch) {
-  constexpr uint64_t UB = VEC ? 16 : EB;
-  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;
-  const DevOp op = p.ops[c.op_begin + c.step];
-  u64* area = slice_area(p.sync_cur, p, c.slice);
-  const u64* flags = area;
-  const u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
-  const u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
-  const int t = op.type;
+template <bool VEC, bool LL>
+__device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const KernelParams& p, uint32_t epoch, const DevOp& op) {
+  const int t = (int)(op.word & 15u);
+  const int cnt = (int)(op.word >> kOpCntShift);
+  const bool out_staged = op.word & kOpOutStaged, in_place = op.word & kOpInPlace;
   c.type = t;
-  c.hasdep = op.hasdep;
+  c.hasdep = (op.word & kOpHasdep) ? 1 : 0;
   const bool rcv = is_recv(t), snd = is_send(t);
-  c.sseq = snd ? c.pass * (uint32_t)c.nsend + (uint32_t)op.send_seq : 0;
-  c.rseq = rcv ? c.pass * (uint32_t)c.nrecv + (uint32_t)op.recv_seq : 0;
   c.w0 = c.w1 = c.w2 = nullptr;
   c.t0 = c.t1 = c.t2 = 0;
-  if (op.dep_tb >= 0) { c.w0 = flags + (uint64_t)op.dep_tb * kSyncStrideWords; c.t0 = c.pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1; }
-  if (snd && c.sseq >= (uint32_t)p.depth) { c.w2 = tails + (uint64_t)c.send_conn * kSyncStrideWords; c.t2 = c.sseq + 1 - (uint32_t)p.depth; }
-  c.moves = !(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !op.out_staged));
+  if (op.dep_tb >= 0) { c.w0 = p.sync_cur + (h.flags + (uint32_t)op.dep_tb * kSyncStrideWords); c.t0 = c.pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1; }
+  if (snd && c.sseq >= (uint32_t)p.depth) { c.w2 = p.sync_cur + h.tail_in; c.t2 = c.sseq + 1 - (uint32_t)p.depth; }
+  c.moves = !(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !out_staged));
 
-  const uint64_t done = (uint64_t)c.pass * p.piece_units;
-  const uint32_t n = (uint32_t)(c.slice_units - done < (uint64_t)p.piece_units ? c.slice_units - done : (uint64_t)p.piece_units);
-  const u64 off = (c.slice_begin + done) * UB;  // this piece inside any chunk, in bytes
+  const uint32_t n = c.left < p.piece_units ? c.left : p.piece_units;
   // out: the slot to fill, or 0 when the receiver will read this step's payload in place
-  const u64 out = (snd && op.out_staged) ? c.out_slots + (u64)(c.sseq % (uint32_t)p.depth) * c.out_slot_units * FB : 0;
+  const u64 out = (snd && out_staged) ? (u64)p.fifo + (u64)h.out_slots * (VEC ? 16 : 1) + c.sslot : 0;
   // in: the incoming payload -- packed in a slot, or still where the sender has it (then its rows are
   // a chunk apart, like any rank buffer)
   u64 in = 0;
   int in_packed = kAPacked;
   if (rcv) {
-    if (op.in_place) { in = op.in_addr + off; in_packed = 0; }
-    else in = c.in_slots + (u64)(c.rseq % (uint32_t)p.depth) * c.in_slot_units * FB;
+    if (in_place) { in = op.in_addr + c.off; in_packed = 0; }
+    else in = (u64)p.fifo + (u64)h.in_slots * (VEC ? 16 : 1) + c.rslot;
     if (LL) {
-      c.w1 = (const u64*)(in + ((uint64_t)op.cnt * n - 1) * kLLUnitBytes + 24);
+      c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
       c.t1 = ll_flag(epoch, c.rseq);
     } else {
-      c.w1 = heads + (uint64_t)c.recv_conn * kSyncStrideWords;
+      c.w1 = p.sync_cur + h.head_in;
       c.t1 = c.rseq + 1;
     }
   }
   Move& m = c.m;
-  m.n = n; m.rows = op.cnt;
-  m.a = in; m.dst = op.dst_addr + off; m.out = out;
-  const int nt = op.nt_store ? kNt1 : 0;
+  m.n = n; m.rows = cnt;
+  m.a = in; m.dst = op.dst_addr + c.off; m.out = out;
+  const int nt = (op.word & kOpNtStore) ? kNt1 : 0;
   int kind = 0;
   switch (t) {
-    case MSCCLX_OP_SEND: m.a = op.src_addr + off; kind = LL ? kLLKind | kLLSend : (int)kToSlot; break;
+    case MSCCLX_OP_SEND: m.a = op.src_addr + c.off; kind = LL ? kLLKind | kLLSend : (int)kToSlot; break;
     case MSCCLX_OP_RECV: kind = LL ? kLLKind | (nt ? kLLRecvNt : kLLRecv) : in_packed | nt; break;
     case MSCCLX_OP_RCS: kind = LL ? kLLKind | kLLRcs : in_packed | (out ? (int)kHasO2 : 0); break;
     case MSCCLX_OP_RRC: kind = LL ? kLLKind | kLLRrc : in_packed | kHasB; break;
     case MSCCLX_OP_RRS: kind = LL ? kLLKind | kLLRrs : in_packed | kHasB | kToSlot; break;
     case MSCCLX_OP_RRCS: kind = LL ? kLLKind | kLLRrcs : in_packed | kHasB | (out ? (int)kHasO2 : 0); break;
-    case MSCCLX_OP_COPY: m.a = op.src_addr + off; kind = nt; break;
-    case MSCCLX_OP_REDUCE: m.a = op.src_addr + off; kind = kHasB; break;
+    case MSCCLX_OP_COPY: m.a = op.src_addr + c.off; kind = nt; break;
+    case MSCCLX_OP_REDUCE: m.a = op.src_addr + c.off; kind = kHasB; break;
     default: break;
   }
   m.kind = kind;
 }
 
-// Announce the completed step and move the context to its next one.
-template <bool VEC, int EB, bool LL>
-__device__ __forceinline__ void finish_step(Context& c, const KernelParams& p, uint32_t epoch) {
-  u64* area = slice_area(p.sync_cur, p, c.slice);
-  u64* heads = area + (uint64_t)p.ntbs * kSyncStrideWords;
-  u64* tails = heads + (uint64_t)p.nconns * kSyncStrideWords;
-  if (!LL && is_send(c.type)) publish(heads + (uint64_t)c.send_conn * kSyncStrideWords, (u64)c.sseq + 1);  // LL: the lines announce themselves
-  if (is_recv(c.type)) publish(tails + (uint64_t)c.recv_conn * kSyncStrideWords, (u64)c.rseq + 1);
-  if (c.hasdep) publish(area + (uint64_t)c.tb * kSyncStrideWords, (u64)c.pass * (u64)c.nops + (u64)c.step + 1);
-  if (++c.step == c.nops) { c.step = 0; ++c.pass; }
-  if (c.pass >= c.npasses) c.active = false;
-  else describe_step<VEC, EB, LL>(c, p, epoch);
+// The description of the step after the one `c` stands at.  It is fetched before the counters of
+// the finished step are stored: a load issued after those stores would come back only after they
+// are acknowledged, and the context could not look for its next message any earlier.
+__device__ __forceinline__ DevOp fetch_next_op(const Context& c, const Hosted& h, const KernelParams& p) {
+  const int next = c.step + 1 == h.nops ? 0 : c.step + 1;
+  return p.ops[h.op_begin + next];
+}
+
+// Announce the completed step and move the context to its next one, described by `next`.
+template <int UB, bool LL>
+__device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next) {
+  const Hosted h = entry;  // one batch of LDS reads, one wait -- not one wait per field as they are needed
+  if (is_send(c.type)) {
+    if (!LL) publish(p.sync_cur + h.head_out, (u64)c.sseq + 1);  // LL: the lines announce themselves
+    ++c.sseq;
+    c.sslot += h.out_slot_bytes;
+    if (c.sslot == h.out_wrap) c.sslot = 0;
+  }
+  if (is_recv(c.type)) {
+    publish(p.sync_cur + h.tail_out, (u64)c.rseq + 1);
+    ++c.rseq;
+    c.rslot += h.in_slot_bytes;
+    if (c.rslot == h.in_wrap) c.rslot = 0;
+  }
+  ++c.count;
+  if (c.hasdep) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * nops + step + 1
+  if (++c.step == h.nops) {
+    c.step = 0;
+    ++c.pass;
+    c.left -= c.left < p.piece_units ? c.left : p.piece_units;
+    c.off += (u64)p.piece_units * UB;
+  }
+  if (c.pass >= h.npasses) c.active = false;
+  else describe_step<UB == 16, LL>(c, h, p, epoch, next);
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -499,7 +525,7 @@ __device__ __forceinline__ void finish_step(Context& c, const KernelParams& p, u
 // reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
 // share the resident workgroups without deadlock.
 template <class R, bool VEC, bool LL>
-__global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_params) {
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
   static_assert(VEC || !LL, "LL lines carry 16-byte units");
   constexpr int EB = R::kElemBytes;
   constexpr uint64_t UB = VEC ? 16 : EB;
@@ -528,35 +554,49 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
   // watch for it; the moving threads go straight to the lines and retry them until they are there.
   const bool direct = LL && hosted == 1;
 
+  __shared__ Hosted sh_hosted[kMaxHosted];
+  Hosted& h = sh_hosted[lane & (kMaxHosted - 1)];  // this lane's entry; lanes of other waves never look at it
   Context c;
   c.active = false;
   if (poller && lane < hosted) {
-    c.tb = p.ctx_tb[ctx_begin + lane];
-    c.slice = p.ctx_slice[ctx_begin + lane];
-    const DevTb tb = p.tbs[c.tb];
-    c.nops = tb.nops; c.op_begin = tb.op_begin; c.send_conn = tb.send_conn; c.recv_conn = tb.recv_conn;
-    c.nsend = tb.nsend; c.nrecv = tb.nrecv;
-    c.step = 0; c.pass = 0;
-    const uint64_t u0 = p.chunk_units * (uint64_t)c.slice / p.slices, u1 = p.chunk_units * (uint64_t)(c.slice + 1) / p.slices;
-    c.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
-    c.slice_begin = u0;
-    c.slice_units = (uint32_t)(u1 - u0);
-    const u64 slice_fifo = (u64)p.fifo + (uint64_t)c.slice * p.slice_fifo_units * FB;
-    c.in_slots = c.out_slots = 0; c.in_slot_units = c.out_slot_units = 0;
-    if (c.recv_conn >= 0) { const DevConn cn = p.conns[c.recv_conn]; c.in_slots = slice_fifo + cn.fifo_off * FB; c.in_slot_units = cn.slot_units; }
-    if (c.send_conn >= 0) { const DevConn cn = p.conns[c.send_conn]; c.out_slots = slice_fifo + cn.fifo_off * FB; c.out_slot_units = cn.slot_units; }
-    c.active = c.nops > 0 && c.npasses > 0;
+    h.tb = p.ctx_tb[ctx_begin + lane];
+    h.slice = p.ctx_slice[ctx_begin + lane];
+    const DevTb tb = p.tbs[h.tb];
+    h.nops = tb.nops; h.op_begin = tb.op_begin;
+    const uint64_t u0 = p.chunk_units * (uint64_t)h.slice / p.slices, u1 = p.chunk_units * (uint64_t)(h.slice + 1) / p.slices;
+    h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
+    const uint64_t slice_fifo = (uint64_t)h.slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16)
+    const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)h.slice * p.sync_slice_words);
+    const uint32_t heads = area + (uint32_t)p.ntbs * kSyncStrideWords, tails = heads + (uint32_t)p.nconns * kSyncStrideWords;
+    h.flags = area;
+    h.my_flag = area + (uint32_t)h.tb * kSyncStrideWords;
+    h.in_slots = h.out_slots = 0; h.in_slot_bytes = h.out_slot_bytes = 0; h.in_wrap = h.out_wrap = 0;
+    h.head_in = h.tail_out = h.head_out = h.tail_in = 0;
+    if (tb.recv_conn >= 0) {
+      const DevConn cn = p.conns[tb.recv_conn];
+      h.in_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.in_slot_bytes = (uint32_t)(cn.slot_units * FB); h.in_wrap = h.in_slot_bytes * (uint32_t)p.depth;
+      h.head_in = heads + (uint32_t)tb.recv_conn * kSyncStrideWords; h.tail_out = tails + (uint32_t)tb.recv_conn * kSyncStrideWords;
+    }
+    if (tb.send_conn >= 0) {
+      const DevConn cn = p.conns[tb.send_conn];
+      h.out_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.out_slot_bytes = (uint32_t)(cn.slot_units * FB); h.out_wrap = h.out_slot_bytes * (uint32_t)p.depth;
+      h.head_out = heads + (uint32_t)tb.send_conn * kSyncStrideWords; h.tail_in = tails + (uint32_t)tb.send_conn * kSyncStrideWords;
+    }
+    c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
+    c.left = (uint32_t)(u1 - u0);
+    c.off = u0 * UB;
+    c.active = tb.nops > 0 && h.npasses > 0;
     // clear, for the next launch, the counters this context is the only writer of
-    u64* nxt = slice_area(p.sync_nxt, p, c.slice);
-    nxt[(uint64_t)c.tb * kSyncStrideWords] = 0;
-    if (c.send_conn >= 0) nxt[((uint64_t)p.ntbs + c.send_conn) * kSyncStrideWords] = 0;
-    if (c.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + c.recv_conn) * kSyncStrideWords] = 0;
-    if (c.active) describe_step<VEC, EB, LL>(c, p, epoch);
+    u64* nxt = slice_area(p.sync_nxt, p, h.slice);
+    nxt[(uint64_t)h.tb * kSyncStrideWords] = 0;
+    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
+    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
+    if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[tb.op_begin]);
   }
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
   int cursor = 0;
 #ifdef MSCCLX_PROFILE
-  u64 prof_wait = 0, prof_move = 0;
+  u64 prof_wait = 0, prof_move = 0, prof_ack = 0, prof_fin = 0;
   const u64 prof_start = wall_clock64();
 #endif
 
@@ -584,7 +624,8 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
         }
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
-          finish_step<VEC, EB, LL>(c, p, epoch);
+          const DevOp next = fetch_next_op(c, h, p);
+          finish_step<(int)UB, LL>(c, h, p, epoch, next);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
         }
@@ -614,7 +655,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
                 else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
                 else if (c.w2 && load_counter(c.w2) < c.t2) what = 2;
                 mscclx_status* hs = p.host_status;
-                hs->tb = c.tb; hs->step = c.step; hs->slice = c.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
+                hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
                 __threadfence_system();
                 __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
               }
@@ -625,7 +666,7 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
       }
       if (choice >= 0 && lane == choice) {
         sh_move = c.m;
-        if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = c.tb; sh_who[1] = c.step; sh_who[2] = c.slice; sh_who[3] = (int)c.pass; }
+        if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = h.tb; sh_who[1] = c.step; sh_who[2] = h.slice; sh_who[3] = (int)c.pass; }
       }
       if (lane == 0) sh_choice = choice;
       cursor = choice >= 0 ? (choice + 1) & 63 : cursor;
@@ -671,16 +712,28 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
         }
       }
     }
-    // every wave waits until its own device-scope stores are acknowledged; after the barrier the
-    // polling wave may announce the whole workgroup's data with plain counter stores
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t2 = wall_clock64();
+#endif
+    // every wave waits until its own device-scope stores are acknowledged (the context's lane asks
+    // for its next step's description meanwhile); after the barrier that lane may announce the whole
+    // workgroup's data with plain counter stores
+    const bool mine = poller && lane == choice;
+    DevOp next;
+    if (mine) next = fetch_next_op(c, h, p);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (poller && lane == choice) finish_step<VEC, EB, LL>(c, p, epoch);
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t3 = wall_clock64();
+#endif
+    if (mine) finish_step<(int)UB, LL>(c, h, p, epoch, next);
 #ifdef MSCCLX_PROFILE
     if (threadIdx.x == 0) {
-      const u64 prof_t2 = wall_clock64();
+      const u64 prof_t4 = wall_clock64();
       prof_wait += prof_t1 - prof_t0;
       prof_move += prof_t2 - prof_t1;
+      prof_ack += prof_t3 - prof_t2;
+      prof_fin += prof_t4 - prof_t3;
     }
 #endif
   }
@@ -694,10 +747,12 @@ __global__ void __launch_bounds__(512) exec_kernel(const KernelParams launch_par
   }
 #ifdef MSCCLX_PROFILE
   if (threadIdx.x == 0 && p.prof) {
-    p.prof[(size_t)blockIdx.x * 4 + 0] = prof_wait;
-    p.prof[(size_t)blockIdx.x * 4 + 1] = prof_move;
-    p.prof[(size_t)blockIdx.x * 4 + 2] = wall_clock64() - prof_start;
-    p.prof[(size_t)blockIdx.x * 4 + 3] = prof_start;
+    p.prof[(size_t)blockIdx.x * 8 + 0] = prof_wait;
+    p.prof[(size_t)blockIdx.x * 8 + 1] = prof_move;
+    p.prof[(size_t)blockIdx.x * 8 + 2] = wall_clock64() - prof_start;
+    p.prof[(size_t)blockIdx.x * 8 + 3] = prof_start;
+    p.prof[(size_t)blockIdx.x * 8 + 4] = prof_ack;
+    p.prof[(size_t)blockIdx.x * 8 + 5] = prof_fin;
   }
 #endif
 }
@@ -747,7 +802,7 @@ struct DeviceState {
   kernel_fn kernel = nullptr;
   bool dirty = false;  // counters must be cleared before the next launch (after a failed launch)
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: 4 words per workgroup
+  unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: 8 words per workgroup
 };
 
 void destroy_device_state(DeviceState* d) {
@@ -893,7 +948,6 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
       const Op& op = plan->ops[o];
       DevOp& dv = hop[o];
       dv = DevOp{};
-      dv.type = op.type; dv.cnt = op.cnt;
       auto chunk_addr = [&](int buf, int off) -> uint64_t {
         if (buf < 0 || buf > 2 || off < 0) return 0;
         return (uint64_t)(uintptr_t)bufs[(size_t)tb.rank * 3 + buf] + (uint64_t)off * plan->chunk_bytes;
@@ -906,15 +960,17 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
         dv.dep_step = op.deps;
         dv.dep_nops = plan->tbs[dv.dep_tb].op_end - plan->tbs[dv.dep_tb].op_begin;
       }
-      dv.hasdep = op.hasdep; dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
-      dv.nt_store = op.final_write;
-      dv.out_staged = is_send_type(op.type) && (g.staging || !op.zero_copy) ? 1 : 0;
+      dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
+      dv.word = (uint32_t)op.type | ((uint32_t)std::max(op.cnt, 0) << kOpCntShift);
+      if (op.hasdep) dv.word |= kOpHasdep;
+      if (op.final_write) dv.word |= kOpNtStore;
+      if (is_send_type(op.type) && (g.staging || !op.zero_copy)) dv.word |= kOpOutStaged;
       if (is_recv_type(op.type) && !g.staging) {
         const Op& sender = plan->ops[op.match_send];
         if (sender.zero_copy) {  // read the payload where the sending rank keeps it
           const int sender_rank = plan->tbs[plan->conns[tb.recv_conn].send_tb].rank;
           const bool from_src = sender.type == MSCCLX_OP_SEND;
-          dv.in_place = 1;
+          dv.word |= kOpInPlace;
           dv.in_addr = (uint64_t)(uintptr_t)bufs[(size_t)sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf)] +
                        (uint64_t)(from_src ? sender.srcoff : sender.dstoff) * plan->chunk_bytes;
         }
@@ -943,7 +999,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipEventCreate(&d->ev0));
   HIP_TRY(hipEventCreate(&d->ev1));
 #ifdef MSCCLX_PROFILE
-  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * 4 * g.workgroups));
+  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * 8 * g.workgroups));
 #endif
   return MSCCLX_OK;
 }
@@ -996,18 +1052,16 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
 #ifdef MSCCLX_PROFILE
   if (d->prof && getenv("MSCCLX_PROFILE_DUMP")) {
     const size_t nwg = plan->geo.workgroups;
-    std::vector<unsigned long long> h(nwg * 4);
+    std::vector<unsigned long long> h(nwg * 8);
     (void)hipMemcpy(h.data(), d->prof, h.size() * 8, hipMemcpyDeviceToHost);
-    double sw = 0, sm = 0, st_ = 0; unsigned long long first = ~0ull, last = 0; size_t worst = 0;
+    double sw = 0, sm = 0, sa = 0, sf = 0, st_ = 0; unsigned long long first = ~0ull, last = 0;
     for (size_t w = 0; w < nwg; ++w) {
-      sw += h[w * 4]; sm += h[w * 4 + 1]; st_ += h[w * 4 + 2];
-      if (h[w * 4 + 3] < first) first = h[w * 4 + 3];
-      if (h[w * 4 + 3] + h[w * 4 + 2] > last) last = h[w * 4 + 3] + h[w * 4 + 2];
-      if (h[w * 4 + 1] > h[worst * 4 + 1]) worst = w;
+      sw += h[w * 8]; sm += h[w * 8 + 1]; st_ += h[w * 8 + 2]; sa += h[w * 8 + 4]; sf += h[w * 8 + 5];
+      if (h[w * 8 + 3] < first) first = h[w * 8 + 3];
+      if (h[w * 8 + 3] + h[w * 8 + 2] > last) last = h[w * 8 + 3] + h[w * 8 + 2];
     }
-    fprintf(stderr, "[prof] wgs=%zu span=%.1f us  mean per wg: wait %.1f us move %.1f us total %.1f us | busiest wg %zu (tb %zu): wait %.1f move %.1f total %.1f us\n",
-            nwg, (last - first) / 100.0, sw / nwg / 100, sm / nwg / 100, st_ / nwg / 100, worst, (size_t)0,
-            h[worst * 4] / 100.0, h[worst * 4 + 1] / 100.0, h[worst * 4 + 2] / 100.0);
+    fprintf(stderr, "[prof] wgs=%zu span=%.1f us  mean per wg: poll %.1f us  move %.1f us  ack+barrier %.1f us  finish+describe %.1f us  total %.1f us\n",
+            nwg, (last - first) / 100.0, sw / nwg / 100, sm / nwg / 100, sa / nwg / 100, sf / nwg / 100, st_ / nwg / 100);
   }
 #endif
   if (st.code != MSCCLX_OK) {

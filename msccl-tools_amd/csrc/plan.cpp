@@ -250,6 +250,7 @@ static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
       const std::string at = where(*p, t, o - tb.op_begin);
       if (op.type < MSCCLX_OP_NOP || op.type > MSCCLX_OP_REDUCE) return fail(MSCCLX_ERR_BAD_IR, at + ": unknown step type " + std::to_string(op.type));
       if (op.type != MSCCLX_OP_NOP && op.cnt < 1) return fail(MSCCLX_ERR_BAD_IR, at + ": cnt must be >= 1");
+      if (op.cnt >= (1 << 24)) return fail(MSCCLX_ERR_BAD_IR, at + ": cnt must be below 2^24");
       auto check_ref = [&](int buf, int off, const char* what) -> int {
         if (buf < 0 || buf > 2) return fail(MSCCLX_ERR_BAD_IR, at + ": bad " + what + " buffer");
         const int extent = p->rank_chunks[(size_t)tb.rank * 3 + buf];
@@ -464,6 +465,11 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (piece_units > most_units) piece_units = most_units;
   g.piece_units = (uint32_t)piece_units;
   g.passes = (int)((longest_slice + piece_units - 1) / piece_units);
+  for (const Conn& c : plan.conns) {  // the kernel addresses a connection's ring of slots with 32-bit byte offsets
+    const uint64_t ring = (uint64_t)depth * (uint64_t)(g.staging ? c.max_cnt : c.max_staged_cnt) * piece_units * fifo_unit_bytes;
+    if (ring >= (1ull << 32))
+      return fail(MSCCLX_ERR_CAPACITY, "the slots of one connection would take 4 GiB or more; use a smaller piece_bytes or fifo_depth");
+  }
   {  // the kernel keeps step and message numbers of one launch in 32 bits
     int64_t longest = 0;
     for (const Tb& tb : plan.tbs) longest = std::max<int64_t>(longest, tb.op_end - tb.op_begin);
@@ -550,6 +556,11 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
   const uint64_t sync_bytes = ((kSyncHeaderWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
   g.fifo_byte_off = sync_bytes;
+  {  // the kernel keeps slot positions as 32-bit offsets (16-byte steps on the vector path, bytes otherwise) and counter positions as 32-bit word indices
+    const uint64_t fifo_bytes = g.slice_fifo_units * g.slices * fifo_unit_bytes;
+    if (fifo_bytes >= (g.vector_path ? (1ull << 36) : (1ull << 32)) || g.sync_words >= (1ull << 31))
+      return fail(MSCCLX_ERR_CAPACITY, "the FIFO slots or counters of this geometry exceed what the kernel can address; use fewer slices or a smaller piece_bytes");
+  }
   g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * fifo_unit_bytes + 256;
   *out = std::move(g);
   return MSCCLX_OK;

@@ -49,20 +49,21 @@ inline bool touches_local_dst(int t) { return is_recv_type(t) || t == MSCCLX_OP_
 
 // ---- device-side images (plain data, uploaded at bind) ----
 struct DevOp {
-  int32_t type, cnt;
+  // bits 0-3 type, 4 hasdep, 5 out_staged (send-type: 1 = copy the payload into a FIFO slot, 0 = the
+  // receiver reads it in place), 6 nt_store (the local destination is never read again: store it
+  // non-temporally), 7 in_place (recv-type: the payload is read where the sender keeps it), 8-31 cnt
+  uint32_t word;
   int32_t dep_tb, dep_step;  // global threadblock row / step, or -1
   int32_t dep_nops;          // number of steps of the threadblock depended on
-  int32_t hasdep;
   int32_t send_seq, recv_seq;
-  int32_t out_staged;        // send-type: 1 = copy the payload into a FIFO slot, 0 = the receiver reads it in place
-  int32_t nt_store;          // 1 = the local destination is never read again: store it non-temporally
-  int32_t in_place;          // recv-type: 1 = the payload is read where the sender keeps it (in_addr), 0 = from a FIFO slot
-  int32_t pad;
   // byte addresses of the first named chunk, resolved when buffers are bound (0 where the step has none)
   uint64_t src_addr;         // local source of s / cpy / re
   uint64_t dst_addr;         // local destination (and local reduction operand) of every step but s
   uint64_t in_addr;          // in_place: the chunk of the sending rank's buffer that holds the payload
 };
+static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
+constexpr uint32_t kOpHasdep = 1u << 4, kOpOutStaged = 1u << 5, kOpNtStore = 1u << 6, kOpInPlace = 1u << 7;
+constexpr int kOpCntShift = 8;
 
 struct DevTb {
   int32_t op_begin, nops;
