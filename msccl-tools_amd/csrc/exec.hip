@@ -256,6 +256,10 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
 __device__ __forceinline__ u64 load_counter(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+__device__ __forceinline__ u64 first_lane(u64 v) {  // the first lane's value, as a value the compiler knows to be the same in all lanes
+  return ((u64)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) | (u64)__builtin_amdgcn_readfirstlane((uint32_t)v);
+}
+
 __device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
 __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
 
@@ -492,23 +496,25 @@ __device__ __forceinline__ DevOp fetch_next_op(const Context& c, const Hosted& h
 }
 
 // Announce the completed step and move the context to its next one, described by `next`.
+// `writer`: this thread stores the counters (the context's lane; one thread of a wave that runs a
+// context with all its lanes).
 template <int UB, bool LL>
-__device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next) {
+__device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next, bool writer = true) {
   const Hosted h = entry;  // one batch of LDS reads, one wait -- not one wait per field as they are needed
   if (is_send(c.type)) {
-    if (!LL) publish(p.sync_cur + h.head_out, (u64)c.sseq + 1);  // LL: the lines announce themselves
+    if (!LL && writer) publish(p.sync_cur + h.head_out, (u64)c.sseq + 1);  // LL: the lines announce themselves
     ++c.sseq;
     c.sslot += h.out_slot_bytes;
     if (c.sslot == h.out_wrap) c.sslot = 0;
   }
   if (is_recv(c.type)) {
-    publish(p.sync_cur + h.tail_out, (u64)c.rseq + 1);
+    if (writer) publish(p.sync_cur + h.tail_out, (u64)c.rseq + 1);
     ++c.rseq;
     c.rslot += h.in_slot_bytes;
     if (c.rslot == h.in_wrap) c.rslot = 0;
   }
   ++c.count;
-  if (c.hasdep) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * nops + step + 1
+  if (c.hasdep && writer) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * nops + step + 1
   if (++c.step == h.nops) {
     c.step = 0;
     ++c.pass;
@@ -517,6 +523,160 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
   }
   if (c.pass >= h.npasses) c.active = false;
   else describe_step<UB == 16, LL>(c, h, p, epoch, next);
+}
+
+// Set up the context (threadblock tbi, slice) : its constants in `h`, its state in `c`, standing at
+// its first step.  `writer` also clears, for the next launch, the counters this context alone writes.
+template <bool VEC, int EB, bool LL>
+__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int tbi, int slice, bool writer) {
+  constexpr uint64_t UB = VEC ? 16 : EB;
+  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;
+  h.tb = tbi;
+  h.slice = slice;
+  const DevTb tb = p.tbs[tbi];
+  h.nops = tb.nops; h.op_begin = tb.op_begin;
+  const uint64_t u0 = p.chunk_units * (uint64_t)slice / p.slices, u1 = p.chunk_units * (uint64_t)(slice + 1) / p.slices;
+  h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
+  const uint64_t slice_fifo = (uint64_t)slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
+  const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words);
+  const uint32_t heads = area + (uint32_t)p.ntbs * kSyncStrideWords, tails = heads + (uint32_t)p.nconns * kSyncStrideWords;
+  h.flags = area;
+  h.my_flag = area + (uint32_t)tbi * kSyncStrideWords;
+  h.in_slots = h.out_slots = 0; h.in_slot_bytes = h.out_slot_bytes = 0; h.in_wrap = h.out_wrap = 0;
+  h.head_in = h.tail_out = h.head_out = h.tail_in = 0;
+  if (tb.recv_conn >= 0) {
+    const DevConn cn = p.conns[tb.recv_conn];
+    h.in_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.in_slot_bytes = (uint32_t)(cn.slot_units * FB); h.in_wrap = h.in_slot_bytes * (uint32_t)p.depth;
+    h.head_in = heads + (uint32_t)tb.recv_conn * kSyncStrideWords; h.tail_out = tails + (uint32_t)tb.recv_conn * kSyncStrideWords;
+  }
+  if (tb.send_conn >= 0) {
+    const DevConn cn = p.conns[tb.send_conn];
+    h.out_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.out_slot_bytes = (uint32_t)(cn.slot_units * FB); h.out_wrap = h.out_slot_bytes * (uint32_t)p.depth;
+    h.head_out = heads + (uint32_t)tb.send_conn * kSyncStrideWords; h.tail_in = tails + (uint32_t)tb.send_conn * kSyncStrideWords;
+  }
+  c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
+  c.left = (uint32_t)(u1 - u0);
+  c.off = u0 * UB;
+  c.active = tb.nops > 0 && h.npasses > 0;
+  if (writer) {
+    u64* nxt = slice_area(p.sync_nxt, p, slice);
+    nxt[(uint64_t)tbi * kSyncStrideWords] = 0;
+    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
+    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
+  }
+  if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[tb.op_begin]);
+}
+
+// The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
+// incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
+template <class R, bool VEC, bool LL>
+__device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
+                                        int tb, int step, int slice, unsigned pass) {
+  const u64 cs = p.chunk_units;
+  unsigned char* const dst = (unsigned char*)m.dst;
+  unsigned char* const out = (unsigned char*)m.out;
+  const unsigned char* const a = (const unsigned char*)m.a;
+  if (LL && (m.kind & kLLKind)) {
+    const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
+    const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tb, step, slice, (u64)pass};
+    switch (m.kind & 7) {
+      case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+      case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+      case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+      case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
+      case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+      case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+      case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+      default: break;
+    }
+  } else {
+    const u64 stride_a = (m.kind & kAPacked) ? (u64)m.n : cs;
+    unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
+    const u64 stride_o1 = (m.kind & kToSlot) ? (u64)m.n : cs;
+    switch (m.kind & 7) {
+      case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
+      case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
+      case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n); break;
+      case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n); break;
+      case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n); break;
+      default: break;
+    }
+  }
+}
+
+// LL, one context on a workgroup of one wave: the wave runs the context with all its lanes.  Every
+// value of the bookkeeping is then the same in all lanes, so it lives in scalar registers and runs
+// on the scalar unit; there is no hand-over through LDS and no barrier, and the lanes go straight
+// from one message's lines to the next one's.  This is the shape of latency-bound programs (small
+// pieces, as many workgroups as contexts).  Measured on a 64-rank ring all-reduce of 2 KiB pieces it
+// takes 15% off the LL time; with the counter protocol it gains nothing (a hop is then bound by the
+// memory round trips of payload, acknowledgement and counter, not by instructions), so that
+// protocol always runs hosted.  Returns false if the launch was given up.
+template <class R, bool VEC, bool LL>
+__device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, int ctx, unsigned long long* prof4) {
+  constexpr int EB = R::kElemBytes;
+  constexpr int UB = VEC ? 16 : EB;
+  const bool writer = threadIdx.x == 0;
+  u64* const abort_word = p.sync_cur;
+  Hosted h;
+  Context c;
+  init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+  while (c.active) {
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t0 = wall_clock64();
+#endif
+    {  // wait until the step may start.  LL: not for the message itself -- the lines are retried by the threads that read them
+      const bool watch1 = c.w1 && !LL;
+      unsigned spins = 0;
+      u64 deadline = 0;
+      bool armed = false;
+      for (;;) {
+        // one lane asks memory, the wave shares the answers
+        u64 l0 = 0, l1 = 0, l2 = 0;
+        if (writer) {
+          if (c.w0) l0 = load_counter(c.w0);
+          if (watch1) l1 = load_counter(c.w1);
+          if (c.w2) l2 = load_counter(c.w2);
+        }
+        const u64 v0 = first_lane(l0), v1 = first_lane(l1), v2 = first_lane(l2);
+        const int what = (c.w0 && v0 < c.t0) ? 0 : (watch1 && v1 < c.t1) ? 1 : (c.w2 && v2 < c.t2) ? 2 : -1;
+        if (what < 0) break;
+        __builtin_amdgcn_s_sleep(1);
+        if ((++spins & 0x3fu) == 0) {
+          const u64 now = wall_clock64();
+          if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
+          if (load_counter(abort_word) != 0) return false;
+          if (now > deadline) {
+            if (writer && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
+              mscclx_status* hs = p.host_status;
+              hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
+              __threadfence_system();
+              __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            return false;
+          }
+        }
+      }
+    }
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t1 = wall_clock64();
+#endif
+    if (c.moves) do_move<R, VEC, LL>(c.m, p, epoch, c.rseq, c.sseq, h.tb, c.step, h.slice, c.pass);
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t2 = wall_clock64();
+#endif
+    const DevOp next = fetch_next_op(c, h, p);
+    if (c.moves) __builtin_amdgcn_s_waitcnt(0);  // this wave's stores are acknowledged: the counters may announce them
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t3 = wall_clock64();
+#endif
+    finish_step<UB, LL>(c, h, p, epoch, next, writer);
+#ifdef MSCCLX_PROFILE
+    const u64 prof_t4 = wall_clock64();
+    prof4[0] += prof_t1 - prof_t0; prof4[1] += prof_t2 - prof_t1; prof4[2] += prof_t3 - prof_t2; prof4[3] += prof_t4 - prof_t3;
+#endif
+  }
+  return true;
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -558,47 +718,20 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   Hosted& h = sh_hosted[lane & (kMaxHosted - 1)];  // this lane's entry; lanes of other waves never look at it
   Context c;
   c.active = false;
-  if (poller && lane < hosted) {
-    h.tb = p.ctx_tb[ctx_begin + lane];
-    h.slice = p.ctx_slice[ctx_begin + lane];
-    const DevTb tb = p.tbs[h.tb];
-    h.nops = tb.nops; h.op_begin = tb.op_begin;
-    const uint64_t u0 = p.chunk_units * (uint64_t)h.slice / p.slices, u1 = p.chunk_units * (uint64_t)(h.slice + 1) / p.slices;
-    h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
-    const uint64_t slice_fifo = (uint64_t)h.slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16)
-    const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)h.slice * p.sync_slice_words);
-    const uint32_t heads = area + (uint32_t)p.ntbs * kSyncStrideWords, tails = heads + (uint32_t)p.nconns * kSyncStrideWords;
-    h.flags = area;
-    h.my_flag = area + (uint32_t)h.tb * kSyncStrideWords;
-    h.in_slots = h.out_slots = 0; h.in_slot_bytes = h.out_slot_bytes = 0; h.in_wrap = h.out_wrap = 0;
-    h.head_in = h.tail_out = h.head_out = h.tail_in = 0;
-    if (tb.recv_conn >= 0) {
-      const DevConn cn = p.conns[tb.recv_conn];
-      h.in_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.in_slot_bytes = (uint32_t)(cn.slot_units * FB); h.in_wrap = h.in_slot_bytes * (uint32_t)p.depth;
-      h.head_in = heads + (uint32_t)tb.recv_conn * kSyncStrideWords; h.tail_out = tails + (uint32_t)tb.recv_conn * kSyncStrideWords;
-    }
-    if (tb.send_conn >= 0) {
-      const DevConn cn = p.conns[tb.send_conn];
-      h.out_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.out_slot_bytes = (uint32_t)(cn.slot_units * FB); h.out_wrap = h.out_slot_bytes * (uint32_t)p.depth;
-      h.head_out = heads + (uint32_t)tb.send_conn * kSyncStrideWords; h.tail_in = tails + (uint32_t)tb.send_conn * kSyncStrideWords;
-    }
-    c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
-    c.left = (uint32_t)(u1 - u0);
-    c.off = u0 * UB;
-    c.active = tb.nops > 0 && h.npasses > 0;
-    // clear, for the next launch, the counters this context is the only writer of
-    u64* nxt = slice_area(p.sync_nxt, p, h.slice);
-    nxt[(uint64_t)h.tb * kSyncStrideWords] = 0;
-    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
-    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
-    if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[tb.op_begin]);
-  }
-  if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
-  int cursor = 0;
 #ifdef MSCCLX_PROFILE
   u64 prof_wait = 0, prof_move = 0, prof_ack = 0, prof_fin = 0;
   const u64 prof_start = wall_clock64();
 #endif
+  if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
+  if (LL && hosted == 1 && blockDim.x == 64) {
+    unsigned long long prof4[4] = {0, 0, 0, 0};
+    run_solo<R, VEC, LL>(p, epoch, ctx_begin, prof4);
+#ifdef MSCCLX_PROFILE
+    prof_wait = prof4[0]; prof_move = prof4[1]; prof_ack = prof4[2]; prof_fin = prof4[3];
+#endif
+  } else {
+  if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
+  int cursor = 0;
 
   for (;;) {
 #ifdef MSCCLX_PROFILE
@@ -681,36 +814,8 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     // ---- the chosen context's step: move one piece ----
     {
       const Move m = sh_move;
-      const u64 cs = p.chunk_units;
-      unsigned char* const dst = (unsigned char*)m.dst;
-      unsigned char* const out = (unsigned char*)m.out;
-      const unsigned char* const a = (const unsigned char*)m.a;
-      if (LL && (m.kind & kLLKind)) {
-        const uint32_t fin = ll_flag(epoch, sh_seq[0]), fout = ll_flag(epoch, sh_seq[1]);
-        const LLWatch watch{abort_word, p.host_status, p.timeout_ticks, sh_who[0], sh_who[1], sh_who[2], (u64)(unsigned)sh_who[3]};
-        switch (m.kind & 7) {
-          case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-          case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-          case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-          case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-          case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-          case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-          case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-          default: break;
-        }
-      } else {
-        const u64 stride_a = (m.kind & kAPacked) ? (u64)m.n : cs;
-        unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
-        const u64 stride_o1 = (m.kind & kToSlot) ? (u64)m.n : cs;
-        switch (m.kind & 7) {
-          case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-          case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-          case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n); break;
-          case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n); break;
-          case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n); break;
-          default: break;
-        }
-      }
+      if (LL) do_move<R, VEC, LL>(m, p, epoch, sh_seq[0], sh_seq[1], sh_who[0], sh_who[1], sh_who[2], (unsigned)sh_who[3]);
+      else do_move<R, VEC, LL>(m, p, epoch, 0, 0, 0, 0, 0, 0);
     }
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
@@ -737,6 +842,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
 #endif
   }
+  }  // hosted contexts
   if (threadIdx.x == 0) {
     // the last workgroup out re-arms the control block: next launch uses the other counter area
     const u64 finished = __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

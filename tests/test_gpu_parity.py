@@ -280,8 +280,10 @@ def test_watchdog_reports_instead_of_hanging():
     assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
 
 
-def test_watchdog_in_ll_mode():
-    """Flag-in-data lines, one context per workgroup: the receiving threads themselves wait on the
+@pytest.mark.parametrize("threads", [0, 64])
+def test_watchdog_in_ll_mode(threads):
+    """Flag-in-data lines, one context per workgroup (threads=64: a workgroup of one wave, which runs
+    its context without a polling lane): the receiving threads themselves wait on the
     lines, so they carry the watchdog.  Same scenario as above; afterwards the same binding is launched
     again (the library clears counters and lines after a lost launch) -- it times out the same way,
     cleanly -- and a fresh plan with the default limit delivers."""
@@ -289,8 +291,8 @@ def test_watchdog_in_ll_mode():
     xml = ir_samples.slow_producer_xml(24)
     nbytes = 64 << 20
     ex = Executor(xml)
-    info = ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, protocol="ll")
-    assert info.protocol == 2
+    info = ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, protocol="ll", threads=threads)
+    assert info.protocol == 2 and info.max_hosted == 1
     x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
     ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
     ex.bind(ins, outs)
