@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM-side bytes per launch of the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/exec_kernel_c2_ring_allgather_pmc.txt), each scaled by what the same counter reads for a
 # plain device copy of 1 GiB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Not measured for the others.
-MEASURED_TRAFFIC_BYTES = {"c2": 3766862474}
+MEASURED_TRAFFIC_BYTES = {"c2": 3763781849}
 
 
 def ensure_built():
