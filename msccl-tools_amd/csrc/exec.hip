@@ -535,7 +535,7 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
   h.slice = slice;
   const DevTb tb = p.tbs[tbi];
   h.nops = tb.nops; h.op_begin = tb.op_begin;
-  const uint64_t u0 = p.chunk_units * (uint64_t)slice / p.slices, u1 = p.chunk_units * (uint64_t)(slice + 1) / p.slices;
+  const uint64_t u0 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice), u1 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice + 1);
   h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
   const uint64_t slice_fifo = (uint64_t)slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
   const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words);
@@ -1135,6 +1135,7 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
   kp.sync_slice_words = g.sync_slice_words;
   kp.timeout_ticks = (uint64_t)plan->timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
+  kp.slice_grain = g.slice_grain;
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan->tbs.size(); kp.nconns = (int)plan->conns.size();
   kp.wg_begin = d->hosting;
   kp.ctx_tb = d->hosting + g.wg_begin.size();

@@ -3,6 +3,7 @@
 #include "plan.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -386,6 +387,29 @@ static int decide_geometry_simple_retry(mscclx_plan& plan, size_t chunk_bytes, i
   return decide_geometry(plan, chunk_bytes, dtype, simple, num_cus, capacity_by_threads, fifo_budget_bytes, out);
 }
 
+// How evenly longest-processing-time-first spreads `slices` copies of every threadblock over `wgs`
+// workgroups of at most kMaxHosted contexts: mean load / largest load, 1 = perfectly even.
+static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t slices, int64_t wgs) {
+  std::vector<uint64_t> sorted(tb_works);
+  std::sort(sorted.begin(), sorted.end(), std::greater<uint64_t>());
+  typedef std::pair<uint64_t, int> Load;  // (work so far, contexts so far)
+  std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+  for (int64_t w = 0; w < wgs; ++w) heap.push({0, 0});
+  uint64_t total = 0, largest = 0;
+  for (uint64_t work : sorted)
+    for (int64_t j = 0; j < slices; ++j) {
+      if (heap.empty()) return 0.0;
+      Load l = heap.top();
+      heap.pop();
+      l.first += work / (uint64_t)slices + 1;
+      l.second += 1;
+      total += work / (uint64_t)slices + 1;
+      largest = std::max(largest, l.first);
+      if (l.second < kMaxHosted) heap.push(l);
+    }
+  return largest ? (double)total / (double)wgs / (double)largest : 1.0;
+}
+
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);
@@ -417,23 +441,48 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.depth = depth;
 
   // Slices are independent copies of the program on 1/slices of every chunk; they are what keeps
-  // the chip busy while one copy waits on its dependency chain.  Aim at pieces of about 256 KiB,
-  // bounded by what the resident workgroups can host.
+  // the chip busy while one copy waits on its dependency chain.
   const int most_threads_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
   const int64_t host_limit = (int64_t)most_threads_capacity * kMaxHosted;
   if (ntbs > host_limit)
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
   int64_t slices = cfg.slices;
   if (!slices) {
-    // big chunks: pieces of about 128 KiB amortise the per-step hand-off; small chunks: enough
-    // slices that every compute unit has a context or two, but no piece below 2 KiB
-    const int64_t by_piece = (int64_t)(chunk_bytes / (128 * 1024));
-    const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;
-    slices = std::max<int64_t>(1, std::max(by_piece, to_fill));
-    slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
-    // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~32
-    const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 32) / ntbs);
-    slices = std::min(slices, comfortable);
+    const int64_t by_piece = (int64_t)(chunk_bytes / (128 * 1024));  // most slices of at least 128 KiB
+    const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs; // fewest slices that give every compute unit a context or two
+    if (by_piece >= 2) {
+      // Big chunks.  Measured on MI355X (16 to 1920 threadblocks, 2 to 8 MiB chunks): what matters
+      // is (1) that the contexts spread EVENLY over the resident workgroups -- 7.5 contexts per
+      // workgroup on average means some host 8, and the launch takes as long as those take --
+      // (2) about a dozen contexts per workgroup: enough to always find one ready, few enough to poll,
+      // and (3) several passes of 64 KiB pieces over a slice rather than one big piece, so that
+      // the phases of a program overlap (pass k+1 of an early phase runs beside pass k of a later one).
+      const int threads = cfg.threads && thread_index(cfg.threads) >= 0 ? cfg.threads : 512;
+      int64_t wgs_all = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
+      wgs_all = std::max<int64_t>(1, std::min<int64_t>(wgs_all, capacity_by_threads[thread_index(threads)]));
+      std::vector<uint64_t> works;
+      for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
+      const int64_t lo = std::max<int64_t>(1, std::min(to_fill, by_piece));
+      const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(by_piece, (wgs_all * kMaxHosted) / ntbs));
+      std::vector<int64_t> candidates = {lo, hi};
+      for (int64_t base = 1; base <= hi; base *= 2)
+        for (int64_t c : {base, base * 3})
+          if (c >= lo && c <= hi) candidates.push_back(c);
+      double best_score = -1e9;
+      for (int64_t c : candidates) {
+        const int64_t wgs = std::min<int64_t>(wgs_all, c * ntbs);
+        const double per_wg = (double)(c * ntbs) / (double)wgs;
+        const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / 12.0));
+        if (score > best_score + 1e-9 || (std::fabs(score - best_score) <= 1e-9 && c < slices)) { best_score = score; slices = c; }
+      }
+    } else {
+      // small chunks: enough slices that every compute unit has a context or two, but no piece below 2 KiB
+      slices = std::max<int64_t>(1, std::max(by_piece, to_fill));
+      slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
+      // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~32
+      const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 32) / ntbs);
+      slices = std::min(slices, comfortable);
+    }
   }
   slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
   if (slices < 1 || (cfg.slices && (uint64_t)cfg.slices > g.chunk_units)) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");
@@ -444,8 +493,20 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.slices = (int)slices;
 
   // piece: the whole slice in one pass unless the FIFO slots of staged messages would not fit the budget
-  const uint64_t longest_slice = (g.chunk_units + slices - 1) / slices;
+  g.slice_grain = std::max<uint32_t>(1, 256 / g.unit_bytes);
+  if (g.chunk_units / g.slice_grain < (uint64_t)slices) g.slice_grain = 1;
+  uint64_t longest_slice = 0;
+  for (int64_t j = 0; j < slices; ++j)
+    longest_slice = std::max(longest_slice, slice_begin(g.chunk_units, g.slice_grain, (int32_t)slices, (int32_t)j + 1) -
+                                                slice_begin(g.chunk_units, g.slice_grain, (int32_t)slices, (int32_t)j));
   uint64_t piece_units = cfg.piece_bytes ? std::max<uint64_t>(1, (uint64_t)cfg.piece_bytes / g.unit_bytes) : longest_slice;
+  if (!cfg.piece_bytes && longest_slice * g.unit_bytes > 128 * 1024) {
+    // equal passes of at most 64 KiB (a short last pass costs as many hand-offs as a full one), on 256-byte boundaries
+    const uint64_t target = (uint64_t)(64 * 1024) / g.unit_bytes;
+    const uint64_t passes = (longest_slice + target - 1) / target;
+    piece_units = (longest_slice + passes - 1) / passes;
+    piece_units = (piece_units + g.slice_grain - 1) / g.slice_grain * g.slice_grain;
+  }
   piece_units = std::min(piece_units, longest_slice);
   // protocol: flag-in-data lines pay twice the slot traffic and stage every message to take the
   // counter round trip out of a hand-off.  Chosen only on request: measured on MI355X a hop is bound
@@ -493,7 +554,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
   } else {
     const uint64_t piece_bytes = piece_units * g.unit_bytes;
-    threads = piece_bytes >= 64 * 1024 ? 512 : piece_bytes >= 32 * 1024 ? 256 : piece_bytes >= 16 * 1024 ? 128 : 64;
+    threads = piece_bytes >= 48 * 1024 ? 512 : piece_bytes >= 24 * 1024 ? 256 : piece_bytes >= 12 * 1024 ? 128 : 64;
     while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
   }
   const int capacity = capacity_by_threads[thread_index(threads)];

@@ -83,6 +83,7 @@ struct Geometry {
   uint32_t unit_bytes = 0;
   uint32_t piece_units = 0;
   int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
+  uint32_t slice_grain = 1;       // see slice_begin()
   int32_t staging = 0;            // 1: every message goes through a FIFO slot
   int32_t ll = 0;                 // 1: flag-in-data lines in the slots (implies staging); FIFO bytes double
   int32_t workgroups = 0;         // resident workgroups; each hosts up to kMaxHosted (threadblock, slice) contexts
@@ -112,11 +113,25 @@ struct KernelParams {
   uint64_t sync_words;
   uint64_t timeout_ticks;
   uint32_t piece_units;
+  uint32_t slice_grain;
   int32_t slices, depth, ntbs, nconns;
   const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
   const int32_t* ctx_tb;        // hosted contexts, grouped by workgroup: threadblock row ...
   const int32_t* ctx_slice;     // ... and slice
 };
+
+#ifdef __HIPCC__
+#define MSCCLX_HOST_DEVICE __host__ __device__
+#else
+#define MSCCLX_HOST_DEVICE
+#endif
+// First unit of slice j of a chunk (j = slices: one past the chunk's last unit).  The chunk is dealt
+// out in groups of `grain` units (256 bytes where a chunk has at least one such group per slice, so
+// that no slice starts in the middle of a cache line; else 1); the last slice takes the remainder.
+MSCCLX_HOST_DEVICE inline uint64_t slice_begin(uint64_t chunk_units, uint32_t grain, int32_t slices, int32_t j) {
+  if (j >= slices) return chunk_units;
+  return (chunk_units / grain) * (uint64_t)j / (uint64_t)slices * grain;
+}
 
 constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes

@@ -262,7 +262,7 @@ def test_watchdog_reports_instead_of_hanging():
     xml = ir_samples.slow_producer_xml(24)
     nbytes = 64 << 20
     ex = Executor(xml)
-    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1)  # one pass: the receive waits for all 24 copies
+    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, piece_bytes=nbytes)  # one pass: the receive waits for all 24 copies
     x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
     ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
     ex.bind(ins, outs)
@@ -291,7 +291,7 @@ def test_watchdog_in_ll_mode(threads):
     xml = ir_samples.slow_producer_xml(24)
     nbytes = 64 << 20
     ex = Executor(xml)
-    info = ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, protocol="ll", threads=threads)
+    info = ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, piece_bytes=nbytes, protocol="ll", threads=threads)
     assert info.protocol == 2 and info.max_hosted == 1
     x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
     ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
