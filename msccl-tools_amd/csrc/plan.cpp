@@ -380,13 +380,6 @@ static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
   return w;
 }
 
-static int decide_geometry_simple_retry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg, int num_cus,
-                                        const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
-  mscclx_config simple = cfg;
-  simple.protocol = MSCCLX_PROTO_SIMPLE;
-  return decide_geometry(plan, chunk_bytes, dtype, simple, num_cus, capacity_by_threads, fifo_budget_bytes, out);
-}
-
 // How evenly longest-processing-time-first spreads `slices` copies of every threadblock over `wgs`
 // workgroups of at most kMaxHosted contexts: mean load / largest load, 1 = perfectly even.
 static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t slices, int64_t wgs) {
@@ -540,12 +533,8 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (g.ll) {  // a message's flag carries its sequence number in 22 bits
     int64_t most = 0;
     for (const Conn& c : plan.conns) most = std::max<int64_t>(most, c.nmsg);
-    if (most * g.passes >= (1 << 22) - 1) {
-      if (cfg.protocol == MSCCLX_PROTO_LL) return fail(MSCCLX_ERR_UNSUPPORTED, "too many messages per connection for the LL protocol");
-      g.ll = 0;
-      g.staging = cfg.staging ? 1 : 0;
-      return decide_geometry_simple_retry(plan, chunk_bytes, dtype, cfg, num_cus, capacity_by_threads, fifo_budget_bytes, out);
-    }
+    if (most * g.passes >= (1 << 22) - 1)
+      return fail(MSCCLX_ERR_UNSUPPORTED, "too many messages per connection for the LL protocol; use a larger piece_bytes");
   }
 
   // threads: enough to cover a piece with 8 16-byte loads per thread

@@ -308,3 +308,33 @@ def test_watchdog_in_ll_mode(threads):
     ins, outs, _ = collective_buffers(ex2.tables, nbytes, "uint8", inputs=x)
     ex2.run(ins, outs)
     assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
+
+
+@pytest.mark.parametrize("knobs", [dict(threads=64), dict(threads=128, workgroups=2)])
+def test_ll_launch_number_wraps(knobs):
+    """The flag of an LL line carries the launch number in 10 bits.  1040 launches on one binding, each
+    on the previous launch's results (in-place all-reduce of 3 ranks on 32-bit integers: after k launches every
+    element is 3^(k-1) times the first sum, modulo 2^32, so every launch moves different bits and a line
+    taken from an earlier launch would show): checked before, at and after the number wraps."""
+    from msccl.executor import Executor, collective_buffers
+    n, E = 3, 300
+    xml = ir_samples.ring_allreduce_xml(n)
+    ex = Executor(xml)
+    info = ex.setup(E * 4, "int32", protocol="ll", piece_bytes=512, **knobs)  # several passes: slots are reused inside a launch too
+    assert info.protocol == 2 and info.passes >= 2
+    rng = np.random.default_rng(11)
+    x = [rng.integers(0, 2**32, n * E, dtype=np.uint64).astype(np.uint32) for _ in range(n)]
+    ins, outs, _ = collective_buffers(ex.tables, E * 4, "int32", inputs=[torch.from_numpy(v.view(np.int32)).clone() for v in x])
+    ex.bind(ins, outs)
+    first = (x[0].astype(np.uint64) + x[1] + x[2]).astype(np.uint32)
+    check_at = {1, 2, 3, 1022, 1023, 1024, 1025, 1026, 1040}
+    print(f"case: ll launch-number wrap knobs={knobs}", flush=True)
+    for k in range(1, 1041):
+        ex.launch()
+        if k in check_at:
+            ex.wait()
+            want = (first.astype(np.uint64) * pow(3, k - 1, 2**32) % 2**32).astype(np.uint32)
+            for r in range(n):
+                got = ins[r].cpu().numpy().view(np.uint32)
+                assert np.array_equal(got, want), (k, r, int(np.flatnonzero(got != want)[0]))
+    ex.wait()
