@@ -25,11 +25,10 @@ for p in (ROOT, os.path.join(ROOT, "msccl-tools_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM-side bytes per launch of the headline workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/exec_kernel_c2_ring_allgather_pmc.txt), each scaled by what the same counter reads for a
-# plain device copy of 1 GiB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Not measured for the others.
-MEASURED_TRAFFIC_BYTES = {"c2": 3763781849}
-
+# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/exec_kernel_c2_c3_c4_pmc.txt),
+# each scaled by what the same counter reads for a plain device copy of 1 GiB (FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0).  Not measured for the two latency-bound workloads.
+MEASURED_TRAFFIC_BYTES = {"c2": 3763771775, "c3": 3230774849, "c4": 20917183064}
 
 def ensure_built():
     from msccl.executor import binding
@@ -211,6 +210,7 @@ def main():
             r = run_workload(key, max(5, args.steps // 2), args.warmup)
             line["others"][key] = {k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items() if k != "geometry"}
             line["others"][key].update(r["geometry"])
+            line["others"][key]["traffic"] = MEASURED_TRAFFIC_BYTES.get(key)
     print(json.dumps(line))
 
 
