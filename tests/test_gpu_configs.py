@@ -10,6 +10,7 @@ import pytest
 import torch
 
 import golden_util
+import ir_samples
 from msccl.executor.workloads import WORKLOADS, numpy_input, torch_input
 from oracle import collectives as oc
 from oracle import ir_interp as oi
@@ -136,6 +137,43 @@ def test_config_full_size_properties(key):
             for r in range(n):
                 assert torch.equal(res[r][c * E:(c + 1) * E].view(itype), want.view(itype)), (c, r)
     del x, ins, outs, res
+    torch.cuda.empty_cache()
+
+
+def test_chunks_beyond_4_gib():
+    """Chunks larger than 4 GiB: every offset inside a rank buffer needs more than 32 bits.  A two-rank
+    in-place all-gather of 5 GiB chunks (ragged against the slices) and a three-rank in-place all-reduce
+    of 4.5 GiB per rank (its rrs results go through FIFO slots), both checked against closed forms on
+    the device."""
+    from msccl.executor import Executor, collective_buffers
+    dev = "cuda:0"
+    cb = (5 << 30) + 48
+    ex = Executor(ir_samples.ring_allgather_xml(2, 1))
+    print("case: 5 GiB chunks, all-gather", flush=True)
+    info = ex.setup(cb, "uint8")
+    x = [torch.randint(0, 256, (cb,), dtype=torch.uint8, device=dev) for _ in range(2)]
+    ins, outs, res = collective_buffers(ex.tables, cb, "uint8", device=dev, inputs=x)
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    for r in range(2):
+        assert torch.equal(res[r][:cb], x[0]) and torch.equal(res[r][cb:], x[1]), r
+    del x, ins, outs, res, ex
+    torch.cuda.empty_cache()
+
+    cb = (3 << 29) + 64
+    E = cb // 4
+    ex = Executor(ir_samples.ring_allreduce_xml(3))
+    print("case: 3 x 1.5 GiB chunks per rank, all-reduce", flush=True)
+    info = ex.setup(cb, "int32")
+    assert info.passes > 1 and info.staged_messages > 0
+    x = [torch.randint(-2**31, 2**31 - 1, (3 * E,), dtype=torch.int32, device=dev) for _ in range(3)]
+    want = x[0] + x[1] + x[2]
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", device=dev, inputs=x)
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    for r in range(3):
+        assert torch.equal(res[r], want), r
+    del x, ins, outs, res, want, ex
     torch.cuda.empty_cache()
 
 
