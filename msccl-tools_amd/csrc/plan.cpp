@@ -380,6 +380,52 @@ static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
   return w;
 }
 
+// How many threadblocks there are for every threadblock that is busy, on average, while the program
+// runs: threadblocks x depth of the dataflow / moving steps, where the depth is the longest chain of
+// moving steps through step order, depid/deps and send -> matching receive (connections unbounded).
+// 1 = every threadblock always has something to do (a ring); a program in phases, or one whose
+// threadblocks mostly wait for each other, scores higher and needs more contexts per workgroup for a
+// workgroup to find a ready one.
+static double waiting_ratio(const mscclx_plan& plan) {
+  const int ntb = (int)plan.tbs.size();
+  std::vector<int> pc(ntb, 0);
+  std::vector<int32_t> level(plan.ops.size(), -1);
+  size_t remaining = plan.ops.size();
+  int64_t moving = 0;
+  int32_t depth = 0;
+  while (remaining) {
+    size_t progressed = 0;
+    for (int t = 0; t < ntb; ++t) {
+      const Tb& tb = plan.tbs[t];
+      while (tb.op_begin + pc[t] < tb.op_end) {
+        const int o = tb.op_begin + pc[t];
+        const Op& op = plan.ops[o];
+        int32_t l = pc[t] ? level[o - 1] : 0;
+        if (op.depid >= 0) {
+          const Tb& dep = plan.tbs[plan.rank_tb_begin[tb.rank] + op.depid];
+          const int32_t dl = level[dep.op_begin + op.deps];
+          if (dl < 0) break;
+          l = std::max(l, dl);
+        }
+        if (is_recv_type(op.type)) {
+          const int32_t sl = level[op.match_send];
+          if (sl < 0) break;
+          l = std::max(l, sl);
+        }
+        const bool moves = op.type != MSCCLX_OP_NOP && !(op.type == MSCCLX_OP_SEND && op.zero_copy);
+        level[o] = l + (moves ? 1 : 0);
+        moving += moves ? 1 : 0;
+        depth = std::max(depth, level[o]);
+        ++pc[t];
+        ++progressed;
+      }
+    }
+    if (!progressed) return 1.0;  // (a program that cannot finish is refused elsewhere)
+    remaining -= progressed;
+  }
+  return moving ? std::max(1.0, (double)ntb * (double)depth / (double)moving) : 1.0;
+}
+
 // How evenly longest-processing-time-first spreads `slices` copies of every threadblock over `wgs`
 // workgroups of at most kMaxHosted contexts: mean load / largest load, 1 = perfectly even.
 static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t slices, int64_t wgs) {
@@ -394,9 +440,9 @@ static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t sli
       if (heap.empty()) return 0.0;
       Load l = heap.top();
       heap.pop();
-      l.first += work / (uint64_t)slices + 1;
+      l.first += work + 1;  // the weights the hosting table itself is built with
       l.second += 1;
-      total += work / (uint64_t)slices + 1;
+      total += work + 1;
       largest = std::max(largest, l.first);
       if (l.second < kMaxHosted) heap.push(l);
     }
@@ -443,11 +489,12 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (!slices) {
     const int64_t by_piece = (int64_t)(chunk_bytes / (128 * 1024));  // most slices of at least 128 KiB
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs; // fewest slices that give every compute unit a context or two
-    if (by_piece >= 2) {
-      // Big chunks.  Measured on MI355X (16 to 1920 threadblocks, 2 to 8 MiB chunks): what matters
+    if (by_piece >= 2 && by_piece >= to_fill) {
+      // Big chunks: slices of 128 KiB or more can occupy every compute unit.  Measured on MI355X (16 to 1920 threadblocks, 2 to 8 MiB chunks): what matters
       // is (1) that the contexts spread EVENLY over the resident workgroups -- 7.5 contexts per
       // workgroup on average means some host 8, and the launch takes as long as those take --
-      // (2) about a dozen contexts per workgroup: enough to always find one ready, few enough to poll,
+      // (2) enough contexts per workgroup to always find one ready -- four for every threadblock
+      // that is busy at a time (waiting_ratio), between 4 and 32 --
       // and (3) several passes of 64 KiB pieces over a slice rather than one big piece, so that
       // the phases of a program overlap (pass k+1 of an early phase runs beside pass k of a later one).
       const int threads = cfg.threads && thread_index(cfg.threads) >= 0 ? cfg.threads : 512;
@@ -455,17 +502,18 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       wgs_all = std::max<int64_t>(1, std::min<int64_t>(wgs_all, capacity_by_threads[thread_index(threads)]));
       std::vector<uint64_t> works;
       for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
-      const int64_t lo = std::max<int64_t>(1, std::min(to_fill, by_piece));
+      const int64_t lo = std::max<int64_t>(1, to_fill);
       const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(by_piece, (wgs_all * kMaxHosted) / ntbs));
       std::vector<int64_t> candidates = {lo, hi};
       for (int64_t base = 1; base <= hi; base *= 2)
         for (int64_t c : {base, base * 3})
           if (c >= lo && c <= hi) candidates.push_back(c);
+      const double wanted_per_wg = std::min(32.0, 4.0 * waiting_ratio(plan));
       double best_score = -1e9;
       for (int64_t c : candidates) {
         const int64_t wgs = std::min<int64_t>(wgs_all, c * ntbs);
         const double per_wg = (double)(c * ntbs) / (double)wgs;
-        const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / 12.0));
+        const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / wanted_per_wg));
         if (score > best_score + 1e-9 || (std::fabs(score - best_score) <= 1e-9 && c < slices)) { best_score = score; slices = c; }
       }
     } else {
