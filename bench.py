@@ -2,6 +2,7 @@
 """Benchmark of the MI355X MSCCL-IR executor.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-others] [--no-cpu]
+    python bench.py --config c4 --sweep 1048576:536870912        (message-size sweep of one algorithm)
 
 A step is one execution of the whole compiled algorithm (one launch of the executor kernel) over
 buffers already resident in HBM.  The headline workload is the ring AllGather configuration
@@ -83,19 +84,19 @@ def fold_orders(key):
     return None
 
 
-def run_workload(key, steps, warmup, device="cuda:0"):
+def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None):
     import torch
     from msccl.executor import Executor, collective_buffers
     from msccl.executor.workloads import WORKLOADS, torch_input
-    w = WORKLOADS[key]
-    xml = w.build()
+    w = WORKLOADS[key] if bytes_per_rank is None else WORKLOADS[key].scaled(bytes_per_rank)
+    xml = WORKLOADS[key].build()
     ex = Executor(xml, device=device)
     info = ex.setup(w.chunk_bytes, w.dtype)
     x = [torch_input(w, r, device) for r in range(w.ranks)]
     ins, outs, res = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, device=device, inputs=x)
     ex.run(ins, outs)  # first execution from pristine inputs: the one that is verified
     torch.cuda.synchronize()
-    ok = verify(w, x, res, fold_orders(key))
+    ok = verify(w, x, res, fold_orders(key)) if bytes_per_rank is None else None  # the closed forms are written for the full size
     for _ in range(warmup):
         ex.launch()
     ex.wait()
@@ -113,7 +114,7 @@ def run_workload(key, steps, warmup, device="cuda:0"):
     kernel_s = e0.elapsed_time(e1) * 1e-3 / steps
     ab = ex.algorithmic_bytes()
     out = {"workload": w.description, "dtype": w.dtype, "ranks": w.ranks, "bytes_per_rank": w.bytes_per_rank,
-           "ms_per_step": wall_s * 1e3, "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": ab, "verified": bool(ok),
+           "ms_per_step": wall_s * 1e3, "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": ab, "verified": None if ok is None else bool(ok),
            "geometry": {k: v for k, v in info.as_dict().items() if k in ("workgroups", "threads", "slices", "piece_bytes", "fifo_depth", "passes")}}
     out.update({k: round(v, 4) for k, v in w.bandwidths(wall_s, ab).items()})
     out["roofline_frac_kernel"] = round(ab / kernel_s / 1e9 / HBM_PEAK_GBPS, 4)
@@ -165,6 +166,8 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy baseline")
+    ap.add_argument("--sweep", metavar="LO:HI", help="instead of the benchmark line: time the chosen algorithm on LO, 2*LO, ... HI bytes per "
+                    "rank (same inputs, same timing; results not verified) and print one JSON line holding the list")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run five plain device copies of 1 GiB (known traffic: 1 GiB read + 1 GiB written each), "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -187,6 +190,17 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "5 device copies of 1073741824 bytes"}))
+        return
+    if args.sweep:
+        lo, hi = (int(v) for v in args.sweep.split(":"))
+        rows = []
+        size = lo
+        while size <= hi:
+            r = run_workload(args.config, args.steps, args.warmup, bytes_per_rank=size)
+            rows.append({"bytes_per_rank": size, "kernel_us": round(r["kernel_ms"] * 1e3, 1), "algbw_GBps": round(r["algbw_GBps"], 2),
+                         "busbw_GBps": round(r["busbw_GBps"], 2), "hbm_fraction": round(r["roofline_frac_kernel"], 4), **r["geometry"]})
+            size *= 2
+        print(json.dumps({"sweep": args.config, "workload": r["workload"].split(";")[0], "dtype": r["dtype"], "steps": args.steps, "rows": rows}))
         return
     head = run_workload(args.config, args.steps, args.warmup)
     traffic = MEASURED_TRAFFIC_BYTES.get(args.config)
