@@ -380,6 +380,11 @@ static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
   return w;
 }
 
+// threads: enough to cover a piece with a few 16-byte loads per thread
+static int threads_for_piece(uint64_t piece_bytes) {
+  return piece_bytes >= 48 * 1024 ? 512 : piece_bytes >= 24 * 1024 ? 256 : piece_bytes >= 12 * 1024 ? 128 : 64;
+}
+
 // How many threadblocks there are for every threadblock that is busy, on average, while the program
 // runs: threadblocks x depth of the dataflow / moving steps, where the depth is the longest chain of
 // moving steps through step order, depid/deps and send -> matching receive (connections unbounded).
@@ -487,23 +492,22 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
   int64_t slices = cfg.slices;
   if (!slices) {
-    const int64_t by_piece = (int64_t)(chunk_bytes / (128 * 1024));  // most slices of at least 128 KiB
-    const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs; // fewest slices that give every compute unit a context or two
-    if (by_piece >= 2 && by_piece >= to_fill) {
-      // Big chunks: slices of 128 KiB or more can occupy every compute unit.  Measured on MI355X (16 to 1920 threadblocks, 2 to 8 MiB chunks): what matters
-      // is (1) that the contexts spread EVENLY over the resident workgroups -- 7.5 contexts per
-      // workgroup on average means some host 8, and the launch takes as long as those take --
-      // (2) enough contexts per workgroup to always find one ready -- four for every threadblock
-      // that is busy at a time (waiting_ratio), between 4 and 32 --
-      // and (3) several passes of 64 KiB pieces over a slice rather than one big piece, so that
-      // the phases of a program overlap (pass k+1 of an early phase runs beside pass k of a later one).
-      const int threads = cfg.threads && thread_index(cfg.threads) >= 0 ? cfg.threads : 512;
-      int64_t wgs_all = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
-      wgs_all = std::max<int64_t>(1, std::min<int64_t>(wgs_all, capacity_by_threads[thread_index(threads)]));
+    const int64_t finest = (int64_t)(chunk_bytes / (32 * 1024));       // most slices of at least 32 KiB
+    const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;  // fewest slices that give every compute unit a context or two
+    if (finest >= 2 && finest >= to_fill) {
+      // Slices of 32 KiB or more can occupy every compute unit.  Measured on MI355X (8 to 1920
+      // threadblocks, 128 KiB to 64 MiB chunks), what matters is (1) that the contexts spread EVENLY
+      // over the resident workgroups -- 7.5 contexts per workgroup on average means some host 8, and
+      // the launch takes as long as those take -- (2) enough contexts per workgroup to always find
+      // one ready -- four for every threadblock that is busy at a time (waiting_ratio), between
+      // 4 and 32 -- and (3) several passes of 64 KiB pieces over a big slice rather than one big
+      // piece, so that the phases of a program overlap (pass k+1 of an early phase runs beside
+      // pass k of a later one).  Candidates are scored on (1) and (2); (3) follows below.
       std::vector<uint64_t> works;
       for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
+      const int most_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
       const int64_t lo = std::max<int64_t>(1, to_fill);
-      const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(by_piece, (wgs_all * kMaxHosted) / ntbs));
+      const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(finest, ((int64_t)most_capacity * kMaxHosted) / ntbs));
       std::vector<int64_t> candidates = {lo, hi};
       for (int64_t base = 1; base <= hi; base *= 2)
         for (int64_t c : {base, base * 3})
@@ -511,14 +515,22 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       const double wanted_per_wg = std::min(32.0, 4.0 * waiting_ratio(plan));
       double best_score = -1e9;
       for (int64_t c : candidates) {
-        const int64_t wgs = std::min<int64_t>(wgs_all, c * ntbs);
+        // the workgroups this choice would run on: threads follow the piece, workgroups the threads
+        const uint64_t slice_bytes = chunk_bytes / (uint64_t)c;
+        const uint64_t piece_bytes = slice_bytes > 128 * 1024 ? 64 * 1024 : slice_bytes;
+        int threads = cfg.threads && thread_index(cfg.threads) >= 0 ? cfg.threads : threads_for_piece(piece_bytes);
+        while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
+        int64_t wgs = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
+        wgs = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(wgs, capacity_by_threads[thread_index(threads)]), c * ntbs));
+        if (wgs * kMaxHosted < c * ntbs) continue;
         const double per_wg = (double)(c * ntbs) / (double)wgs;
         const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / wanted_per_wg));
         if (score > best_score + 1e-9 || (std::fabs(score - best_score) <= 1e-9 && c < slices)) { best_score = score; slices = c; }
       }
+      if (!slices) slices = lo;
     } else {
       // small chunks: enough slices that every compute unit has a context or two, but no piece below 2 KiB
-      slices = std::max<int64_t>(1, std::max(by_piece, to_fill));
+      slices = std::max<int64_t>(1, std::max(finest, to_fill));
       slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
       // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~32
       const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 32) / ntbs);
@@ -591,7 +603,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
   } else {
     const uint64_t piece_bytes = piece_units * g.unit_bytes;
-    threads = piece_bytes >= 48 * 1024 ? 512 : piece_bytes >= 24 * 1024 ? 256 : piece_bytes >= 12 * 1024 ? 128 : 64;
+    threads = threads_for_piece(piece_bytes);
     while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
   }
   const int capacity = capacity_by_threads[thread_index(threads)];
