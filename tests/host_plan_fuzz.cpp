@@ -11,7 +11,7 @@
 
 namespace mscclx { void destroy_device_state(DeviceState*) {} }  // no device half in this build
 
-static int run_once(int nranks, const std::vector<int32_t>& rc, const std::vector<int32_t>& tbs, const std::vector<int32_t>& ops, bool expect_ok) {
+static int run_once(int nranks, const std::vector<int32_t>& rc, const std::vector<int32_t>& tbs, const std::vector<int32_t>& ops, bool expect_ok, int variants) {
   mscclx_plan_desc d{nranks, (int32_t)(tbs.size() / MSCCLX_TB_COLS), (int32_t)(ops.size() / MSCCLX_OP_COLS), rc.data(), tbs.data(), ops.data()};
   mscclx_plan* p = nullptr;
   int rc_create = mscclx_plan_create(&d, &p);
@@ -23,14 +23,17 @@ static int run_once(int nranks, const std::vector<int32_t>& rc, const std::vecto
   (void)mscclx_plan_simulate(p, 2);
   (void)mscclx_plan_algorithmic_units(p);
   const int capacity[4] = {4096, 2048, 1024, 512};
-  mscclx_config cfg = {};
   mscclx::Geometry g;
+  for (int variant = 0; variant < variants; ++variant)  // 0 automatic, 1 LL lines, 2 explicit knobs with staging
   for (size_t chunk : {(size_t)4, (size_t)4096, (size_t)(1 << 20) + 16, (size_t)3 << 20}) {
+    mscclx_config cfg = {};
+    if (variant == 1) cfg.protocol = MSCCLX_PROTO_LL;
+    if (variant == 2) { cfg.staging = 1; cfg.slices = 3; cfg.piece_bytes = 4096; }
     int r = mscclx::decide_geometry(*p, chunk, MSCCLX_F32, cfg, 256, capacity, 1ull << 30, &g);
     if (r == MSCCLX_OK) {
       size_t hosted = g.ctx_tb.size();
       if (hosted != p->tbs.size() * (size_t)g.slices || g.wg_begin.back() != (int32_t)hosted) { fprintf(stderr, "hosting table does not cover every context\n"); return 1; }
-    } else if (expect_ok && r != MSCCLX_ERR_DEADLOCK && r != MSCCLX_ERR_CAPACITY) {
+    } else if (expect_ok && r != MSCCLX_ERR_DEADLOCK && r != MSCCLX_ERR_CAPACITY && r != MSCCLX_ERR_UNSUPPORTED && r != MSCCLX_ERR_INVALID_ARG) {
       fprintf(stderr, "geometry failed on valid tables: %s\n", mscclx_last_error());
       return 1;
     }
@@ -49,7 +52,7 @@ int main(int argc, char** argv) {
   if (fread(rc.data(), 4, rc.size(), f) != rc.size() || fread(tbs.data(), 4, tbs.size(), f) != tbs.size() ||
       fread(ops.data(), 4, ops.size(), f) != ops.size()) return 2;
   fclose(f);
-  if (run_once(hdr[0], rc, tbs, ops, true)) return 1;
+  if (run_once(hdr[0], rc, tbs, ops, true, 3)) return 1;
   std::mt19937 rng(12345);
   const int mutations = atoi(argv[2]);
   const int32_t nasty[] = {-2147483647 - 1, -2, -1, 0, 1, 2, 7, 63, 64, 65, 1000, 2147483647};
@@ -61,7 +64,7 @@ int main(int argc, char** argv) {
       if (v.empty()) continue;
       v[rng() % v.size()] = (rng() % 2) ? nasty[rng() % 12] : (int32_t)(rng() % 40) - 4;
     }
-    if (run_once(hdr[0], a, b, c, false)) return 1;
+    if (run_once(hdr[0], a, b, c, false, m % 8 == 0 ? 3 : 1)) return 1;
   }
   printf("ok: %d mutated tables handled\n", mutations);
   return 0;
