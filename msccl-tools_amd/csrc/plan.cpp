@@ -391,7 +391,7 @@ static int threads_for_piece(uint64_t piece_bytes) {
 // 1 = every threadblock always has something to do (a ring); a program in phases, or one whose
 // threadblocks mostly wait for each other, scores higher and needs more contexts per workgroup for a
 // workgroup to find a ready one.
-static double waiting_ratio(const mscclx_plan& plan) {
+static double waiting_ratio(const mscclx_plan& plan, int32_t* depth_out = nullptr) {
   const int ntb = (int)plan.tbs.size();
   std::vector<int> pc(ntb, 0);
   std::vector<int32_t> level(plan.ops.size(), -1);
@@ -425,9 +425,10 @@ static double waiting_ratio(const mscclx_plan& plan) {
         ++progressed;
       }
     }
-    if (!progressed) return 1.0;  // (a program that cannot finish is refused elsewhere)
+    if (!progressed) { if (depth_out) *depth_out = 1; return 1.0; }  // (a program that cannot finish is refused elsewhere)
     remaining -= progressed;
   }
+  if (depth_out) *depth_out = std::max<int32_t>(1, depth);
   return moving ? std::max(1.0, (double)ntb * (double)depth / (double)moving) : 1.0;
 }
 
@@ -495,7 +496,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     const int64_t finest = (int64_t)(chunk_bytes / (32 * 1024));       // most slices of at least 32 KiB
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;  // fewest slices that give every compute unit a context or two
     if (finest >= 2 && finest >= to_fill) {
-      // Slices of 32 KiB or more can occupy every compute unit.  Measured on MI355X (8 to 1920
+      // Slices of 32 KiB or more can give every compute unit a context.  Measured on MI355X (8 to 1920
       // threadblocks, 128 KiB to 64 MiB chunks), what matters is (1) that the contexts spread EVENLY
       // over the resident workgroups -- 7.5 contexts per workgroup on average means some host 8, and
       // the launch takes as long as those take -- (2) enough contexts per workgroup to always find
@@ -529,9 +530,21 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       }
       if (!slices) slices = lo;
     } else {
-      // small chunks: enough slices that every compute unit has a context or two, but no piece below 2 KiB
-      slices = std::max<int64_t>(1, std::max(finest, to_fill));
-      slices = std::min<int64_t>(slices, std::max<int64_t>(1, (int64_t)(chunk_bytes / 2048)));
+      // Small chunks: the launch is bound by latency.  Its time is about
+      //   a * contexts + depth * (h0 + b * piece bytes)
+      // -- a fixed cost per workgroup launched, and one hand-off plus one small move for every step
+      // on the longest chain of the program's dataflow.  More slices shrink the pieces but add
+      // workgroups; the minimum is at slices = sqrt(b/a * depth * chunk / threadblocks).  Fitted on
+      // MI355X with workgroups of one wave: a = 16 ns per workgroup, b = 100 ns per KiB, which puts
+      // an 8-rank ring on 1 MiB at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.
+      // Never finer than a context or two per compute unit, nor pieces below 512 bytes.
+      int32_t depth_of_dataflow = 1;
+      (void)waiting_ratio(plan, &depth_of_dataflow);
+      const double best = std::sqrt(6.25 * (double)depth_of_dataflow * ((double)chunk_bytes / 1024.0) / (double)ntbs);
+      const int64_t most = std::max<int64_t>(1, std::min<int64_t>(std::max(finest, to_fill), (int64_t)(chunk_bytes / 512)));
+      // a power of two (small chunks divide evenly only by those): the nearest one, not above `most`
+      slices = 1;
+      while (slices * 2 <= most && (double)(slices * 2) <= best * 1.41421356) slices *= 2;
       // hosting many contexts per workgroup is cheap, but polling them is not free: keep it to ~32
       const int64_t comfortable = std::max<int64_t>(1, ((int64_t)2 * num_cus * 32) / ntbs);
       slices = std::min(slices, comfortable);
