@@ -191,3 +191,19 @@ def test_protocol_choice(mscclx_lib):
     with pytest.raises(MscclxError) as e:
         p.configure(64 << 10, "float32", max_workgroups=2048, protocol=7)
     assert e.value.code == binding.ERR_INVALID_ARG
+
+
+def test_geometry_of_the_benchmark_workloads(mscclx_lib):
+    """The automatic geometry of the five benchmark workloads on a 256-CU part, as measured best on
+    MI355X: (workgroups, threads, slices, piece bytes, passes, most contexts on a workgroup)."""
+    from msccl.executor.workloads import WORKLOADS
+    want = {
+        "c1": (256, 64, 32, 4096, 1, 1),        # latency bound: few workgroups of one wave, 4 KiB pieces
+        "c2": (512, 512, 64, 131072, 1, 4),     # a ring is always busy: 4 contexts per workgroup, one pass
+        "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
+        "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
+        "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed
+    }
+    for key, w in WORKLOADS.items():
+        i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
+        assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
