@@ -46,9 +46,15 @@ class Executor:
 
     # -- geometry ---------------------------------------------------------------------------------
     def setup(self, chunk_bytes, dtype, redop="sum", **knobs):
-        """Fix chunk size / element type / reduction and allocate scratch + workspace."""
+        """Fix chunk size / element type / reduction and allocate scratch + workspace.
+
+        protocol="ir" follows the algorithm's own `proto` attribute (msccl/language/ir.py:322):
+        LL and LL128 run as flag-in-data lines, Simple as counters.  The default ignores the
+        attribute and lets the library choose, as the attribute is a hint about another machine."""
         if not torch.cuda.is_available():
             raise RuntimeError("the MSCCL-IR executor needs a GPU; there is no CPU path")
+        if knobs.get("protocol") == "ir":
+            knobs = dict(knobs, protocol="ll" if self.tables.proto.upper().startswith("LL") else "simple")
         self.dtype = dtype_name(dtype)
         self.chunk_bytes = int(chunk_bytes)
         self._setup_args = (chunk_bytes, dtype, redop, dict(knobs))

@@ -338,3 +338,14 @@ def test_ll_launch_number_wraps(knobs):
                 got = ins[r].cpu().numpy().view(np.uint32)
                 assert np.array_equal(got, want), (k, r, int(np.flatnonzero(got != want)[0]))
     ex.wait()
+
+
+def test_protocol_from_the_ir():
+    """protocol="ir": the <algo proto=...> attribute picks the protocol (LL, LL128 -> lines)."""
+    xml = ir_samples.ring_allreduce_xml(4)
+    for proto, want in (("Simple", 1), ("LL", 2), ("LL128", 2)):
+        doc = xml.replace('proto="Simple"', f'proto="{proto}"')
+        assert f'proto="{proto}"' in doc
+        got, ref, _, info = run_both(doc, 2048, "float32", protocol="ir")
+        assert info.protocol == want
+        assert_same(got, ref)
