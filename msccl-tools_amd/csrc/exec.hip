@@ -699,8 +699,8 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   const uint32_t epoch = (uint32_t)launch_no & 0x3ffu;
   {
     const u64 parity = launch_no & 1ull;
-    p.sync_cur = p.sync_base + kSyncHeaderWords + parity * p.sync_words;
-    p.sync_nxt = p.sync_base + kSyncHeaderWords + (parity ^ 1ull) * p.sync_words;
+    p.sync_cur = p.sync_base + kControlWords + parity * p.sync_words;
+    p.sync_nxt = p.sync_base + kControlWords + (parity ^ 1ull) * p.sync_words;
   }
   __shared__ int sh_choice;
   __shared__ Move sh_move;
@@ -844,11 +844,18 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   }
   }  // hosted contexts
   if (threadIdx.x == 0) {
-    // the last workgroup out re-arms the control block: next launch uses the other counter area
-    const u64 finished = __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (finished == (u64)gridDim.x - 1) {
-      publish(p.sync_base + 1, 0);
-      publish(p.sync_base, launch_no + 1);
+    // The last workgroup out re-arms the control block: the next launch uses the other counter area.
+    // "Last" is found group by group (the last of a group reports for the group), so that no
+    // address sees more than a few dozen atomics.
+    const unsigned per = p.finish_group, group = blockIdx.x / per, groups = (gridDim.x + per - 1) / per;
+    const unsigned members = group + 1 < groups ? per : gridDim.x - group * per;
+    u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
+    if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
+      publish(group_count, 0);
+      if (__hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
+        publish(p.sync_base + 1, 0);
+        publish(p.sync_base, launch_no + 1);
+      }
     }
   }
 #ifdef MSCCLX_PROFILE
@@ -1136,6 +1143,12 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
   kp.timeout_ticks = (uint64_t)plan->timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
   kp.slice_grain = g.slice_grain;
+  {  // groups of about sqrt(workgroups), at most kFinishGroups of them
+    uint32_t per = 1;
+    while ((uint64_t)per * per < (uint64_t)g.workgroups) ++per;
+    per = std::max<uint32_t>(per, ((uint32_t)g.workgroups + kFinishGroups - 1) / kFinishGroups);
+    kp.finish_group = per;
+  }
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan->tbs.size(); kp.nconns = (int)plan->conns.size();
   kp.wg_begin = d->hosting;
   kp.ctx_tb = d->hosting + g.wg_begin.size();

@@ -534,9 +534,9 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       //   a * contexts + depth * (h0 + b * piece bytes)
       // -- a fixed cost per workgroup launched, and one hand-off plus one small move for every step
       // on the longest chain of the program's dataflow.  More slices shrink the pieces but add
-      // workgroups; the minimum is at slices = sqrt(b/a * depth * chunk / threadblocks).  Fitted on
-      // MI355X with workgroups of one wave: a = 16 ns per workgroup, b = 100 ns per KiB, which puts
-      // an 8-rank ring on 1 MiB at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.
+      // workgroups; the minimum is at slices = sqrt(b/a * depth * chunk / threadblocks).  With
+      // b/a = 6.25 per KiB (fitted on MI355X, workgroups of one wave) an 8-rank ring on 1 MiB comes
+      // out at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.
       // Never finer than a context or two per compute unit, nor pieces below 512 bytes.
       int32_t depth_of_dataflow = 1;
       (void)waiting_ratio(plan, &depth_of_dataflow);
@@ -677,7 +677,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.slice_fifo_units = slot_chunks * g.piece_units;
   g.sync_slice_words = (uint64_t)(plan.tbs.size() + 2 * plan.conns.size()) * kSyncStrideWords;
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
-  const uint64_t sync_bytes = ((kSyncHeaderWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
+  const uint64_t sync_bytes = ((kControlWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
   g.fifo_byte_off = sync_bytes;
   {  // the kernel keeps slot positions as 32-bit offsets (16-byte steps on the vector path, bytes otherwise) and counter positions as 32-bit word indices
     const uint64_t fifo_bytes = g.slice_fifo_units * g.slices * fifo_unit_bytes;

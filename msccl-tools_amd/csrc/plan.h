@@ -101,7 +101,7 @@ struct KernelParams {
   const DevTb* tbs;
   const DevOp* ops;
   const DevConn* conns;
-  unsigned long long* sync_base; // control block: word 0 = launches finished so far (its parity picks the counter area), word 1 = workgroups finished
+  unsigned long long* sync_base; // control block (kControlWords): word 0 = launches finished so far (its parity picks the counter area)
   unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
   unsigned long long* sync_nxt;  // next launch's counters   } from the control block
   unsigned char* fifo;
@@ -114,6 +114,7 @@ struct KernelParams {
   uint64_t timeout_ticks;
   uint32_t piece_units;
   uint32_t slice_grain;
+  uint32_t finish_group;        // workgroups per group of the end-of-launch count
   int32_t slices, depth, ntbs, nconns;
   const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
   const int32_t* ctx_tb;        // hosted contexts, grouped by workgroup: threadblock row ...
@@ -136,6 +137,14 @@ MSCCLX_HOST_DEVICE inline uint64_t slice_begin(uint64_t chunk_units, uint32_t gr
 constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
+// The control block in front of the two counter areas: word 0 = launches finished so far, word 1 =
+// groups of workgroups finished, then one counter per group of workgroups (each alone in 128 bytes).
+// Workgroups report the end of a launch group by group: one counter for all of them would put one
+// returning atomic per workgroup on a single address at the end of every launch (measured 10 ns
+// each: 5 us of a 512-workgroup launch).
+constexpr int kFinishGroups = 64;
+constexpr int kFinishStrideWords = 16;
+constexpr int kControlWords = 8 + kFinishGroups * kFinishStrideWords;
 
 struct DeviceState;  // defined in exec.hip
 
