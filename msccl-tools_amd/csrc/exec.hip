@@ -1,35 +1,5 @@
-// MI355X (gfx950) executor kernels for MSCCL-IR and the device half of the C ABI.
-//
-// Execution model.  All ranks of the algorithm are virtual ranks whose buffers live in this GPU's
-// HBM.  The program is run as `slices` independent copies, copy j on the j-th 1/slices part of
-// EVERY chunk -- legal because every IR step is element-wise -- each with its own FIFOs and counters.
-// A context is one <tb> in one slice; it walks its step list once per "pass", a pass moving one piece
-// (piece_units) of each chunk its steps name.  Contexts are spread over a fixed number of resident
-// workgroups; a workgroup hosts up to 64 of them, polls what all of them wait for in one round of
-// loads (one lane of wave 0 per context), and runs whichever is ready, so it never blocks on one
-// context and the number of threadblocks is not tied to what fits on the chip.
-//
-// Synchronisation (all counters monotone, 64-bit, one per 64 bytes, agent scope, per slice):
-//   flag[tb]   = pass*nsteps + step + 1 of the last finished step with hasdep=1     (depid/deps wait)
-//   head[conn] = messages produced;  tail[conn] = messages consumed                  (FIFO hand-off)
-// Payload is read and written with device-scope (sc1) accesses only, so a producer publishes by
-// waiting for its stores to be acknowledged, a workgroup barrier, and a counter store; a consumer
-// reads the payload after its poll succeeds.  No cache-wide write-back or invalidate is issued.
-// A receiver reads a payload where the sender keeps it when the plan proved that safe; only the
-// other messages are copied through FIFO slots in HBM.
-// Two counter areas alternate between launches: a launch clears the area the next launch will
-// use, so no memset sits between launches.
-//
-// LL variant (flag-in-data, for small pieces): every message is written into its FIFO slot as 16-byte
-// lines {d0, flag, d1, flag}, two lines per 16 bytes of payload.  The flag names the launch and the
-// message, so a receiver needs no counter: its threads load the lines and retry the ones whose flags
-// do not match yet.  The sender's "stores acknowledged -> barrier -> counter store" and the receiver's
-// counter poll drop out of the hand-off.  Each 8-byte half of a line carries its own flag, so the
-// scheme only relies on 8-byte accesses being indivisible.  Free slots are still granted through the
-// tail counters.
-//
-// A workgroup that makes no progress for the watchdog period raises the area's abort word; all
-// other workgroups see it while they poll, and every wave leaves the kernel.
+// Host half of the C ABI of the MI355X executor for MSCCL-IR: configure, bind, launch, wait.
+// The kernels live in exec_device.h / exec_kernels.hip.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -43,9 +13,6 @@
 
 namespace mscclx {
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned long long u64;
-
 #define HIP_TRY(expr)                                                                              \
   do {                                                                                             \
     hipError_t e_ = (expr);                                                                        \
@@ -54,852 +21,22 @@ typedef unsigned long long u64;
   } while (0)
 
 // ------------------------------------------------------------------------------------------------
-// element-wise reducers.  Reducer<DT, OP>::combine<S>(a, b) reduces two storage words of type S
-// (one element of 1/2/4/8 bytes, or 16 bytes of elements) element by element.
-// ------------------------------------------------------------------------------------------------
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-
-template <int OP, typename T>
-__device__ __forceinline__ T red_int(T a, T b) {
-  if (OP == MSCCLX_SUM) return (T)(a + b);
-  if (OP == MSCCLX_PROD) return (T)(a * b);
-  if (OP == MSCCLX_MAX) return a > b ? a : b;
-  return a < b ? a : b;
-}
-template <int OP>
-__device__ __forceinline__ float red_float(float a, float b) {
-  if (OP == MSCCLX_SUM) return a + b;
-  if (OP == MSCCLX_PROD) return a * b;
-  if (OP == MSCCLX_MAX) return fmaxf(a, b);
-  return fminf(a, b);
-}
-template <int OP>
-__device__ __forceinline__ double red_double(double a, double b) {
-  if (OP == MSCCLX_SUM) return a + b;
-  if (OP == MSCCLX_PROD) return a * b;
-  if (OP == MSCCLX_MAX) return fmax(a, b);
-  return fmin(a, b);
-}
-
-__device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
-__device__ __forceinline__ unsigned short f32_to_bf16(float f) {  // round to nearest even, quiet NaN
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x0040u);
-  return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
-__device__ __forceinline__ float f16_to_f32(unsigned short h) { return (float)__builtin_bit_cast(_Float16, h); }
-__device__ __forceinline__ unsigned short f32_to_f16(float f) { return __builtin_bit_cast(unsigned short, (_Float16)f); }
-
-// Element arithmetic per dtype on raw element storage E (unsigned type of the element's size).
-// 16-bit floats: widen to fp32, operate, round to nearest even once.  For sum this equals the
-// correctly rounded 16-bit result (24 >= 2p+2 for p = 11 and p = 8); products of two 16-bit values
-// are exact in fp32, so they too are rounded once.
-template <int DT, int OP> struct ElemOp;
-#define MSCCLX_INT_ELEM(DT, T, E)                                                                  \
-  template <int OP> struct ElemOp<DT, OP> {                                                        \
-    typedef E store;                                                                               \
-    static __device__ __forceinline__ E op(E a, E b) { return (E)red_int<OP, T>((T)a, (T)b); }     \
-  };
-MSCCLX_INT_ELEM(MSCCLX_U8, unsigned char, unsigned char)
-MSCCLX_INT_ELEM(MSCCLX_I8, signed char, unsigned char)
-MSCCLX_INT_ELEM(MSCCLX_I32, int, unsigned int)
-MSCCLX_INT_ELEM(MSCCLX_U32, unsigned int, unsigned int)
-MSCCLX_INT_ELEM(MSCCLX_I64, long long, unsigned long long)
-MSCCLX_INT_ELEM(MSCCLX_U64, unsigned long long, unsigned long long)
-template <int OP> struct ElemOp<MSCCLX_F16, OP> {
-  typedef unsigned short store;
-  static __device__ __forceinline__ unsigned short op(unsigned short a, unsigned short b) { return f32_to_f16(red_float<OP>(f16_to_f32(a), f16_to_f32(b))); }
-};
-template <int OP> struct ElemOp<MSCCLX_BF16, OP> {
-  typedef unsigned short store;
-  static __device__ __forceinline__ unsigned short op(unsigned short a, unsigned short b) { return f32_to_bf16(red_float<OP>(bf16_to_f32(a), bf16_to_f32(b))); }
-};
-template <int OP> struct ElemOp<MSCCLX_F32, OP> {
-  typedef unsigned int store;
-  static __device__ __forceinline__ unsigned int op(unsigned int a, unsigned int b) { return __float_as_uint(red_float<OP>(__uint_as_float(a), __uint_as_float(b))); }
-};
-template <int OP> struct ElemOp<MSCCLX_F64, OP> {
-  typedef unsigned long long store;
-  static __device__ __forceinline__ unsigned long long op(unsigned long long a, unsigned long long b) {
-    return __builtin_bit_cast(unsigned long long, red_double<OP>(__builtin_bit_cast(double, a), __builtin_bit_cast(double, b)));
-  }
-};
-
-template <int DT, int OP> struct Reducer {
-  typedef ElemOp<DT, OP> E;
-  typedef typename E::store store;
-  static constexpr int kElemBytes = sizeof(store);
-  // 16 bytes of elements
-  static __device__ __forceinline__ u32x4 combine(u32x4 a, u32x4 b) {
-    typedef store vt __attribute__((ext_vector_type(16 / sizeof(store))));
-    vt x = __builtin_bit_cast(vt, a), y = __builtin_bit_cast(vt, b), r;
-#pragma unroll
-    for (int i = 0; i < (int)(16 / sizeof(store)); ++i) r[i] = E::op(x[i], y[i]);
-    return __builtin_bit_cast(u32x4, r);
-  }
-  // one element held in the word a buffer access of its size returns
-  static __device__ __forceinline__ unsigned char combine(unsigned char a, unsigned char b) { return (unsigned char)E::op((store)a, (store)b); }
-  static __device__ __forceinline__ unsigned short combine(unsigned short a, unsigned short b) { return (unsigned short)E::op((store)a, (store)b); }
-  static __device__ __forceinline__ unsigned int combine(unsigned int a, unsigned int b) { return (unsigned int)E::op((store)a, (store)b); }
-  static __device__ __forceinline__ u32x2 combine(u32x2 a, u32x2 b) {
-    return __builtin_bit_cast(u32x2, (unsigned long long)E::op((store)__builtin_bit_cast(unsigned long long, a), (store)__builtin_bit_cast(unsigned long long, b)));
-  }
-};
-
-// ------------------------------------------------------------------------------------------------
-// memory access.  Every load and store of payload goes through a raw buffer descriptor with the
-// device-scope cache policy (sc1): stores are written through this XCD's L2 and loads do not hit
-// lines the L2 may hold from before, so data handed from one workgroup to another (possibly on
-// another XCD, with its own L2) needs no cache-wide write-back or invalidate -- only
-// "my stores are acknowledged" (s_waitcnt vmcnt(0)) before the counter that announces them.
-// The descriptor also bounds every access: lanes past the end of a piece load 0 and store nothing.
-// ------------------------------------------------------------------------------------------------
-#ifndef MSCCLX_AUX
-#define MSCCLX_AUX 16 /* sc1 = device scope */
-#endif
-// Loads are marked non-temporal: every payload byte is read exactly once by the step that loads it.
-// Stores stay cacheable (a peer or a later step reads most of them soon, and the memory-side cache
-// then serves that read) except the ones the plan proved are never read again.
-#ifndef MSCCLX_AUX_LD
-#define MSCCLX_AUX_LD (MSCCLX_AUX | 2)
-#endif
-#ifndef MSCCLX_AUX_ST
-#define MSCCLX_AUX_ST MSCCLX_AUX
-#endif
-#ifndef MSCCLX_AUX_ST_FINAL
-#define MSCCLX_AUX_ST_FINAL (MSCCLX_AUX | 2)
-#endif
-constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family dword 3)
-
-template <int W> struct Access;
-template <> struct Access<16> {
-  typedef u32x4 word;
-  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, AUX); }
-  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, AUX); }
-};
-template <> struct Access<8> {
-  typedef u32x2 word;
-  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, AUX); }
-  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, AUX); }
-};
-template <> struct Access<4> {
-  typedef unsigned int word;
-  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, AUX); }
-  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, AUX); }
-};
-template <> struct Access<2> {
-  typedef unsigned short word;
-  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, AUX); }
-  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b16(v, r, off, 0, AUX); }
-};
-template <> struct Access<1> {
-  typedef unsigned char word;
-  template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b8(r, off, 0, AUX); }
-  template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b8(v, r, off, 0, AUX); }
-};
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kBufferFlags);
-}
-
-#ifndef MSCCLX_UNROLL
-#define MSCCLX_UNROLL 8
-#endif
-constexpr int kUnroll = MSCCLX_UNROLL;
-
-// out1[, out2] = a [(+) b] over n units of W bytes.
-template <class R, int W, bool HAS_B, bool HAS_O2, bool NT1>
-__device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n) {
-  typedef Access<W> A;
-  typedef typename A::word word;
-  constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const uint32_t bytes = n * W;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
-  const uint32_t T = blockDim.x;
-  // kUnroll loads are in flight per thread either way: all of a, or half of a and half of b
-  constexpr int UA = HAS_B ? (kUnroll / 2 > 0 ? kUnroll / 2 : 1) : kUnroll;
-  for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
-    word x[UA], y[UA];
-#pragma unroll
-    for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * W));
-    if (HAS_B) {
-#pragma unroll
-      for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * W));
-#pragma unroll
-      for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < UA; ++u) A::template st<X1>(r1, (int)((i + u * T) * W), x[u]);
-    if (HAS_O2) {
-#pragma unroll
-      for (int u = 0; u < UA; ++u) A::template st<XS>(r2, (int)((i + u * T) * W), x[u]);
-    }
-  }
-}
-
-// rows x n units.  Consecutive rows of an operand are `stride_*` units apart: a chunk for rank
-// buffers, n for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
-// buffer, o2 (the forwarded copy) always a FIFO slot.
-template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool NT1 = false>
-__device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
-                                          const unsigned char* b, uint64_t stride_b, int rows, uint32_t n) {
-  constexpr int W = VEC ? 16 : R::kElemBytes;
-  for (int r = 0; r < rows; ++r)
-    move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
-                                    a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
-}
-
-// ------------------------------------------------------------------------------------------------
-// the executor kernel
-// ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ u64 load_counter(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-
-__device__ __forceinline__ u64 first_lane(u64 v) {  // the first lane's value, as a value the compiler knows to be the same in all lanes
-  return ((u64)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) | (u64)__builtin_amdgcn_readfirstlane((uint32_t)v);
-}
-
-__device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
-__device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
-
-// ------------------------------------------------------------------------------------------------
-// LL lines.  One unit (16 payload bytes d0..d3) occupies 32 bytes of a slot: {d0,f,d1,f}{d2,f,d3,f}.
-// f = launch number (10 bits) | message number + 1 (22 bits): never 0, so a cleared slot matches
-// nothing, and what an earlier message or launch left in a line cannot be taken for this message.
-// ------------------------------------------------------------------------------------------------
-constexpr int kLLUnitBytes = 32;
-__device__ __forceinline__ uint32_t ll_flag(uint32_t epoch, u64 seq) { return ((epoch & 0x3ffu) << 22) | (uint32_t)((seq + 1) & 0x3fffffu); }
-__device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { return l0.y == f && l0.w == f && l1.y == f && l1.w == f; }
-
-// What a thread needs to give up on a message that never arrives.
-struct LLWatch {
-  u64* abort_word;
-  mscclx_status* host_status;
-  u64 timeout_ticks;
-  int tb, step, slice;
-  u64 pass;
-};
-
-// (arguments by value: a struct handed to a function that is not inlined would have to live in memory)
-__device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int tb, int step, int slice, u64 pass) {
-  if (atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
-    hs->tb = tb; hs->step = step; hs->slice = slice; hs->pass = (int64_t)pass; hs->waiting_on = 1;
-    __threadfence_system();
-    __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-  }
-}
-
-// o1 (rank buffer) [and llo (LL slot)] = a [(+) b] over n units of 16 bytes.  a is an LL slot row when
-// IN_LL (its lines are retried until they carry `fin`), a rank buffer otherwise; b is a rank buffer.
-template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1>
-__device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* llo, const unsigned char* a, const unsigned char* b, uint32_t n,
-                                              uint32_t fin, uint32_t fout, const LLWatch& watch) {
-  typedef Access<16> A;
-  // XV: the retried loads must really be issued again each time round the loop (bit 31 = volatile, for the compiler only)
-  constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, XV = (int)(0x80000000u | MSCCLX_AUX), X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, n * (IN_LL ? kLLUnitBytes : 16));
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, n * (HAS_B ? 16 : (IN_LL ? kLLUnitBytes : 16)));
-  const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? n * 16 : 0);
-  const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * kLLUnitBytes : 0);
-  const uint32_t T = blockDim.x;
-  constexpr int UA = 2;  // small pieces: few lines per thread, few registers
-  for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
-    u32x4 x[UA], y[UA];
-    if (IN_LL) {
-      static_assert(UA == 2, "the retry below names its two units");
-      const uint32_t ia = i, ib = i + T;
-      u32x4 a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)), a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16));
-      u32x4 b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)), b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16));
-      if (HAS_B) {
-#pragma unroll
-        for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
-      }
-      unsigned spins = 0;
-      u64 since = 0;
-      for (;;) {
-        const bool ok_a = ll_valid(a0, a1, fin), ok_b = ib >= n || ll_valid(b0, b1, fin);
-        if (ok_a && ok_b) break;
-        if (!ok_a) { a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)); a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16)); }
-        if (!ok_b) { b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)); b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16)); }
-        if ((++spins & 0x7fu) == 0) {
-          const u64 now = wall_clock64();
-          if (!since) since = now;
-          const bool expired = now - since > watch.timeout_ticks;
-          if (expired) ll_give_up(watch.abort_word, watch.host_status, watch.tb, watch.step, watch.slice, watch.pass);
-          if (expired || load_counter(watch.abort_word) != 0) break;  // the launch is lost; leave with what is there
-        }
-      }
-      x[0] = u32x4{a0.x, a0.z, a1.x, a1.z};
-      x[1] = u32x4{b0.x, b0.z, b1.x, b1.z};
-    } else {
-#pragma unroll
-      for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * 16));
-      if (HAS_B) {
-#pragma unroll
-        for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
-      }
-    }
-    if (HAS_B) {
-#pragma unroll
-      for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
-    }
-    if (OUT_LL) {  // the forwarded lines first: the next rank is waiting for them
-#pragma unroll
-      for (int u = 0; u < UA; ++u) {
-        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes), u32x4{x[u].x, fout, x[u].y, fout});
-        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
-      }
-    }
-    if (HAS_O1) {
-#pragma unroll
-      for (int u = 0; u < UA; ++u) A::template st<X1>(r1, (int)((i + u * T) * 16), x[u]);
-    }
-  }
-}
-
-// rows x n units; rank-buffer rows are `stride_*` units apart, slot rows are packed.
-template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1 = false>
-__device__ __forceinline__ void move_rows_ll(unsigned char* o1, uint64_t stride_o1, unsigned char* llo, const unsigned char* a, uint64_t stride_a,
-                                             const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t fin, uint32_t fout,
-                                             const LLWatch& watch) {
-  for (int r = 0; r < rows; ++r)
-    move_units_ll<R, IN_LL, HAS_B, HAS_O1, OUT_LL, NT1>(HAS_O1 ? o1 + (uint64_t)r * stride_o1 * 16 : nullptr,
-                                                       OUT_LL ? llo + (uint64_t)r * n * kLLUnitBytes : nullptr,
-                                                       a + (uint64_t)r * (IN_LL ? (uint64_t)n * kLLUnitBytes : stride_a * 16),
-                                                       HAS_B ? b + (uint64_t)r * stride_b * 16 : nullptr, n, fin, fout, watch);
-}
-
-// What the workgroup does for one step of one context: operands as byte addresses, filled in by the
-// context's lane when the context arrives at the step and handed to the other threads through LDS.
-struct Move {
-  u64 a;      // source: the incoming payload (slot, or the sender's buffer) or the local source
-  u64 dst;    // local destination, which is also the local operand of a reduction
-  u64 out;    // slot to fill
-  uint32_t n; // units per row
-  int rows, kind;
-};
-// kind: how the operands are used.  Rows of a rank buffer are a chunk apart, rows in a slot are packed.
-enum {
-  kHasB = 1,     // reduce: a (+) dst
-  kHasO2 = 2,    // also forward the result into `out`
-  kNt1 = 4,      // the first destination is never read again
-  kLLKind = 8,   // flag-in-data lines: bits 0-2 then say which movement (kLL* below)
-  kAPacked = 16, // a is a slot
-  kToSlot = 32,  // the first (only) destination is `out` instead of dst
-};
-enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
-
-// One hosted context = (threadblock, slice), run by one lane of wave 0.  What never changes while it
-// runs sits in LDS (one entry per lane, touched by that lane only), so that it occupies no registers
-// while the workgroup moves data; what changes from step to step is the lane's Context.
-struct Hosted {
-  int nops, op_begin;
-  unsigned npasses;
-  // Slots: offsets from the start of the FIFO region, in 16-byte steps on the vector path and in bytes otherwise; counters: 64-bit word index
-  // inside this launch's counter area.  32 bits each, so that the lot is read from LDS in one go.
-  uint32_t in_slots, out_slots;    // first slot of the incoming / outgoing connection, in this slice
-  uint32_t in_slot_bytes, out_slot_bytes;
-  uint32_t in_wrap, out_wrap;      // depth * slot bytes: where the ring of slots starts over
-  uint32_t flags;                  // flag of threadblock t of this slice is flags + t * kSyncStrideWords
-  uint32_t my_flag;
-  uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
-  uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
-  int tb, slice;                   // for the watchdog's report only
-};
-
-__device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int slice) {
-  return base + kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words;
-}
-
-// The changing part.  Everything that depends on the pass or on how many messages went by is kept
-// as a running value, advanced when a step finishes: the lane's instructions between two moves are
-// on the critical path of a latency-bound program, and multiplications and divisions dominate them.
-struct Context {
-  int step;
-  unsigned pass;
-  bool active;
-  uint32_t count;           // steps finished so far in this launch (all passes)
-  uint32_t sseq, rseq;      // messages sent / received so far = number of the next message on its connection
-  uint32_t sslot, rslot;    // byte offset of that message's slot inside the connection's ring
-  uint32_t left;            // units of the slice not yet covered before this pass
-  u64 off;                  // byte offset of this pass's piece inside any chunk
-  // the step the context stands at
-  bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
-  int type, hasdep;
-  const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
-  uint32_t t0, t1, t2;      // ... until they reach these values (every counter of a launch stays below 2^32)
-  Move m;
-};
-
-// Describe the step `c` stands at: what it must wait for, whether it moves data, and from where to
-// where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
-// last 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order,
-// so this is a hint that the message is about to be complete; the threads that read it check every line.
-template <bool VEC, bool LL>
-__device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const KernelParams& p, uint32_t epoch, const DevOp& op) {
-  const int t = (int)(op.word & 15u);
-  const int cnt = (int)(op.word >> kOpCntShift);
-  const bool out_staged = op.word & kOpOutStaged, in_place = op.word & kOpInPlace;
-  c.type = t;
-  c.hasdep = (op.word & kOpHasdep) ? 1 : 0;
-  const bool rcv = is_recv(t), snd = is_send(t);
-  c.w0 = c.w1 = c.w2 = nullptr;
-  c.t0 = c.t1 = c.t2 = 0;
-  if (op.dep_tb >= 0) { c.w0 = p.sync_cur + (h.flags + (uint32_t)op.dep_tb * kSyncStrideWords); c.t0 = c.pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1; }
-  if (snd && c.sseq >= (uint32_t)p.depth) { c.w2 = p.sync_cur + h.tail_in; c.t2 = c.sseq + 1 - (uint32_t)p.depth; }
-  c.moves = !(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !out_staged));
-
-  const uint32_t n = c.left < p.piece_units ? c.left : p.piece_units;
-  // out: the slot to fill, or 0 when the receiver will read this step's payload in place
-  const u64 out = (snd && out_staged) ? (u64)p.fifo + (u64)h.out_slots * (VEC ? 16 : 1) + c.sslot : 0;
-  // in: the incoming payload -- packed in a slot, or still where the sender has it (then its rows are
-  // a chunk apart, like any rank buffer)
-  u64 in = 0;
-  int in_packed = kAPacked;
-  if (rcv) {
-    if (in_place) { in = op.in_addr + c.off; in_packed = 0; }
-    else in = (u64)p.fifo + (u64)h.in_slots * (VEC ? 16 : 1) + c.rslot;
-    if (LL) {
-      c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
-      c.t1 = ll_flag(epoch, c.rseq);
-    } else {
-      c.w1 = p.sync_cur + h.head_in;
-      c.t1 = c.rseq + 1;
-    }
-  }
-  Move& m = c.m;
-  m.n = n; m.rows = cnt;
-  m.a = in; m.dst = op.dst_addr + c.off; m.out = out;
-  const int nt = (op.word & kOpNtStore) ? kNt1 : 0;
-  int kind = 0;
-  switch (t) {
-    case MSCCLX_OP_SEND: m.a = op.src_addr + c.off; kind = LL ? kLLKind | kLLSend : (int)kToSlot; break;
-    case MSCCLX_OP_RECV: kind = LL ? kLLKind | (nt ? kLLRecvNt : kLLRecv) : in_packed | nt; break;
-    case MSCCLX_OP_RCS: kind = LL ? kLLKind | kLLRcs : in_packed | (out ? (int)kHasO2 : 0); break;
-    case MSCCLX_OP_RRC: kind = LL ? kLLKind | kLLRrc : in_packed | kHasB; break;
-    case MSCCLX_OP_RRS: kind = LL ? kLLKind | kLLRrs : in_packed | kHasB | kToSlot; break;
-    case MSCCLX_OP_RRCS: kind = LL ? kLLKind | kLLRrcs : in_packed | kHasB | (out ? (int)kHasO2 : 0); break;
-    case MSCCLX_OP_COPY: m.a = op.src_addr + c.off; kind = nt; break;
-    case MSCCLX_OP_REDUCE: m.a = op.src_addr + c.off; kind = kHasB; break;
-    default: break;
-  }
-  m.kind = kind;
-}
-
-// The description of the step after the one `c` stands at.  It is fetched before the counters of
-// the finished step are stored: a load issued after those stores would come back only after they
-// are acknowledged, and the context could not look for its next message any earlier.
-__device__ __forceinline__ DevOp fetch_next_op(const Context& c, const Hosted& h, const KernelParams& p) {
-  const int next = c.step + 1 == h.nops ? 0 : c.step + 1;
-  return p.ops[h.op_begin + next];
-}
-
-// Announce the completed step and move the context to its next one, described by `next`.
-// `writer`: this thread stores the counters (the context's lane; one thread of a wave that runs a
-// context with all its lanes).
-template <int UB, bool LL>
-__device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next, bool writer = true) {
-  const Hosted h = entry;  // one batch of LDS reads, one wait -- not one wait per field as they are needed
-  if (is_send(c.type)) {
-    if (!LL && writer) publish(p.sync_cur + h.head_out, (u64)c.sseq + 1);  // LL: the lines announce themselves
-    ++c.sseq;
-    c.sslot += h.out_slot_bytes;
-    if (c.sslot == h.out_wrap) c.sslot = 0;
-  }
-  if (is_recv(c.type)) {
-    if (writer) publish(p.sync_cur + h.tail_out, (u64)c.rseq + 1);
-    ++c.rseq;
-    c.rslot += h.in_slot_bytes;
-    if (c.rslot == h.in_wrap) c.rslot = 0;
-  }
-  ++c.count;
-  if (c.hasdep && writer) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * nops + step + 1
-  if (++c.step == h.nops) {
-    c.step = 0;
-    ++c.pass;
-    c.left -= c.left < p.piece_units ? c.left : p.piece_units;
-    c.off += (u64)p.piece_units * UB;
-  }
-  if (c.pass >= h.npasses) c.active = false;
-  else describe_step<UB == 16, LL>(c, h, p, epoch, next);
-}
-
-// Set up the context (threadblock tbi, slice) : its constants in `h`, its state in `c`, standing at
-// its first step.  `writer` also clears, for the next launch, the counters this context alone writes.
-template <bool VEC, int EB, bool LL>
-__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int tbi, int slice, bool writer) {
-  constexpr uint64_t UB = VEC ? 16 : EB;
-  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;
-  h.tb = tbi;
-  h.slice = slice;
-  const DevTb tb = p.tbs[tbi];
-  h.nops = tb.nops; h.op_begin = tb.op_begin;
-  const uint64_t u0 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice), u1 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice + 1);
-  h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
-  const uint64_t slice_fifo = (uint64_t)slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
-  const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words);
-  const uint32_t heads = area + (uint32_t)p.ntbs * kSyncStrideWords, tails = heads + (uint32_t)p.nconns * kSyncStrideWords;
-  h.flags = area;
-  h.my_flag = area + (uint32_t)tbi * kSyncStrideWords;
-  h.in_slots = h.out_slots = 0; h.in_slot_bytes = h.out_slot_bytes = 0; h.in_wrap = h.out_wrap = 0;
-  h.head_in = h.tail_out = h.head_out = h.tail_in = 0;
-  if (tb.recv_conn >= 0) {
-    const DevConn cn = p.conns[tb.recv_conn];
-    h.in_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.in_slot_bytes = (uint32_t)(cn.slot_units * FB); h.in_wrap = h.in_slot_bytes * (uint32_t)p.depth;
-    h.head_in = heads + (uint32_t)tb.recv_conn * kSyncStrideWords; h.tail_out = tails + (uint32_t)tb.recv_conn * kSyncStrideWords;
-  }
-  if (tb.send_conn >= 0) {
-    const DevConn cn = p.conns[tb.send_conn];
-    h.out_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.out_slot_bytes = (uint32_t)(cn.slot_units * FB); h.out_wrap = h.out_slot_bytes * (uint32_t)p.depth;
-    h.head_out = heads + (uint32_t)tb.send_conn * kSyncStrideWords; h.tail_in = tails + (uint32_t)tb.send_conn * kSyncStrideWords;
-  }
-  c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
-  c.left = (uint32_t)(u1 - u0);
-  c.off = u0 * UB;
-  c.active = tb.nops > 0 && h.npasses > 0;
-  if (writer) {
-    u64* nxt = slice_area(p.sync_nxt, p, slice);
-    nxt[(uint64_t)tbi * kSyncStrideWords] = 0;
-    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
-    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
-  }
-  if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[tb.op_begin]);
-}
-
-// The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
-// incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool VEC, bool LL>
-__device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
-                                        int tb, int step, int slice, unsigned pass) {
-  const u64 cs = p.chunk_units;
-  unsigned char* const dst = (unsigned char*)m.dst;
-  unsigned char* const out = (unsigned char*)m.out;
-  const unsigned char* const a = (const unsigned char*)m.a;
-  if (LL && (m.kind & kLLKind)) {
-    const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
-    const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tb, step, slice, (u64)pass};
-    switch (m.kind & 7) {
-      case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-      default: break;
-    }
-  } else {
-    const u64 stride_a = (m.kind & kAPacked) ? (u64)m.n : cs;
-    unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
-    const u64 stride_o1 = (m.kind & kToSlot) ? (u64)m.n : cs;
-    switch (m.kind & 7) {
-      case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n); break;
-      case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n); break;
-      default: break;
-    }
-  }
-}
-
-// LL, one context on a workgroup of one wave: the wave runs the context with all its lanes.  Every
-// value of the bookkeeping is then the same in all lanes, so it lives in scalar registers and runs
-// on the scalar unit; there is no hand-over through LDS and no barrier, and the lanes go straight
-// from one message's lines to the next one's.  This is the shape of latency-bound programs (small
-// pieces, as many workgroups as contexts).  Measured on a 64-rank ring all-reduce of 2 KiB pieces it
-// takes 15% off the LL time; with the counter protocol it gains nothing (a hop is then bound by the
-// memory round trips of payload, acknowledgement and counter, not by instructions), so that
-// protocol always runs hosted.  Returns false if the launch was given up.
-template <class R, bool VEC, bool LL>
-__device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, int ctx, unsigned long long* prof4) {
-  constexpr int EB = R::kElemBytes;
-  constexpr int UB = VEC ? 16 : EB;
-  const bool writer = threadIdx.x == 0;
-  u64* const abort_word = p.sync_cur;
-  Hosted h;
-  Context c;
-  init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
-  while (c.active) {
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t0 = wall_clock64();
-#endif
-    {  // wait until the step may start.  LL: not for the message itself -- the lines are retried by the threads that read them
-      const bool watch1 = c.w1 && !LL;
-      unsigned spins = 0;
-      u64 deadline = 0;
-      bool armed = false;
-      for (;;) {
-        // one lane asks memory, the wave shares the answers
-        u64 l0 = 0, l1 = 0, l2 = 0;
-        if (writer) {
-          if (c.w0) l0 = load_counter(c.w0);
-          if (watch1) l1 = load_counter(c.w1);
-          if (c.w2) l2 = load_counter(c.w2);
-        }
-        const u64 v0 = first_lane(l0), v1 = first_lane(l1), v2 = first_lane(l2);
-        const int what = (c.w0 && v0 < c.t0) ? 0 : (watch1 && v1 < c.t1) ? 1 : (c.w2 && v2 < c.t2) ? 2 : -1;
-        if (what < 0) break;
-        __builtin_amdgcn_s_sleep(1);
-        if ((++spins & 0x3fu) == 0) {
-          const u64 now = wall_clock64();
-          if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
-          if (load_counter(abort_word) != 0) return false;
-          if (now > deadline) {
-            if (writer && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
-              mscclx_status* hs = p.host_status;
-              hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
-              __threadfence_system();
-              __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-            }
-            return false;
-          }
-        }
-      }
-    }
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t1 = wall_clock64();
-#endif
-    if (c.moves) do_move<R, VEC, LL>(c.m, p, epoch, c.rseq, c.sseq, h.tb, c.step, h.slice, c.pass);
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t2 = wall_clock64();
-#endif
-    const DevOp next = fetch_next_op(c, h, p);
-    if (c.moves) __builtin_amdgcn_s_waitcnt(0);  // this wave's stores are acknowledged: the counters may announce them
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t3 = wall_clock64();
-#endif
-    finish_step<UB, LL>(c, h, p, epoch, next, writer);
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t4 = wall_clock64();
-    prof4[0] += prof_t1 - prof_t0; prof4[1] += prof_t2 - prof_t1; prof4[2] += prof_t3 - prof_t2; prof4[3] += prof_t4 - prof_t3;
-#endif
-  }
-  return true;
-}
-
-// A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
-// active context waits for (one round of loads covers all of them), finishes steps that move no data
-// on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
-// reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
-// share the resident workgroups without deadlock.
-template <class R, bool VEC, bool LL>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
-  static_assert(VEC || !LL, "LL lines carry 16-byte units");
-  constexpr int EB = R::kElemBytes;
-  constexpr uint64_t UB = VEC ? 16 : EB;
-  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;  // bytes one unit takes inside a FIFO slot
-  // The number of launches so far is kept on the device (control word 0) and is advanced by the
-  // last workgroup to finish, so a launch carries no host-side state and the same launch can be
-  // replayed (stream order guarantees the next launch sees the new value).  Its lowest bit picks
-  // which of the two counter areas this launch uses; its low 10 bits mark the LL lines.
-  KernelParams p = launch_params;
-  const u64 launch_no = load_counter(p.sync_base);
-  const uint32_t epoch = (uint32_t)launch_no & 0x3ffu;
-  {
-    const u64 parity = launch_no & 1ull;
-    p.sync_cur = p.sync_base + kControlWords + parity * p.sync_words;
-    p.sync_nxt = p.sync_base + kControlWords + (parity ^ 1ull) * p.sync_words;
-  }
-  __shared__ int sh_choice;
-  __shared__ Move sh_move;
-  __shared__ uint32_t sh_seq[2];   // LL: numbers of the incoming and the outgoing message
-  __shared__ int sh_who[4];        // LL: threadblock, step, slice, pass of the chosen step, for the watchdog's report
-  u64* const abort_word = p.sync_cur;
-  const int lane = threadIdx.x;
-  const bool poller = threadIdx.x < 64;
-  const int ctx_begin = p.wg_begin[blockIdx.x], hosted = p.wg_begin[blockIdx.x + 1] - ctx_begin;
-  // LL, one hosted context: nothing else could run while it waits for a message, so the lane does not
-  // watch for it; the moving threads go straight to the lines and retry them until they are there.
-  const bool direct = LL && hosted == 1;
-
-  __shared__ Hosted sh_hosted[kMaxHosted];
-  Hosted& h = sh_hosted[lane & (kMaxHosted - 1)];  // this lane's entry; lanes of other waves never look at it
-  Context c;
-  c.active = false;
-#ifdef MSCCLX_PROFILE
-  u64 prof_wait = 0, prof_move = 0, prof_ack = 0, prof_fin = 0;
-  const u64 prof_start = wall_clock64();
-#endif
-  if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
-  if (LL && hosted == 1 && blockDim.x == 64) {
-    unsigned long long prof4[4] = {0, 0, 0, 0};
-    run_solo<R, VEC, LL>(p, epoch, ctx_begin, prof4);
-#ifdef MSCCLX_PROFILE
-    prof_wait = prof4[0]; prof_move = prof4[1]; prof_ack = prof4[2]; prof_fin = prof4[3];
-#endif
-  } else {
-  if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
-  int cursor = 0;
-
-  for (;;) {
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t0 = wall_clock64();
-#endif
-    if (poller) {
-      int choice = -2;
-      unsigned spins = 0;
-      // The watchdog period starts when this workgroup last made progress.  The clock is only read
-      // while nothing is ready, so a workgroup that keeps finding work never pays for it.
-      u64 deadline = 0;
-      bool armed = false;
-      while (choice == -2) {
-        bool ready = false;
-        if (c.active) {
-          // the (up to three) counters are loaded together: one round trip to memory, not one each
-          const bool watch1 = c.w1 && !direct;
-          const u64 v0 = c.w0 ? load_counter(c.w0) : 0;
-          const u64 v1 = watch1 ? load_counter(c.w1) : 0;
-          const u64 v2 = c.w2 ? load_counter(c.w2) : 0;
-          ready = (!c.w0 || v0 >= c.t0) && (!c.w2 || v2 >= c.t2) &&
-                  (!watch1 || (LL ? (uint32_t)(v1 >> 32) == (uint32_t)c.t1 : v1 >= c.t1));
-        }
-        bool progressed = false;
-        if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
-          const DevOp next = fetch_next_op(c, h, p);
-          finish_step<(int)UB, LL>(c, h, p, epoch, next);
-          progressed = true;
-          ready = false;  // the context now stands at another step, whose conditions are not yet known
-        }
-        const u64 movers = __ballot(ready && c.moves && c.active);
-        if (movers) {
-          const u64 from_cursor = movers & ~((cursor >= 64) ? ~0ull : ((1ull << cursor) - 1ull));
-          choice = __ffsll((long long)(from_cursor ? from_cursor : movers)) - 1;
-        } else if (!__any(c.active)) {
-          choice = -1;  // every hosted context has run to its end
-        } else if (__any(progressed)) {
-          armed = false;
-        } else {
-          __builtin_amdgcn_s_sleep(1);
-          if ((++spins & 0x3fu) == 0) {
-            const u64 now = wall_clock64();
-            if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
-            bool stop = false;
-            if (lane == 0) stop = load_counter(abort_word) != 0;
-            if (__any(stop)) { choice = -3; }
-            else if (now > deadline) {
-              // report the first context that is still waiting
-              const u64 stuck = __ballot(c.active);
-              const int who = __ffsll((long long)stuck) - 1;
-              if (lane == who && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
-                int what = 3;
-                if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
-                else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
-                else if (c.w2 && load_counter(c.w2) < c.t2) what = 2;
-                mscclx_status* hs = p.host_status;
-                hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
-                __threadfence_system();
-                __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-              }
-              choice = -3;
-            }
-          }
-        }
-      }
-      if (choice >= 0 && lane == choice) {
-        sh_move = c.m;
-        if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = h.tb; sh_who[1] = c.step; sh_who[2] = h.slice; sh_who[3] = (int)c.pass; }
-      }
-      if (lane == 0) sh_choice = choice;
-      cursor = choice >= 0 ? (choice + 1) & 63 : cursor;
-    }
-    __syncthreads();
-    const int choice = sh_choice;
-    if (choice < 0) break;  // done (-1) or giving up (-3); uniform for the workgroup
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t1 = wall_clock64();
-#endif
-
-    // ---- the chosen context's step: move one piece ----
-    {
-      const Move m = sh_move;
-      if (LL) do_move<R, VEC, LL>(m, p, epoch, sh_seq[0], sh_seq[1], sh_who[0], sh_who[1], sh_who[2], (unsigned)sh_who[3]);
-      else do_move<R, VEC, LL>(m, p, epoch, 0, 0, 0, 0, 0, 0);
-    }
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t2 = wall_clock64();
-#endif
-    // every wave waits until its own device-scope stores are acknowledged (the context's lane asks
-    // for its next step's description meanwhile); after the barrier that lane may announce the whole
-    // workgroup's data with plain counter stores
-    const bool mine = poller && lane == choice;
-    DevOp next;
-    if (mine) next = fetch_next_op(c, h, p);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t3 = wall_clock64();
-#endif
-    if (mine) finish_step<(int)UB, LL>(c, h, p, epoch, next);
-#ifdef MSCCLX_PROFILE
-    if (threadIdx.x == 0) {
-      const u64 prof_t4 = wall_clock64();
-      prof_wait += prof_t1 - prof_t0;
-      prof_move += prof_t2 - prof_t1;
-      prof_ack += prof_t3 - prof_t2;
-      prof_fin += prof_t4 - prof_t3;
-    }
-#endif
-  }
-  }  // hosted contexts
-  if (threadIdx.x == 0) {
-    // The last workgroup out re-arms the control block: the next launch uses the other counter area.
-    // "Last" is found group by group (the last of a group reports for the group), so that no
-    // address sees more than a few dozen atomics.
-    const unsigned per = p.finish_group, group = blockIdx.x / per, groups = (gridDim.x + per - 1) / per;
-    const unsigned members = group + 1 < groups ? per : gridDim.x - group * per;
-    u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
-    if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
-      publish(group_count, 0);
-      if (__hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
-        publish(p.sync_base + 1, 0);
-        publish(p.sync_base, launch_no + 1);
-      }
-    }
-  }
-#ifdef MSCCLX_PROFILE
-  if (threadIdx.x == 0 && p.prof) {
-    p.prof[(size_t)blockIdx.x * 8 + 0] = prof_wait;
-    p.prof[(size_t)blockIdx.x * 8 + 1] = prof_move;
-    p.prof[(size_t)blockIdx.x * 8 + 2] = wall_clock64() - prof_start;
-    p.prof[(size_t)blockIdx.x * 8 + 3] = prof_start;
-    p.prof[(size_t)blockIdx.x * 8 + 4] = prof_ack;
-    p.prof[(size_t)blockIdx.x * 8 + 5] = prof_fin;
-  }
-#endif
-}
-
-// ------------------------------------------------------------------------------------------------
 // host: kernel table, configure, bind, launch
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
-
-template <int DT, int OP> static kernel_fn pick_vec(bool vec, bool ll) {
-  if (ll) return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, true> : nullptr;
-  return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false> : (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false>;
-}
-template <int DT> static kernel_fn pick_op(int op, bool vec, bool ll) {
-  switch (op) {
-    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec, ll);
-    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec, ll);
-    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec, ll);
-    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec, ll);
-    default: return nullptr;
-  }
-}
+// The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
+kernel_fn pick_kernel_group_0(int dtype, int op, bool vec, bool ll);
+kernel_fn pick_kernel_group_1(int dtype, int op, bool vec, bool ll);
+kernel_fn pick_kernel_group_2(int dtype, int op, bool vec, bool ll);
+kernel_fn pick_kernel_group_3(int dtype, int op, bool vec, bool ll);
+kernel_fn pick_kernel_group_4(int dtype, int op, bool vec, bool ll);
 static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll) {
-  switch (dtype) {
-    case MSCCLX_U8: return pick_op<MSCCLX_U8>(op, vec, ll);
-    case MSCCLX_I8: return pick_op<MSCCLX_I8>(op, vec, ll);
-    case MSCCLX_I32: return pick_op<MSCCLX_I32>(op, vec, ll);
-    case MSCCLX_U32: return pick_op<MSCCLX_U32>(op, vec, ll);
-    case MSCCLX_I64: return pick_op<MSCCLX_I64>(op, vec, ll);
-    case MSCCLX_U64: return pick_op<MSCCLX_U64>(op, vec, ll);
-    case MSCCLX_F16: return pick_op<MSCCLX_F16>(op, vec, ll);
-    case MSCCLX_BF16: return pick_op<MSCCLX_BF16>(op, vec, ll);
-    case MSCCLX_F32: return pick_op<MSCCLX_F32>(op, vec, ll);
-    case MSCCLX_F64: return pick_op<MSCCLX_F64>(op, vec, ll);
+  switch (dtype / 2) {
+    case 0: return pick_kernel_group_0(dtype, op, vec, ll);
+    case 1: return pick_kernel_group_1(dtype, op, vec, ll);
+    case 2: return pick_kernel_group_2(dtype, op, vec, ll);
+    case 3: return pick_kernel_group_3(dtype, op, vec, ll);
+    case 4: return pick_kernel_group_4(dtype, op, vec, ll);
     default: return nullptr;
   }
 }

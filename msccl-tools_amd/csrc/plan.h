@@ -146,7 +146,7 @@ constexpr int kFinishGroups = 64;
 constexpr int kFinishStrideWords = 16;
 constexpr int kControlWords = 8 + kFinishGroups * kFinishStrideWords;
 
-struct DeviceState;  // defined in exec.hip
+struct DeviceState;  // defined in exec.hip (host half of the ABI)
 
 }  // namespace mscclx
 
