@@ -248,6 +248,9 @@ __device__ __forceinline__ u64 first_lane(u64 v) {  // the first lane's value, a
   return ((u64)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) | (u64)__builtin_amdgcn_readfirstlane((uint32_t)v);
 }
 
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int l) { return (uint32_t)__builtin_amdgcn_readlane((int)v, l); }  // l: the same in all lanes
+__device__ __forceinline__ u64 lane_value(u64 v, int l) { return ((u64)lane_value((uint32_t)(v >> 32), l) << 32) | (u64)lane_value((uint32_t)v, l); }
+
 __device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
 __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
 
@@ -720,10 +723,14 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   int cursor = 0;
 
+  // A workgroup of one wave needs neither LDS nor a barrier to hand the chosen step to its threads:
+  // they are the lanes of the polling wave, and take the operands from the chosen lane's registers.
+  const bool one_wave = blockDim.x == 64;
   for (;;) {
 #ifdef MSCCLX_PROFILE
     const u64 prof_t0 = wall_clock64();
 #endif
+    int chosen = -2;
     if (poller) {
       int choice = -2;
       unsigned spins = 0;
@@ -784,26 +791,44 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
           }
         }
       }
-      if (choice >= 0 && lane == choice) {
-        sh_move = c.m;
-        if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = h.tb; sh_who[1] = c.step; sh_who[2] = h.slice; sh_who[3] = (int)c.pass; }
+      if (!one_wave) {
+        if (choice >= 0 && lane == choice) {
+          sh_move = c.m;
+          if (LL) { sh_seq[0] = c.rseq; sh_seq[1] = c.sseq; sh_who[0] = h.tb; sh_who[1] = c.step; sh_who[2] = h.slice; sh_who[3] = (int)c.pass; }
+        }
+        if (lane == 0) sh_choice = choice;
       }
-      if (lane == 0) sh_choice = choice;
+      chosen = choice;
       cursor = choice >= 0 ? (choice + 1) & 63 : cursor;
     }
-    __syncthreads();
-    const int choice = sh_choice;
-    if (choice < 0) break;  // done (-1) or giving up (-3); uniform for the workgroup
+    int choice;
+    Move m;
+    uint32_t rseq = 0, sseq = 0;
+    int who_tb = 0, who_step = 0, who_slice = 0;
+    unsigned who_pass = 0;
+    if (one_wave) {
+      choice = __builtin_amdgcn_readfirstlane(chosen);
+      if (choice < 0) break;  // done (-1) or giving up (-3)
+      m.a = lane_value(c.m.a, choice); m.dst = lane_value(c.m.dst, choice); m.out = lane_value(c.m.out, choice);
+      m.n = lane_value(c.m.n, choice); m.rows = (int)lane_value((uint32_t)c.m.rows, choice); m.kind = (int)lane_value((uint32_t)c.m.kind, choice);
+      if (LL) {
+        rseq = lane_value(c.rseq, choice); sseq = lane_value(c.sseq, choice);
+        who_tb = (int)lane_value((uint32_t)h.tb, choice); who_step = (int)lane_value((uint32_t)c.step, choice);
+        who_slice = (int)lane_value((uint32_t)h.slice, choice); who_pass = lane_value(c.pass, choice);
+      }
+    } else {
+      __syncthreads();
+      choice = sh_choice;
+      if (choice < 0) break;  // done (-1) or giving up (-3); uniform for the workgroup
+      m = sh_move;
+      if (LL) { rseq = sh_seq[0]; sseq = sh_seq[1]; who_tb = sh_who[0]; who_step = sh_who[1]; who_slice = sh_who[2]; who_pass = (unsigned)sh_who[3]; }
+    }
 #ifdef MSCCLX_PROFILE
     const u64 prof_t1 = wall_clock64();
 #endif
 
     // ---- the chosen context's step: move one piece ----
-    {
-      const Move m = sh_move;
-      if (LL) do_move<R, VEC, LL>(m, p, epoch, sh_seq[0], sh_seq[1], sh_who[0], sh_who[1], sh_who[2], (unsigned)sh_who[3]);
-      else do_move<R, VEC, LL>(m, p, epoch, 0, 0, 0, 0, 0, 0);
-    }
+    do_move<R, VEC, LL>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
 #endif
@@ -814,7 +839,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     DevOp next;
     if (mine) next = fetch_next_op(c, h, p);
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    if (!one_wave) __syncthreads();
 #ifdef MSCCLX_PROFILE
     const u64 prof_t3 = wall_clock64();
 #endif
