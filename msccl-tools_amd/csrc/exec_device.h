@@ -205,6 +205,19 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
   const uint32_t T = blockDim.x;
+  if (n <= T) {
+    // A small piece (latency-bound programs): at most one unit per thread.  The loads a big piece
+    // needs in flight would only be instructions in the way here (measured: 4 % of a 64-rank ring
+    // all-reduce on 512-byte pieces).
+    const uint32_t i = threadIdx.x;
+    if (i < n) {
+      word x = A::template ld<XL>(ra, (int)(i * W));
+      if (HAS_B) x = R::combine(A::template ld<XL>(rb, (int)(i * W)), x);
+      A::template st<X1>(r1, (int)(i * W), x);
+      if (HAS_O2) A::template st<XS>(r2, (int)(i * W), x);
+    }
+    return;
+  }
   // kUnroll loads are in flight per thread either way: all of a, or half of a and half of b
   constexpr int UA = HAS_B ? (kUnroll / 2 > 0 ? kUnroll / 2 : 1) : kUnroll;
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
