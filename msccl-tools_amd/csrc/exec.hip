@@ -52,7 +52,7 @@ struct DeviceState {
   kernel_fn kernel = nullptr;
   bool dirty = false;  // counters must be cleared before the next launch (after a failed launch)
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: 8 words per workgroup
+  unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: kProfWords words per workgroup
 };
 
 void destroy_device_state(DeviceState* d) {
@@ -249,7 +249,8 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   HIP_TRY(hipEventCreate(&d->ev0));
   HIP_TRY(hipEventCreate(&d->ev1));
 #ifdef MSCCLX_PROFILE
-  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * 8 * g.workgroups));
+  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * kProfWords * g.workgroups));
+  HIP_TRY(hipMemset(d->prof, 0, sizeof(unsigned long long) * kProfWords * g.workgroups));
 #endif
   return MSCCLX_OK;
 }
@@ -309,8 +310,9 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
 #ifdef MSCCLX_PROFILE
   if (d->prof && getenv("MSCCLX_PROFILE_DUMP")) {
     const size_t nwg = plan->geo.workgroups;
-    std::vector<unsigned long long> h(nwg * 8);
-    (void)hipMemcpy(h.data(), d->prof, h.size() * 8, hipMemcpyDeviceToHost);
+    std::vector<unsigned long long> all(nwg * kProfWords), h(nwg * 8);
+    (void)hipMemcpy(all.data(), d->prof, all.size() * 8, hipMemcpyDeviceToHost);
+    for (size_t w = 0; w < nwg; ++w) std::copy(all.begin() + w * kProfWords, all.begin() + w * kProfWords + 8, h.begin() + w * 8);
     double sw = 0, sm = 0, sa = 0, sf = 0, st_ = 0; unsigned long long first = ~0ull, last = 0;
     for (size_t w = 0; w < nwg; ++w) {
       sw += h[w * 8]; sm += h[w * 8 + 1]; st_ += h[w * 8 + 2]; sa += h[w * 8 + 4]; sf += h[w * 8 + 5];
@@ -319,6 +321,43 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
     }
     fprintf(stderr, "[prof] wgs=%zu span=%.1f us  mean per wg: poll %.1f us  move %.1f us  ack+barrier %.1f us  finish+describe %.1f us  total %.1f us\n",
             nwg, (last - first) / 100.0, sw / nwg / 100, sm / nwg / 100, sa / nwg / 100, sf / nwg / 100, st_ / nwg / 100);
+    // When the workgroups ended, and how long each polled: deciles over the workgroups, in microseconds from the first start.
+    std::vector<double> ends(nwg), polls(nwg), starts(nwg);
+    for (size_t w = 0; w < nwg; ++w) {
+      starts[w] = (h[w * 8 + 3] - first) / 100.0;
+      ends[w] = (h[w * 8 + 3] + h[w * 8 + 2] - first) / 100.0;
+      polls[w] = h[w * 8] / 100.0;
+    }
+    std::sort(ends.begin(), ends.end()); std::sort(polls.begin(), polls.end()); std::sort(starts.begin(), starts.end());
+    std::string line = "[prof] deciles";
+    for (const auto* v : {&starts, &ends, &polls}) {
+      line += v == &starts ? "  start:" : v == &ends ? "  end:" : "  poll:";
+      for (int q = 0; q <= 10; ++q) { char b[32]; snprintf(b, sizeof b, " %.0f", (*v)[std::min(nwg - 1, q * nwg / 10)]); line += b; }
+    }
+    fprintf(stderr, "%s\n", line.c_str());
+    // MSCCLX_PROFILE_DUMP=<path ending in .csv>: one row per workgroup, in ticks of 10 ns.
+    const char* path = getenv("MSCCLX_PROFILE_DUMP");
+    if (std::strlen(path) > 4 && !std::strcmp(path + std::strlen(path) - 4, ".csv")) {
+      if (FILE* f = fopen(path, "w")) {
+        fprintf(f, "wg,start,total,poll,move,ack,finish,hw_id,xcc_id\n");
+        for (size_t w = 0; w < nwg; ++w)
+          fprintf(f, "%zu,%llu,%llu,%llu,%llu,%llu,%llu,%llu,%llu\n", w, h[w * 8 + 3] - first, h[w * 8 + 2], h[w * 8], h[w * 8 + 1], h[w * 8 + 4], h[w * 8 + 5], h[w * 8 + 6], h[w * 8 + 7]);
+        fclose(f);
+      }
+      // <path>.moves: one row per logged move (the first kProfTrace of every workgroup)
+      if (FILE* f = fopen((std::string(path) + ".moves").c_str(), "w")) {
+        fprintf(f, "wg,index,tb,slice,start,duration\n");
+        const Geometry& g = plan->geo;
+        for (size_t w = 0; w < nwg; ++w)
+          for (int i = 0; i < kProfTrace; ++i) {
+            const unsigned long long e = all[w * kProfWords + 8 + i];
+            if (!e) break;
+            const int ctx = g.wg_begin[w] + (int)(e & 0xff);
+            fprintf(f, "%zu,%d,%d,%d,%llu,%llu\n", w, i, g.ctx_tb[ctx], g.ctx_slice[ctx], (e >> 32) + h[w * 8 + 3] - first, (e >> 8) & 0xffffff);
+          }
+        fclose(f);
+      }
+    }
   }
 #endif
   if (st.code != MSCCLX_OK) {

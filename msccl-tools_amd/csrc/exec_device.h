@@ -723,6 +723,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   c.active = false;
 #ifdef MSCCLX_PROFILE
   u64 prof_wait = 0, prof_move = 0, prof_ack = 0, prof_fin = 0;
+  unsigned prof_moves = 0;
   const u64 prof_start = wall_clock64();
 #endif
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
@@ -864,6 +865,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
       prof_move += prof_t2 - prof_t1;
       prof_ack += prof_t3 - prof_t2;
       prof_fin += prof_t4 - prof_t3;
+      // the first kProfTrace moves of the workgroup: start (10 ns ticks since the workgroup began), duration up to the barrier, lane
+      if (prof_moves < kProfTrace)
+        p.prof[(size_t)blockIdx.x * kProfWords + 8 + prof_moves] = ((prof_t1 - prof_start) << 32) | (((prof_t3 - prof_t1) & 0xffffffull) << 8) | (u64)(choice & 0xff);
+      ++prof_moves;
     }
 #endif
   }
@@ -885,12 +890,15 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   }
 #ifdef MSCCLX_PROFILE
   if (threadIdx.x == 0 && p.prof) {
-    p.prof[(size_t)blockIdx.x * 8 + 0] = prof_wait;
-    p.prof[(size_t)blockIdx.x * 8 + 1] = prof_move;
-    p.prof[(size_t)blockIdx.x * 8 + 2] = wall_clock64() - prof_start;
-    p.prof[(size_t)blockIdx.x * 8 + 3] = prof_start;
-    p.prof[(size_t)blockIdx.x * 8 + 4] = prof_ack;
-    p.prof[(size_t)blockIdx.x * 8 + 5] = prof_fin;
+    p.prof[(size_t)blockIdx.x * kProfWords + 0] = prof_wait;
+    p.prof[(size_t)blockIdx.x * kProfWords + 1] = prof_move;
+    p.prof[(size_t)blockIdx.x * kProfWords + 2] = wall_clock64() - prof_start;
+    p.prof[(size_t)blockIdx.x * kProfWords + 3] = prof_start;
+    p.prof[(size_t)blockIdx.x * kProfWords + 4] = prof_ack;
+    p.prof[(size_t)blockIdx.x * kProfWords + 5] = prof_fin;
+    // where the workgroup ran: HW_ID (compute unit, shader engine) and XCC_ID hardware registers
+    p.prof[(size_t)blockIdx.x * kProfWords + 6] = __builtin_amdgcn_s_getreg(4 | (31 << 11));
+    p.prof[(size_t)blockIdx.x * kProfWords + 7] = __builtin_amdgcn_s_getreg(20 | (31 << 11));
   }
 #endif
 }

@@ -135,6 +135,8 @@ MSCCLX_HOST_DEVICE inline uint64_t slice_begin(uint64_t chunk_units, uint32_t gr
 }
 
 constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
+constexpr int kProfTrace = 248;       // MSCCLX_PROFILE builds: moves logged per workgroup ...
+constexpr int kProfWords = 8 + kProfTrace;  // ... after its 8 words of totals
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
 // The control block in front of the two counter areas: word 0 = launches finished so far, word 1 =
