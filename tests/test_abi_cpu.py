@@ -126,7 +126,7 @@ def test_geometry_without_a_device(mscclx_lib):
     assert (k.slices, k.piece_bytes, k.passes, k.fifo_depth, k.threads, k.workgroups, k.max_hosted) == (16, 65536, 8, 4, 256, 128, 4)
     # element path when the chunk is not a multiple of 16 bytes
     info = p.configure(1000 * 4 + 4, "int32", max_workgroups=2048)
-    assert info.vector_path == 0 and info.slices == 2
+    assert info.vector_path == 0 and info.slices == 8   # tiny chunks: one slice per XCD
     with pytest.raises(MscclxError):
         p.configure(6, "int32", max_workgroups=2048)              # not a multiple of the element
     # more threadblocks than workgroups is fine: a workgroup hosts up to 64 contexts ...

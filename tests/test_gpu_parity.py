@@ -320,7 +320,7 @@ def test_ll_launch_number_wraps(knobs):
     n, E = 3, 300
     xml = ir_samples.ring_allreduce_xml(n)
     ex = Executor(xml)
-    info = ex.setup(E * 4, "int32", protocol="ll", piece_bytes=512, **knobs)  # several passes: slots are reused inside a launch too
+    info = ex.setup(E * 4, "int32", protocol="ll", slices=1, piece_bytes=512, **knobs)  # several passes: slots are reused inside a launch too
     assert info.protocol == 2 and info.passes >= 2
     rng = np.random.default_rng(11)
     x = [rng.integers(0, 2**32, n * E, dtype=np.uint64).astype(np.uint32) for _ in range(n)]
