@@ -499,10 +499,10 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // Slices of 32 KiB or more can give every compute unit a context.  Measured on MI355X (8 to 1920
       // threadblocks, 128 KiB to 64 MiB chunks), what matters is (1) that the contexts spread EVENLY
       // over the resident workgroups -- 7.5 contexts per workgroup on average means some host 8, and
-      // the launch takes as long as those take -- (2) enough contexts per workgroup to always find
-      // one ready -- four for every threadblock that is busy at a time (waiting_ratio), between
-      // 4 and 32 -- and (3) several passes of 64 KiB pieces over a big slice rather than one big
-      // piece, so that the phases of a program overlap (pass k+1 of an early phase runs beside
+      // the launch takes as long as those take -- (2) enough contexts to always find one ready --
+      // per half compute unit, four for every threadblock that is busy at a time (waiting_ratio),
+      // between 4 and 32 -- and (3) several passes of 64 KiB pieces over a big slice rather than one
+      // big piece, so that the phases of a program overlap (pass k+1 of an early phase runs beside
       // pass k of a later one).  Candidates are scored on (1) and (2); (3) follows below.
       std::vector<uint64_t> works;
       for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
@@ -524,7 +524,10 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
         int64_t wgs = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
         wgs = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(wgs, capacity_by_threads[thread_index(threads)]), c * ntbs));
         if (wgs * kMaxHosted < c * ntbs) continue;
-        const double per_wg = (double)(c * ntbs) / (double)wgs;
+        // (2) is about the compute unit, not the workgroup: smaller pieces run on smaller workgroups, more
+        // of them to a compute unit, and contexts per workgroup would not tell candidates apart.  The
+        // unit is half a compute unit -- one workgroup of 512 threads.
+        const double per_wg = std::max(1.0, (double)(c * ntbs) / (2.0 * num_cus));
         const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / wanted_per_wg));
         if (score > best_score + 1e-9 || (std::fabs(score - best_score) <= 1e-9 && c < slices)) { best_score = score; slices = c; }
       }
