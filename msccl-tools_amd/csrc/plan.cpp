@@ -539,12 +539,18 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // on the longest chain of the program's dataflow.  More slices shrink the pieces but add
       // workgroups; the minimum is at slices = sqrt(b/a * depth * chunk / threadblocks).  With
       // b/a = 6.25 per KiB (fitted on MI355X, workgroups of one wave) an 8-rank ring on 1 MiB comes
-      // out at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.
-      // Never finer than a context or two per compute unit, nor pieces below 512 bytes.
+      // out at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.  Threadblocks that
+      // mostly wait for each other cost less than the fixed cost each: with waiting_ratio r the
+      // minimum moves to sqrt(r) times as many slices (two-level all-reduce, r = 9.4, 16 KiB chunks:
+      // 4 slices 78 us, 1 slice 86 us).
+      // Never finer than a context or two per compute unit with pieces down to 512 bytes, nor than
+      // r times that with pieces of 4 KiB or more.
       int32_t depth_of_dataflow = 1;
-      (void)waiting_ratio(plan, &depth_of_dataflow);
-      const double best = std::sqrt(6.25 * (double)depth_of_dataflow * ((double)chunk_bytes / 1024.0) / (double)ntbs);
-      const int64_t most = std::max<int64_t>(1, std::min<int64_t>(std::max(finest, to_fill), (int64_t)(chunk_bytes / 512)));
+      const double ratio = waiting_ratio(plan, &depth_of_dataflow);
+      const double best = std::sqrt(ratio * 6.25 * (double)depth_of_dataflow * ((double)chunk_bytes / 1024.0) / (double)ntbs);
+      const int64_t fill = (int64_t)std::ceil((double)to_fill * ratio);
+      const int64_t most = std::max<int64_t>(1, std::max(std::min<int64_t>(std::max(finest, to_fill), (int64_t)(chunk_bytes / 512)),
+                                                         std::min<int64_t>(std::max(finest, fill), (int64_t)(chunk_bytes / 4096))));
       // a power of two (small chunks divide evenly only by those): the nearest one, not above `most`
       slices = 1;
       while (slices * 2 <= most && (double)(slices * 2) <= best * 1.41421356) slices *= 2;
