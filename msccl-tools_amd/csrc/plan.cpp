@@ -508,12 +508,14 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
       const int most_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
       const int64_t lo = std::max<int64_t>(1, to_fill);
-      const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(finest, ((int64_t)most_capacity * kMaxHosted) / ntbs));
+      const double wanted_per_wg = std::min(32.0, 4.0 * waiting_ratio(plan));
+      // pieces of 16 KiB only where 32 KiB pieces leave less than a quarter of the contexts wanted in (2)
+      const int64_t finer = (double)(finest * ntbs) / (2.0 * num_cus) < wanted_per_wg / 4 ? (int64_t)(chunk_bytes / (16 * 1024)) : finest;
+      const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(finer, ((int64_t)most_capacity * kMaxHosted) / ntbs));
       std::vector<int64_t> candidates = {lo, hi};
       for (int64_t base = 1; base <= hi; base *= 2)
         for (int64_t c : {base, base * 3})
           if (c >= lo && c <= hi) candidates.push_back(c);
-      const double wanted_per_wg = std::min(32.0, 4.0 * waiting_ratio(plan));
       double best_score = -1e9;
       for (int64_t c : candidates) {
         // the workgroups this choice would run on: threads follow the piece, workgroups the threads
