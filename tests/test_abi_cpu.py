@@ -207,3 +207,29 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
+
+
+def test_geometry_between_the_benchmark_sizes(mscclx_lib):
+    """Smaller messages of the same algorithms: (threads, slices, piece bytes) as measured best on MI355X."""
+    from msccl.executor.workloads import WORKLOADS
+    want = {
+        # tiny chunks: 8 slices, so that workgroup w (XCD w mod 8) hosts slice w mod 8 and hand-offs stay inside an XCD
+        ("c5", 64 << 10): (64, 8, 128),
+        ("c1", 16 << 10): (64, 8, 256),
+        # threadblocks that mostly wait: more slices than the plain latency model gives, pieces of 4 KiB or more
+        ("c4", 512 << 10): (64, 2, 4096),
+        ("c4", 1 << 20): (64, 4, 4096),
+        ("c3", 512 << 10): (128, 2, 16384),
+        # between latency and bandwidth: contexts are counted per compute unit, whatever the workgroup size
+        ("c3", 1 << 20): (128, 4, 16384),
+        ("c3", 4 << 20): (256, 8, 32768),
+        ("c4", 4 << 20): (128, 4, 16384),
+        ("c4", 8 << 20): (256, 4, 32768),
+        # rings keep the largest pieces that still fill the chip
+        ("c2", 4 << 20): (256, 32, 32768),
+        ("c1", 16 << 20): (256, 64, 32768),
+    }
+    for (key, nbytes), expect in want.items():
+        w = WORKLOADS[key].scaled(nbytes)
+        i = Plan(parse_algo_xml(WORKLOADS[key].build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
+        assert (i.threads, i.slices, i.piece_bytes) == expect, (key, nbytes, (i.threads, i.slices, i.piece_bytes))
