@@ -25,18 +25,18 @@ namespace mscclx {
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
 // The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
-kernel_fn pick_kernel_group_0(int dtype, int op, bool vec, bool ll);
-kernel_fn pick_kernel_group_1(int dtype, int op, bool vec, bool ll);
-kernel_fn pick_kernel_group_2(int dtype, int op, bool vec, bool ll);
-kernel_fn pick_kernel_group_3(int dtype, int op, bool vec, bool ll);
-kernel_fn pick_kernel_group_4(int dtype, int op, bool vec, bool ll);
-static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll) {
+kernel_fn pick_kernel_group_0(int dtype, int op, bool vec, bool ll, bool fold);
+kernel_fn pick_kernel_group_1(int dtype, int op, bool vec, bool ll, bool fold);
+kernel_fn pick_kernel_group_2(int dtype, int op, bool vec, bool ll, bool fold);
+kernel_fn pick_kernel_group_3(int dtype, int op, bool vec, bool ll, bool fold);
+kernel_fn pick_kernel_group_4(int dtype, int op, bool vec, bool ll, bool fold);
+static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll, bool fold) {
   switch (dtype / 2) {
-    case 0: return pick_kernel_group_0(dtype, op, vec, ll);
-    case 1: return pick_kernel_group_1(dtype, op, vec, ll);
-    case 2: return pick_kernel_group_2(dtype, op, vec, ll);
-    case 3: return pick_kernel_group_3(dtype, op, vec, ll);
-    case 4: return pick_kernel_group_4(dtype, op, vec, ll);
+    case 0: return pick_kernel_group_0(dtype, op, vec, ll, fold);
+    case 1: return pick_kernel_group_1(dtype, op, vec, ll, fold);
+    case 2: return pick_kernel_group_2(dtype, op, vec, ll, fold);
+    case 3: return pick_kernel_group_3(dtype, op, vec, ll, fold);
+    case 4: return pick_kernel_group_4(dtype, op, vec, ll, fold);
     default: return nullptr;
   }
 }
@@ -46,6 +46,9 @@ struct DeviceState {
   DevTb* tbs = nullptr;
   DevOp* ops = nullptr;
   DevConn* conns = nullptr;
+  uint32_t* extra_deps = nullptr;
+  std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
+  std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
   int32_t* hosting = nullptr;            // wg_begin | ctx_tb | ctx_slice
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
@@ -60,11 +63,21 @@ void destroy_device_state(DeviceState* d) {
   if (d->tbs) (void)hipFree(d->tbs);
   if (d->ops) (void)hipFree(d->ops);
   if (d->conns) (void)hipFree(d->conns);
+  if (d->extra_deps) (void)hipFree(d->extra_deps);
   if (d->hosting) (void)hipFree(d->hosting);
   if (d->host_status) (void)hipHostFree(d->host_status);
   if (d->ev0) (void)hipEventDestroy(d->ev0);
   if (d->ev1) (void)hipEventDestroy(d->ev1);
   delete d;
+}
+
+// A nop that nobody depends on and that is not its threadblock's last step can be folded into the
+// step after it (mscclx_plan_bind).
+static bool has_foldable_nops(const mscclx_plan& plan) {
+  for (const Tb& tb : plan.tbs)
+    for (int o = tb.op_begin; o + 1 < tb.op_end; ++o)
+      if (plan.ops[o].type == MSCCLX_OP_NOP && !plan.ops[o].hasdep) return true;
+  return false;
 }
 
 static int query_capacity(kernel_fn k, int* num_cus, int capacity[4]) {
@@ -103,7 +116,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     for (int i = 0; i < 4; ++i) capacity[i] = cfg.max_workgroups;
   } else {
     const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
-    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll), &num_cus, capacity);
+    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, vec && !ll && has_foldable_nops(*plan)), &num_cus, capacity);
     if (rc) return rc;
   }
   Geometry g;
@@ -177,7 +190,8 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   DeviceState* d = new DeviceState();
   plan->dev = d;
   HIP_TRY(hipGetDevice(&d->device));
-  d->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0);
+  const bool fold = g.vector_path && !g.ll && has_foldable_nops(*plan);
+  d->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0, fold);
   if (!d->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
 
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
@@ -210,7 +224,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
         dv.dep_step = op.deps;
         dv.dep_nops = plan->tbs[dv.dep_tb].op_end - plan->tbs[dv.dep_tb].op_begin;
       }
-      dv.send_seq = op.send_seq; dv.recv_seq = op.recv_seq;
+      dv.extra = 0; dv.steps = 1;
       dv.word = (uint32_t)op.type | ((uint32_t)std::max(op.cnt, 0) << kOpCntShift);
       if (op.hasdep) dv.word |= kOpHasdep;
       if (op.final_write) dv.word |= kOpNtStore;
@@ -227,11 +241,55 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
       }
     }
   }
+  // Fold runs of nop steps into the step that follows them: that step waits for all their
+  // dependencies at once (one round of counter loads) instead of one hand-off per nop.  A nop that
+  // somebody depends on stays a step of its own, as does the last step of a threadblock.
+  std::vector<uint32_t> extras;
+  {
+    std::vector<DevOp> folded_ops;
+    folded_ops.reserve(nop);
+    d->dev_op_begin.assign(ntb, 0);
+    d->dev_ir_step.clear();
+    for (size_t t = 0; t < ntb; ++t) {
+      const Tb& tb = plan->tbs[t];
+      d->dev_op_begin[t] = (int32_t)folded_ops.size();
+      std::vector<uint32_t> pending;
+      uint32_t folded = 0;
+      for (int o = tb.op_begin; o < tb.op_end; ++o) {
+        DevOp dv = hop[o];
+        const bool nop_step = (dv.word & 15u) == MSCCLX_OP_NOP;
+        if (fold && nop_step && !(dv.word & kOpHasdep) && o + 1 < tb.op_end && pending.size() / kExtraDepWords < (size_t)kMaxExtraDeps &&
+            dv.dep_nops < 65536 && folded < 255) {
+          if (dv.dep_tb >= 0) {
+            pending.push_back((uint32_t)dv.dep_tb * kSyncStrideWords);
+            pending.push_back(((uint32_t)dv.dep_step + 1) | ((uint32_t)dv.dep_nops << 16));
+          }
+          ++folded;
+          continue;
+        }
+        const size_t first = extras.size() / kExtraDepWords;
+        if (first >= (1u << 24)) return fail(MSCCLX_ERR_CAPACITY, "too many folded dependencies");
+        dv.extra = (uint32_t)(first << 8) | (uint32_t)(pending.size() / kExtraDepWords);
+        dv.steps = 1 + folded;
+        extras.insert(extras.end(), pending.begin(), pending.end());
+        pending.clear();
+        folded = 0;
+        folded_ops.push_back(dv);
+        d->dev_ir_step.push_back(o - tb.op_begin);
+      }
+      htb[t].op_begin = d->dev_op_begin[t];
+      htb[t].nops = (int32_t)folded_ops.size() - d->dev_op_begin[t];
+    }
+    hop.swap(folded_ops);
+  }
+  const size_t ndev = hop.size();
   HIP_TRY(hipMalloc((void**)&d->tbs, sizeof(DevTb) * (ntb ? ntb : 1)));
-  HIP_TRY(hipMalloc((void**)&d->ops, sizeof(DevOp) * (nop ? nop : 1)));
+  HIP_TRY(hipMalloc((void**)&d->ops, sizeof(DevOp) * (ndev ? ndev : 1)));
+  HIP_TRY(hipMalloc((void**)&d->extra_deps, sizeof(uint32_t) * (extras.empty() ? kExtraDepWords : extras.size())));
+  if (!extras.empty()) HIP_TRY(hipMemcpy(d->extra_deps, extras.data(), sizeof(uint32_t) * extras.size(), hipMemcpyHostToDevice));
   HIP_TRY(hipMalloc((void**)&d->conns, sizeof(DevConn) * hcn.size()));
   HIP_TRY(hipMemcpy(d->tbs, htb.data(), sizeof(DevTb) * ntb, hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(d->ops, hop.data(), sizeof(DevOp) * nop, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d->ops, hop.data(), sizeof(DevOp) * ndev, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d->conns, hcn.data(), sizeof(DevConn) * hcn.size(), hipMemcpyHostToDevice));
   {
     std::vector<int32_t> table(g.wg_begin);
@@ -267,7 +325,7 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
     d->dirty = false;
   }
   KernelParams kp;
-  kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns;
+  kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns; kp.extra_deps = d->extra_deps;
   unsigned long long* sync = (unsigned long long*)d->workspace;
   kp.sync_base = sync;
   kp.sync_cur = kp.sync_nxt = nullptr;
@@ -306,6 +364,11 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
     return fail(MSCCLX_ERR_HIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(e));
   }
   mscclx_status st = *d->host_status;
+  if (st.code != MSCCLX_OK && st.tb >= 0 && (size_t)st.tb < d->dev_op_begin.size()) {
+    // the kernel counts the steps of its own list, in which runs of nops are folded: report the IR's step
+    const size_t at = (size_t)d->dev_op_begin[(size_t)st.tb] + (size_t)std::max(st.step, 0);
+    if (at < d->dev_ir_step.size()) st.step = d->dev_ir_step[at];
+  }
   if (status) *status = st;
 #ifdef MSCCLX_PROFILE
   if (d->prof && getenv("MSCCLX_PROFILE_DUMP")) {

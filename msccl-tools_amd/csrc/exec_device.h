@@ -430,11 +430,33 @@ struct Context {
   u64 off;                  // byte offset of this pass's piece inside any chunk
   // the step the context stands at
   bool moves;  // false: nop or a send whose payload is read in place -- nothing to copy
-  int type, hasdep;
+  int type, hasdep;         // hasdep: bit 0 = others wait for this step; bits 8.. = IR steps this step stands for (itself and folded nops)
+  uint32_t extra;           // folded dependencies: first entry << 8 | how many
   const u64 *w0, *w1, *w2;  // counters to wait for (null = none) ...
   uint32_t t0, t1, t2;      // ... until they reach these values (every counter of a launch stays below 2^32)
   Move m;
 };
+
+// The dependencies of the nop steps folded into the step `c` stands at: all their counters are
+// loaded in one round, after one round for the table entries.
+__device__ __forceinline__ bool extras_ready(const Context& c, const Hosted& h, const KernelParams& p) {
+  const uint32_t n = c.extra & 255u;
+  const uint2* const e = (const uint2*)p.extra_deps + (c.extra >> 8);
+  const u64* const flags = p.sync_cur + h.flags;
+  uint2 entry[kMaxExtraDeps];
+#pragma unroll
+  for (int k = 0; k < kMaxExtraDeps; ++k)
+    if ((uint32_t)k < n) entry[k] = e[k];
+  u64 v[kMaxExtraDeps];
+#pragma unroll
+  for (int k = 0; k < kMaxExtraDeps; ++k)
+    if ((uint32_t)k < n) v[k] = load_counter(flags + entry[k].x);
+  bool ok = true;
+#pragma unroll
+  for (int k = 0; k < kMaxExtraDeps; ++k)
+    if ((uint32_t)k < n) ok = ok && v[k] >= (u64)(c.pass * (entry[k].y >> 16) + (entry[k].y & 0xffffu));
+  return ok;
+}
 
 // Describe the step `c` stands at: what it must wait for, whether it moves data, and from where to
 // where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
@@ -446,7 +468,8 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
   const int cnt = (int)(op.word >> kOpCntShift);
   const bool out_staged = op.word & kOpOutStaged, in_place = op.word & kOpInPlace;
   c.type = t;
-  c.hasdep = (op.word & kOpHasdep) ? 1 : 0;
+  c.hasdep = ((op.word & kOpHasdep) ? 1 : 0) | (int)(op.steps << 8);
+  c.extra = op.extra;
   const bool rcv = is_recv(t), snd = is_send(t);
   c.w0 = c.w1 = c.w2 = nullptr;
   c.t0 = c.t1 = c.t2 = 0;
@@ -517,8 +540,8 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
     c.rslot += h.in_slot_bytes;
     if (c.rslot == h.in_wrap) c.rslot = 0;
   }
-  ++c.count;
-  if (c.hasdep && writer) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * nops + step + 1
+  c.count += (uint32_t)c.hasdep >> 8;
+  if ((c.hasdep & 1) && writer) publish(p.sync_cur + h.my_flag, (u64)c.count);  // = pass * steps of the IR + IR step + 1
   if (++c.step == h.nops) {
     c.step = 0;
     ++c.pass;
@@ -688,7 +711,9 @@ __device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, 
 // on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
 // reduces that step's piece.  No context ever blocks the workgroup, so any number of threadblocks can
 // share the resident workgroups without deadlock.
-template <class R, bool VEC, bool LL>
+// FOLD: steps may carry the dependencies of nop steps folded into them (a kernel of its own, so that
+// programs without such steps do not pay for the check in the poll loop).
+template <class R, bool VEC, bool LL, bool FOLD = false>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
   static_assert(VEC || !LL, "LL lines carry 16-byte units");
   constexpr int EB = R::kElemBytes;
@@ -762,6 +787,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
           const u64 v2 = c.w2 ? load_counter(c.w2) : 0;
           ready = (!c.w0 || v0 >= c.t0) && (!c.w2 || v2 >= c.t2) &&
                   (!watch1 || (LL ? (uint32_t)(v1 >> 32) == (uint32_t)c.t1 : v1 >= c.t1));
+          if (FOLD && ready && (c.extra & 255u)) ready = extras_ready(c, h, p);  // the nops folded into this step
         }
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
@@ -908,16 +934,17 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
 
-template <int DT, int OP> kernel_fn pick_vec(bool vec, bool ll) {
-  if (ll) return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, true> : nullptr;
+template <int DT, int OP> kernel_fn pick_vec(bool vec, bool ll, bool fold) {
+  if (ll) return vec && !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, true> : nullptr;
+  if (fold) return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false, true> : nullptr;
   return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false> : (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false>;
 }
-template <int DT> kernel_fn pick_op(int op, bool vec, bool ll) {
+template <int DT> kernel_fn pick_op(int op, bool vec, bool ll, bool fold) {
   switch (op) {
-    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec, ll);
-    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec, ll);
-    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec, ll);
-    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec, ll);
+    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec, ll, fold);
+    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec, ll, fold);
+    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec, ll, fold);
+    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec, ll, fold);
     default: return nullptr;
   }
 }

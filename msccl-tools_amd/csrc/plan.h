@@ -55,7 +55,11 @@ struct DevOp {
   uint32_t word;
   int32_t dep_tb, dep_step;  // global threadblock row / step, or -1
   int32_t dep_nops;          // number of steps of the threadblock depended on
-  int32_t send_seq, recv_seq;
+  // A run of nop steps in front of this one is folded into it: their dependencies are entries
+  // [extra >> 8, (extra >> 8) + (extra & 255)) of the extra-dependency table, and finishing this step
+  // finishes `steps` steps of the IR (itself and the folded ones).
+  uint32_t extra;
+  uint32_t steps;
   // byte addresses of the first named chunk, resolved when buffers are bound (0 where the step has none)
   uint64_t src_addr;         // local source of s / cpy / re
   uint64_t dst_addr;         // local destination (and local reduction operand) of every step but s
@@ -64,6 +68,8 @@ struct DevOp {
 static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
 constexpr uint32_t kOpHasdep = 1u << 4, kOpOutStaged = 1u << 5, kOpNtStore = 1u << 6, kOpInPlace = 1u << 7;
 constexpr int kOpCntShift = 8;
+constexpr int kMaxExtraDeps = 3;         // nop steps folded into the step that follows them, at most
+constexpr int kExtraDepWords = 2;        // one folded dependency: counter word (from the slice's first flag); step + 1 | steps per pass of that threadblock << 16
 
 struct DevTb {
   int32_t op_begin, nops;
@@ -101,6 +107,7 @@ struct KernelParams {
   const DevTb* tbs;
   const DevOp* ops;
   const DevConn* conns;
+  const uint32_t* extra_deps;   // kExtraDepWords words per folded dependency
   unsigned long long* sync_base; // control block (kControlWords): word 0 = launches finished so far (its parity picks the counter area)
   unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
   unsigned long long* sync_nxt;  // next launch's counters   } from the control block
