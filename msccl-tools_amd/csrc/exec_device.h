@@ -246,6 +246,39 @@ template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool NT1 = false>
 __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
                                           const unsigned char* b, uint64_t stride_b, int rows, uint32_t n) {
   constexpr int W = VEC ? 16 : R::kElemBytes;
+  if (!HAS_B && !HAS_O2 && __builtin_expect(rows > 1 && n <= blockDim.x, 0)) {  // (plain copies only: the scatter and gather steps of all-pairs and all-to-all programs)
+    // Several short rows (a multi-chunk step of a latency-bound program): one unit per thread and
+    // row.  Four rows are loaded before the first is stored -- row by row, every row would wait
+    // for its own round trip to memory.
+    typedef Access<W> A;
+    typedef typename A::word word;
+    constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
+    constexpr int RB = 4;
+    const uint32_t i = threadIdx.x;
+    if (i >= n) return;
+    const uint32_t bytes = n * W;
+    for (int r0 = 0; r0 < rows; r0 += RB) {
+      word x[RB], y[RB];
+#pragma unroll
+      for (int k = 0; k < RB; ++k)
+        if (r0 + k < rows) x[k] = A::template ld<XL>(make_rsrc(a + (uint64_t)(r0 + k) * stride_a * W, bytes), (int)(i * W));
+      if (HAS_B) {
+#pragma unroll
+        for (int k = 0; k < RB; ++k)
+          if (r0 + k < rows) y[k] = A::template ld<XL>(make_rsrc(b + (uint64_t)(r0 + k) * stride_b * W, bytes), (int)(i * W));
+#pragma unroll
+        for (int k = 0; k < RB; ++k)
+          if (r0 + k < rows) x[k] = R::combine(y[k], x[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < RB; ++k)
+        if (r0 + k < rows) {
+          A::template st<X1>(make_rsrc(o1 + (uint64_t)(r0 + k) * stride_o1 * W, bytes), (int)(i * W), x[k]);
+          if (HAS_O2) A::template st<XS>(make_rsrc(o2 + (uint64_t)(r0 + k) * n * W, bytes), (int)(i * W), x[k]);
+        }
+    }
+    return;
+  }
   for (int r = 0; r < rows; ++r)
     move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
                                     a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
