@@ -854,6 +854,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
                 if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
                 else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
                 else if (c.w2 && load_counter(c.w2) < c.t2) what = 2;
+                else if (FOLD && (c.extra & 255u)) what = 0;  // the dependency of a nop folded into this step
                 mscclx_status* hs = p.host_status;
                 hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
                 __threadfence_system();

@@ -137,6 +137,17 @@ def slow_producer_xml(ncopies):
     ])
 
 
+def slow_dependency_xml(ncopies):
+    """One rank.  Threadblock 0 makes `ncopies` copies of its chunk; threadblock 1 waits for the first
+    and for the last of them through two nop steps (the way msccl-tools gives a step several
+    dependencies, msccl/language/ir.py:296-311) and then copies the result on: its step 2 waits for as
+    long as the copies take."""
+    tb0 = [_step(k, "cpy", "i", 0, "o", 0, 1, hasdep=1 if k in (0, ncopies - 1) else 0) for k in range(ncopies)]
+    tb1 = [_step(0, "nop", "i", -1, "o", -1, 0, depid=0, deps=0), _step(1, "nop", "i", -1, "o", -1, 0, depid=0, deps=ncopies - 1),
+           _step(2, "cpy", "o", 0, "o", 1, 1)]
+    return _algo("slow_dependency", "custom", 0, 1, 1, 2, [_gpu(0, 1, 2, 0, [_tb(0, -1, -1, 0, tb0), _tb(1, -1, -1, 0, tb1)])])
+
+
 # ---- documents in the style of msccl-tools' second emitter (msccl/ncclize.py:658-718) ----------
 # inplace="0", only s / r / rrc / cpy / nop, sending and receiving threadblocks separate, one extra
 # threadblock per rank (send=recv=-1, chan 0) holding the pre/post copies, and on r / rrc steps

@@ -280,6 +280,31 @@ def test_watchdog_reports_instead_of_hanging():
     assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
 
 
+def test_watchdog_names_the_ir_step_of_folded_nops():
+    """Nop steps in front of a step are folded into it at bind; a watchdog report still counts steps
+    as the IR does.  Threadblock 1's step 2 (behind two nops) waits for 24 copies of 64 MiB under a
+    1 ms limit; with a sane limit the same program delivers."""
+    from msccl.executor import Executor, MscclxError
+    xml = ir_samples.slow_dependency_xml(24)
+    nbytes = 64 << 20
+    x = torch.arange(nbytes, dtype=torch.int32).to(torch.uint8).cuda()
+    ex = Executor(xml)
+    ex.setup(nbytes, "uint8", timeout_ms=1, slices=1, piece_bytes=nbytes)
+    out = torch.zeros(2 * nbytes, dtype=torch.uint8, device="cuda")
+    ex.bind([x], [out])
+    print("case: watchdog on a step with folded nops", flush=True)
+    ex.launch()
+    with pytest.raises(MscclxError) as e:
+        ex.wait()
+    assert "watchdog" in str(e.value) and "rank 0 tb 1 step 2" in str(e.value) and "its dependency" in str(e.value)
+    torch.cuda.synchronize()
+    ex2 = Executor(xml)
+    ex2.setup(nbytes, "uint8")
+    out = torch.zeros(2 * nbytes, dtype=torch.uint8, device="cuda")
+    ex2.run([x], [out])
+    assert torch.equal(out[:nbytes], x) and torch.equal(out[nbytes:], x)
+
+
 @pytest.mark.parametrize("threads", [0, 64])
 def test_watchdog_in_ll_mode(threads):
     """Flag-in-data lines, one context per workgroup (threads=64: a workgroup of one wave, which runs
