@@ -282,6 +282,59 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
     }
     hop.swap(folded_ops);
   }
+  if (fold) {
+    // A run of `re` steps of one chunk each into the same destination, from sources a fixed distance
+    // apart (the local reduction of the all-pairs programs: msccl-tools' msccl/programs/allreduce_allpairs.py:18-21),
+    // becomes one step with several sources.  Only the first of them may wait for anything, only
+    // the last may be waited for.
+    std::vector<DevOp> fused;
+    std::vector<int32_t> fused_ir;
+    fused.reserve(hop.size());
+    for (size_t t = 0; t < ntb; ++t) {
+      const int32_t begin = htb[t].op_begin, end = begin + htb[t].nops;
+      const int32_t new_begin = (int32_t)fused.size();
+      for (int32_t i = begin; i < end;) {
+        DevOp dv = hop[(size_t)i];
+        int32_t j = i + 1;
+        auto plain_re = [&](const DevOp& o) { return (o.word & 15u) == MSCCLX_OP_REDUCE && (o.word >> kOpCntShift) == 1; };
+        if (plain_re(dv) && !(dv.word & kOpHasdep)) {
+          uint64_t stride = 0;
+          int sources = 1;
+          bool hasdep = false, nt = (dv.word & kOpNtStore) != 0;
+          uint32_t steps = dv.steps;
+          while (j < end && sources < kMaxReduceSources && !hasdep) {
+            const DevOp& nx = hop[(size_t)j];
+            if (!plain_re(nx) || nx.dst_addr != dv.dst_addr || nx.dep_tb >= 0 || (nx.extra & 255u) || nx.steps != 1) break;
+            const uint64_t expect_stride = nx.src_addr - hop[(size_t)j - 1].src_addr;
+            if (nx.src_addr <= hop[(size_t)j - 1].src_addr || (sources > 1 && expect_stride != stride)) break;
+            // the sources must stay clear of the destination chunk
+            const uint64_t cb = plan->chunk_bytes;
+            if (!(nx.src_addr + cb <= dv.dst_addr || dv.dst_addr + cb <= nx.src_addr)) break;
+            if ((uint64_t)sources * expect_stride + cb >= (1ull << 31)) break;  // one buffer descriptor spans all sources
+            stride = expect_stride;
+            hasdep = (nx.word & kOpHasdep) != 0;
+            nt = (nx.word & kOpNtStore) != 0;
+            ++sources; ++steps; ++j;
+          }
+          if (sources > 1 && (dv.src_addr + plan->chunk_bytes <= dv.dst_addr || dv.dst_addr + plan->chunk_bytes <= dv.src_addr)) {
+            dv.word = (uint32_t)MSCCLX_OP_REDUCE | ((uint32_t)sources << kOpCntShift) | (hasdep ? kOpHasdep : 0u) | (nt ? kOpNtStore : 0u);
+            dv.in_addr = stride;
+            dv.steps = steps;
+          } else {
+            j = i + 1;
+          }
+        }
+        fused.push_back(dv);
+        fused_ir.push_back(d->dev_ir_step[(size_t)i]);
+        i = j;
+      }
+      d->dev_op_begin[t] = new_begin;
+      htb[t].op_begin = new_begin;
+      htb[t].nops = (int32_t)fused.size() - new_begin;
+    }
+    hop.swap(fused);
+    d->dev_ir_step.swap(fused_ir);
+  }
   const size_t ndev = hop.size();
   HIP_TRY(hipMalloc((void**)&d->tbs, sizeof(DevTb) * (ntb ? ntb : 1)));
   HIP_TRY(hipMalloc((void**)&d->ops, sizeof(DevOp) * (ndev ? ndev : 1)));

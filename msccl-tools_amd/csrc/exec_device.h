@@ -163,26 +163,31 @@ template <int W> struct Access;
 template <> struct Access<16> {
   typedef u32x4 word;
   template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ word lds(__amdgpu_buffer_rsrc_t r, int off, int soff) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, AUX); }
   template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, AUX); }
 };
 template <> struct Access<8> {
   typedef u32x2 word;
   template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ word lds(__amdgpu_buffer_rsrc_t r, int off, int soff) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, soff, AUX); }
   template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, AUX); }
 };
 template <> struct Access<4> {
   typedef unsigned int word;
   template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ word lds(__amdgpu_buffer_rsrc_t r, int off, int soff) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, soff, AUX); }
   template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, AUX); }
 };
 template <> struct Access<2> {
   typedef unsigned short word;
   template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ word lds(__amdgpu_buffer_rsrc_t r, int off, int soff) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, soff, AUX); }
   template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b16(v, r, off, 0, AUX); }
 };
 template <> struct Access<1> {
   typedef unsigned char word;
   template <int AUX> static __device__ __forceinline__ word ld(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b8(r, off, 0, AUX); }
+  template <int AUX> static __device__ __forceinline__ word lds(__amdgpu_buffer_rsrc_t r, int off, int soff) { return __builtin_amdgcn_raw_buffer_load_b8(r, off, soff, AUX); }
   template <int AUX> static __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, int off, word v) { __builtin_amdgcn_raw_buffer_store_b8(v, r, off, 0, AUX); }
 };
 
@@ -282,6 +287,32 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
   for (int r = 0; r < rows; ++r)
     move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
                                     a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
+}
+
+// dst = ((dst (+) a0) (+) a1) ... (+) a[m-1] over n units of W bytes; source k starts `stride` bytes
+// after source k-1.  All sources of a unit are in flight together and folded in order, so the result
+// is bit for bit that of m reduce steps -- which would read and write dst m times.
+template <class R, int W, bool NT1>
+__device__ __forceinline__ void move_reduce_many(unsigned char* dst, const unsigned char* a, uint32_t stride, int m, uint32_t n) {
+  typedef Access<W> A;
+  typedef typename A::word word;
+  constexpr int XL = MSCCLX_AUX_LD, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
+  const uint32_t bytes = n * W;
+  const __amdgpu_buffer_rsrc_t rd = make_rsrc(dst, bytes);
+  // one descriptor for all sources (the host keeps their span below 2 GiB); source k is reached
+  // through the scalar offset of the load, so that the sources cost one scalar register each
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(a, (uint32_t)(m - 1) * stride + bytes);
+  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+    word acc = A::template ld<XL>(rd, (int)(i * W));
+    word s[kMaxReduceSources];
+#pragma unroll
+    for (int k = 0; k < kMaxReduceSources; ++k)
+      if (k < m) s[k] = A::template lds<XL>(rs, (int)(i * W), (int)((uint32_t)k * stride));
+#pragma unroll
+    for (int k = 0; k < kMaxReduceSources; ++k)
+      if (k < m) acc = R::combine(acc, s[k]);
+    A::template st<X1>(rd, (int)(i * W), acc);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -424,6 +455,7 @@ enum {
   kLLKind = 8,   // flag-in-data lines: bits 0-2 then say which movement (kLL* below)
   kAPacked = 16, // a is a slot
   kToSlot = 32,  // the first (only) destination is `out` instead of dst
+  kMany = 64,    // dst = ((dst (+) a[0]) (+) a[1]) ...: `rows` sources, `out` bytes apart
 };
 enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
 
@@ -489,6 +521,14 @@ __device__ __forceinline__ bool extras_ready(const Context& c, const Hosted& h, 
   for (int k = 0; k < kMaxExtraDeps; ++k)
     if ((uint32_t)k < n) ok = ok && v[k] >= (u64)(c.pass * (entry[k].y >> 16) + (entry[k].y & 0xffffu));
   return ok;
+}
+
+// FOLD kernels: an `re` with several sources (in_addr = their distance in bytes, cnt = how many).
+__device__ __forceinline__ void mark_many_sources(Context& c, const DevOp& op) {
+  if ((op.word & 15u) == MSCCLX_OP_REDUCE && op.in_addr) {
+    c.m.out = op.in_addr;
+    c.m.kind = kMany | ((op.word & kOpNtStore) ? (int)kNt1 : 0);
+  }
 }
 
 // Describe the step `c` stands at: what it must wait for, whether it moves data, and from where to
@@ -629,13 +669,19 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
 // incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool VEC, bool LL>
+template <class R, bool VEC, bool LL, bool FOLD = false>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
   const u64 cs = p.chunk_units;
   unsigned char* const dst = (unsigned char*)m.dst;
   unsigned char* const out = (unsigned char*)m.out;
   const unsigned char* const a = (const unsigned char*)m.a;
+  if (FOLD && __builtin_expect((m.kind & kMany) != 0, 0)) {  // (only the bind of a FOLD kernel makes such steps)
+    constexpr int W = VEC ? 16 : R::kElemBytes;
+    if (m.kind & kNt1) move_reduce_many<R, W, true>(dst, a, (uint32_t)m.out, m.rows, m.n);
+    else move_reduce_many<R, W, false>(dst, a, (uint32_t)m.out, m.rows, m.n);
+    return;
+  }
   if (LL && (m.kind & kLLKind)) {
     const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
     const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tb, step, slice, (u64)pass};
@@ -793,6 +839,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 #endif
   } else {
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
+  if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
   int cursor = 0;
 
   // A workgroup of one wave needs neither LDS nor a barrier to hand the chosen step to its threads:
@@ -826,6 +873,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
           const DevOp next = fetch_next_op(c, h, p);
           finish_step<(int)UB, LL>(c, h, p, epoch, next);
+          if (FOLD && c.active) mark_many_sources(c, next);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
         }
@@ -902,7 +950,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 #endif
 
     // ---- the chosen context's step: move one piece ----
-    do_move<R, VEC, LL>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
+    do_move<R, VEC, LL, FOLD>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
 #endif
@@ -917,7 +965,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 #ifdef MSCCLX_PROFILE
     const u64 prof_t3 = wall_clock64();
 #endif
-    if (mine) finish_step<(int)UB, LL>(c, h, p, epoch, next);
+    if (mine) {
+      finish_step<(int)UB, LL>(c, h, p, epoch, next);
+      if (FOLD && c.active) mark_many_sources(c, next);
+    }
 #ifdef MSCCLX_PROFILE
     if (threadIdx.x == 0) {
       const u64 prof_t4 = wall_clock64();

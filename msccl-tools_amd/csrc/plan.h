@@ -68,6 +68,10 @@ struct DevOp {
 static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
 constexpr uint32_t kOpHasdep = 1u << 4, kOpOutStaged = 1u << 5, kOpNtStore = 1u << 6, kOpInPlace = 1u << 7;
 constexpr int kOpCntShift = 8;
+// A run of `re` steps with one chunk each, the same destination and sources a fixed distance apart is
+// done as one step on the device -- dst = (..((dst + src0) + src1)..) + src[m-1]: an `re` whose
+// in_addr holds the distance between sources in bytes (0 for an ordinary `re`) and whose cnt holds m.
+constexpr int kMaxReduceSources = 8;
 constexpr int kMaxExtraDeps = 3;         // nop steps folded into the step that follows them, at most
 constexpr int kExtraDepWords = 2;        // one folded dependency: counter word (from the slice's first flag); step + 1 | steps per pass of that threadblock << 16
 
