@@ -62,13 +62,18 @@ def register_mi355x_plans():
     one = lambda x: x == 1
     manual = ThreadblockPolicy.manual
 
-    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=8, inplace=True, instances=1,
-                            sizes=(0, '8MB'), threadblock_policy=manual, machines=one)
-    def mi355x_ring_allreduce_small(prog, nodes):
-        allreduce_ring(size=8, channels=1)
+    # Measured on MI355X, 8 virtual ranks, fp32 (microseconds, all-pairs / ring): 4 KiB to 512 KiB per
+    # rank 20-21 / 34-36, 1 MiB 26 / 36, 4 MiB 40 / 47, 8 MiB 58 / 64, 16 MiB 98 / 100, 32 MiB 206 / 182,
+    # 256 MiB 1774 / 1375.  All-pairs is three hand-offs deep, the ring fourteen; the ring moves
+    # 5(n-1)/n chunks per chunk reduced, all-pairs about 4(n-1)/n + 2 on this executor.
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=1,
+                            sizes=(0, '16MB'), threadblock_policy=manual, interleaved_replication=False,
+                            dependence_nop=True, machines=one)
+    def mi355x_allpairs_allreduce(prog, nodes):
+        allreduce_allpairs(8)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=8, inplace=True, instances=4,
-                            sizes=('8MB', None), threadblock_policy=manual, machines=one)
+                            sizes=('16MB', None), threadblock_policy=manual, machines=one)
     def mi355x_ring_allreduce_large(prog, nodes):
         allreduce_ring(size=8, channels=1)
 

@@ -209,7 +209,7 @@ def test_init_to_run_flow(capsys):
     algos = load_config()
     ag = select(algos, "allgather", nbytes)
     ar = select(algos, "allreduce", nbytes)
-    assert ag is not None and ar is not None and ar.tables.nchunksperloop == 8
+    assert ag is not None and ar is not None and ar.tables.nchunksperloop == 64   # below 16 MB: all-pairs
     rng = np.random.default_rng(3)
     # all-gather
     x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64).astype(np.int32) for _ in range(8)]
@@ -220,12 +220,12 @@ def test_init_to_run_flow(capsys):
     ex.run(ins, outs)
     want = np.concatenate(x)
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(8))
-    # all-reduce (ring order)
+    # all-reduce (all-pairs order: own value, then the peers' in ascending order)
     y = [(rng.random(nbytes // 4, dtype=np.float32) * 2 - 1) for _ in range(8)]
     cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
     ex = Executor(ar.tables)
     ex.setup(cb, "float32")
     ins, outs, res = collective_buffers(ex.tables, cb, "float32", inputs=[torch.from_numpy(v) for v in y])
     ex.run(ins, outs)
-    want = oc.expected_allreduce(y, 8, oc.ring_allreduce_orders(8), "float32")
+    want = oc.expected_allreduce(y, 64, oc.allpairs_allreduce_orders(8), "float32")
     assert all(np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)) for r in range(8))
