@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/exec_kernel_c2_c3_c4_pmc.txt),
 # each scaled by what the same counter reads for a plain device copy of 1 GiB (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0).  Not measured for the two latency-bound workloads.
-MEASURED_TRAFFIC_BYTES = {"c2": 3763669628, "c3": 3229608997, "c4": 20821228262}
+MEASURED_TRAFFIC_BYTES = {"c2": 3763694252, "c3": 3229607986, "c4": 20822006138}
 
 def ensure_built():
     from msccl.executor import binding
