@@ -148,6 +148,22 @@ def slow_dependency_xml(ncopies):
     return _algo("slow_dependency", "custom", 0, 1, 1, 2, [_gpu(0, 1, 2, 0, [_tb(0, -1, -1, 0, tb0), _tb(1, -1, -1, 0, tb1)])])
 
 
+def reduce_chain_xml(m, stride):
+    """One rank.  Threadblock 0 folds `m` chunks of its input, `stride` chunks apart, into chunk 0 with
+    `m` reduce steps in a row (the shape of msccl-tools' msccl/programs/allreduce_allpairs.py:18-21),
+    after a nop that waits for threadblock 1's first copy; threadblock 2 does the same into chunk 1 with
+    its sources in descending order; threadblock 1 copies both results out when they are complete."""
+    last = 2 + (m - 1) * stride
+    up = [_step(0, "nop", "i", -1, "o", -1, 0, depid=1, deps=0)] + \
+         [_step(1 + k, "re", "i", 2 + k * stride, "i", 0, 1, hasdep=1 if k == m - 1 else 0) for k in range(m)]
+    down = [_step(0, "nop", "i", -1, "o", -1, 0, depid=1, deps=0)] + \
+           [_step(1 + k, "re", "i", last - k * stride, "i", 1, 1, hasdep=1 if k == m - 1 else 0) for k in range(m)]
+    out = [_step(0, "cpy", "i", 2, "o", 2, 1, hasdep=1), _step(1, "nop", "i", -1, "o", -1, 0, depid=0, deps=m),
+           _step(2, "cpy", "i", 0, "o", 0, 1, depid=2, deps=m), _step(3, "cpy", "i", 1, "o", 1, 1)]
+    return _algo("reduce_chain", "custom", 0, 1, 1, last + 1,
+                 [_gpu(0, last + 1, 3, 0, [_tb(0, -1, -1, 0, up), _tb(1, -1, -1, 0, out), _tb(2, -1, -1, 0, down)])])
+
+
 # ---- documents in the style of msccl-tools' second emitter (msccl/ncclize.py:658-718) ----------
 # inplace="0", only s / r / rrc / cpy / nop, sending and receiving threadblocks separate, one extra
 # threadblock per rank (send=recv=-1, chan 0) holding the pre/post copies, and on r / rrc steps

@@ -181,6 +181,18 @@ def test_ragged_chunk_sizes(chunk_elems, dtype):
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("knobs", [dict(), dict(slices=1, piece_bytes=4096), dict(threads=256, slices=2), dict(threads=64, slices=3)])
+@pytest.mark.parametrize("dtype,redop", [("bfloat16", "sum"), ("float32", "sum"), ("int32", "max"), ("float16", "prod")])
+@pytest.mark.parametrize("m,stride", [(7, 8), (11, 1), (2, 3)])
+def test_reduce_chains_as_one_step(m, stride, dtype, redop, knobs):
+    """Runs of reduce steps into one destination are done as one step with several sources (at most 8:
+    11 in a row make two), in the order of the IR -- which the rounding of bfloat16 sums and fp16 products
+    shows.  Sources in descending order are left step by step.  Several passes, several waves, ragged slices."""
+    xml = ir_samples.reduce_chain_xml(m, stride)
+    got, want, _, info = run_both(xml, 5000, dtype, seed=m * 10 + stride, redop=redop, **knobs)
+    assert_same(got, want)
+
+
 @pytest.mark.parametrize("knobs", [
     dict(slices=1, piece_bytes=4096, fifo_depth=2, threads=64),
     dict(slices=3, piece_bytes=16 * 7, fifo_depth=3, threads=128),
