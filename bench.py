@@ -1,22 +1,34 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X MSCCL-IR executor.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-others] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c4] [--no-others] [--no-cpu]
     python bench.py --config c4 --sweep 1048576:536870912        (message-size sweep of one algorithm)
 
 A step is one execution of the whole compiled algorithm (one launch of the executor kernel) over
-buffers already resident in HBM.  The headline workload is the ring AllGather configuration
-(8 virtual ranks, 4 instances, int32, 32 MiB per rank); the other four configurations are timed
-the same way and reported under "others".  One JSON line is printed.
+buffers already resident in HBM.  The headline workload is the largest configuration, the two-level
+AllReduce (4 x 8 = 32 virtual ranks, 2 instances, bf16, 128 MiB per rank); the other four
+configurations are timed the same way and reported under "others".  One JSON line is printed.
 
-metric/value: algbw in GB/s (nccl-tests convention, S / t) from the wall clock around exactly K
-back-to-back launches.  "roofline": algorithmic bytes per launch / average launch duration taken
-with HIP events on the launch stream over the same K launches, against the 8 TB/s HBM peak.
-"cpu_baseline": the NumPy interpreter of the same IR on this box's host cores (reported, not a target).
+Timing.  The all-reduce programs run in place, so a launch consumes its input: the send buffers are
+restored from a pristine copy before every launch, outside the timed region, and every timed launch
+reduces the same finite random data as the verified one.  Each of the K timed steps is bracketed by
+a device synchronisation on both sides (wall clock) and by HIP events on the launch stream (kernel
+time); ms_per_step and `value` are the mean of the K wall-clock intervals, `roofline` uses the mean
+of the K event intervals.  The result of the LAST timed launch is verified as well as the first.
+The all-gather and all-to-all programs do not consume their input; they are timed the same way.
+"kernel_ms_queued" is the mean event interval of K more launches queued without host
+synchronisation in between (restores in stream order): a launch on a stream that is kept busy,
+which matters for the two latency-bound workloads (a launch on an idle GPU pays its dispatch).
+
+metric/value: algbw in GB/s (nccl-tests convention, S / t).  "roofline": algorithmic bytes per launch
+/ mean launch duration against the 8 TB/s HBM peak.  "cpu_baseline": the NumPy interpreter of the
+same IR on this box's host cores (reported, not a target).  "host_us": what a caller pays on the host
+for plan creation, configuration, binding and launching.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,10 +38,23 @@ for p in (ROOT, os.path.join(ROOT, "msccl-tools_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/exec_kernel_c2_c3_c4_pmc.txt),
-# each scaled by what the same counter reads for a plain device copy of 1 GiB (FETCH_SIZE x 2.0,
-# WRITE_SIZE x 1.0).  Not measured for the two latency-bound workloads.
-MEASURED_TRAFFIC_BYTES = {"c2": 3763694252, "c3": 3229607986, "c4": 20822006138}
+PMC_SUMMARY = os.path.join(ROOT, "profiles", "exec_kernel_c2_c3_c4_pmc.txt")
+ROOFLINE_NOTE = ("achieved = algorithmic bytes per launch / mean launch duration (HIP events); traffic = rocprofv3 FETCH_SIZE + "
+                 "WRITE_SIZE per launch, counted between L2 and the fabric, so reads served by the memory-side cache are "
+                 "included: the fraction is algorithmic bytes over the HBM peak, not proven DRAM traffic")
+
+
+def measured_traffic():
+    """HBM-side bytes per launch from the committed rocprofv3 --pmc summary (lines 'cN: traffic = B bytes per launch')."""
+    out = {}
+    try:
+        text = open(PMC_SUMMARY).read()
+    except OSError:
+        return out
+    for key, val in re.findall(r"^\s*(c\d) traffic = (\d+) bytes per launch", text, re.M):
+        out[key] = int(val)
+    return out
+
 
 def ensure_built():
     from msccl.executor import binding
@@ -74,6 +99,8 @@ def fold_orders(key):
     if key in ("c1", "c5"):
         n = 8 if key == "c1" else 64
         return [[(k + j) % n for j in range(n)] for k in range(n)]
+    if key == "c5_chain":
+        return [list(range(64))]
     if key == "c4":
         L, N = 8, 4
         one = []
@@ -84,38 +111,92 @@ def fold_orders(key):
     return None
 
 
-def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None):
+def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_costs=False):
     import torch
-    from msccl.executor import Executor, collective_buffers
+    from msccl.executor import Executor, collective_buffers, parse_algo_xml
     from msccl.executor.workloads import WORKLOADS, torch_input
     w = WORKLOADS[key] if bytes_per_rank is None else WORKLOADS[key].scaled(bytes_per_rank)
     xml = WORKLOADS[key].build()
-    ex = Executor(xml, device=device)
+    host = {}
+    t0 = time.perf_counter()
+    tables = parse_algo_xml(xml)
+    host["parse_xml"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    ex = Executor(tables, device=device)
+    host["plan_create"] = time.perf_counter() - t0
     info = ex.setup(w.chunk_bytes, w.dtype)
+    host["configure"] = ex.host_seconds["configure"]
     x = [torch_input(w, r, device) for r in range(w.ranks)]
     ins, outs, res = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, device=device, inputs=x)
-    ex.run(ins, outs)  # first execution from pristine inputs: the one that is verified
+    consumes_input = w.coll == "allreduce"   # in place: a launch overwrites what it reads
+
+    def restore():
+        if consumes_input:
+            for r in range(w.ranks):
+                res[r][:x[r].numel()].copy_(x[r])
+
+    torch.cuda.synchronize()
+    ex.bind(ins, outs)
+    host["bind_first"] = ex.host_seconds["bind"]
+    ex.launch()  # first execution from pristine inputs
+    ex.wait()
     torch.cuda.synchronize()
     ok = verify(w, x, res, fold_orders(key)) if bytes_per_rank is None else None  # the closed forms are written for the full size
+    if host_costs:
+        # a second set of buffers, then the first again: what a caller that passes fresh tensors pays per call
+        ins2, outs2, _ = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, device=device, inputs=None)
+        torch.cuda.synchronize()
+        ex.bind(ins2, outs2)
+        host["bind_again"] = ex.host_seconds["bind"]
+        ex.bind(ins, outs)
+        host["bind_again"] = min(host["bind_again"], ex.host_seconds["bind"])
+        del ins2, outs2
     for _ in range(warmup):
+        restore()
         ex.launch()
     ex.wait()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)  # on the launch stream
-    t0 = time.perf_counter()
-    e0.record()
+    wall, events, launch_host = [], [], []
     for _ in range(steps):
+        restore()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)  # on the launch stream
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
         ex.launch()
-    e1.record()
+        t_l = time.perf_counter()
+        e1.record()
+        ex.wait()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        wall.append(t1 - t0)
+        launch_host.append(t_l - t0)
+        events.append(e0.elapsed_time(e1) * 1e-3)
+    ok_last = verify(w, x, res, fold_orders(key)) if bytes_per_rank is None else None
+    # the same K launches queued behind each other (restores in between, in stream order, no host
+    # synchronisation until the end): what a caller sees whose stream is kept busy
+    pairs = []
+    for _ in range(steps):
+        restore()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        ex.launch()
+        e1.record()
+        pairs.append((e0, e1))
     ex.wait()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_s = (t1 - t0) / steps
-    kernel_s = e0.elapsed_time(e1) * 1e-3 / steps
+    queued_s = sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / steps
+    host["launch"] = sorted(launch_host)[len(launch_host) // 2]
+    wall_s = sum(wall) / steps
+    kernel_s = sum(events) / steps
     ab = ex.algorithmic_bytes()
     out = {"workload": w.description, "dtype": w.dtype, "ranks": w.ranks, "bytes_per_rank": w.bytes_per_rank,
-           "ms_per_step": wall_s * 1e3, "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": ab, "verified": None if ok is None else bool(ok),
-           "geometry": {k: v for k, v in info.as_dict().items() if k in ("workgroups", "threads", "slices", "piece_bytes", "fifo_depth", "passes")}}
+           "ms_per_step": wall_s * 1e3, "kernel_ms": kernel_s * 1e3, "kernel_ms_min": min(events) * 1e3, "kernel_ms_max": max(events) * 1e3,
+           "kernel_ms_queued": queued_s * 1e3,
+           "algorithmic_bytes": ab,
+           "verified": None if ok is None else bool(ok and ok_last), "inputs_restored_before_every_launch": consumes_input,
+           "geometry": {k: v for k, v in info.as_dict().items() if k in ("workgroups", "threads", "slices", "piece_bytes", "fifo_depth", "passes")},
+           "host_us": {k: round(v * 1e6, 1) for k, v in host.items()}}
     out.update({k: round(v, 4) for k, v in w.bandwidths(wall_s, ab).items()})
     out["roofline_frac_kernel"] = round(ab / kernel_s / 1e9 / HBM_PEAK_GBPS, 4)
     del x, ins, outs, res, ex
@@ -123,8 +204,8 @@ def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None):
     return out
 
 
-# per-rank bytes of the CPU sample: the full headline workload, bounded samples of the heavier ones
-CPU_SAMPLE_BYTES = {"c1": 1 << 20, "c2": 32 << 20, "c3": 16 << 20, "c4": 4 << 20, "c5": 256 << 10}
+# per-rank bytes of the CPU sample: bounded samples of the same algorithms (10 to 30 s of host work where the workload is large enough)
+CPU_SAMPLE_BYTES = {"c1": 1 << 20, "c2": 32 << 20, "c3": 64 << 20, "c4": 16 << 20, "c5": 256 << 10, "c5_chain": 256 << 10}
 
 
 def cpu_baseline(key):
@@ -140,7 +221,8 @@ def cpu_baseline(key):
     E = w.chunk_bytes // esz
     x = [numpy_input(w, r) for r in range(w.ranks)]
     best = None
-    for _ in range(2):
+    runs = 2
+    for _ in range(runs):
         bufs = oc.place_inputs(algo, x, E, w.dtype)
         t0 = time.perf_counter()
         oi.Interpreter(algo).run(bufs, E, w.dtype)
@@ -153,17 +235,18 @@ def cpu_baseline(key):
     except AttributeError:
         cores = os.cpu_count()
     return {"value": round(bw["algbw_GBps"], 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{w.bytes_per_rank} of {full.bytes_per_rank} bytes per rank, best of 2 runs, {best:.3f} s; single Python "
-                      f"process (NumPy memcpy/ufuncs are single-threaded); host offers {cores} cores",
+            "sample": f"{w.description.split(';')[0]}; {w.bytes_per_rank} of {full.bytes_per_rank} bytes per rank, best of {runs} runs, "
+                      f"{best:.3f} s; single Python process (NumPy memcpy/ufuncs are single-threaded); host offers {cores} cores",
             "algorithmic_GBps": round(bw["algorithmic_GBps"], 4)}
 
 
 def main():
+    from msccl.executor.workloads import WORKLOADS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy baseline")
     ap.add_argument("--sweep", metavar="LO:HI", help="instead of the benchmark line: time the chosen algorithm on LO, 2*LO, ... HI bytes per "
@@ -202,29 +285,34 @@ def main():
             size *= 2
         print(json.dumps({"sweep": args.config, "workload": r["workload"].split(";")[0], "dtype": r["dtype"], "steps": args.steps, "rows": rows}))
         return
-    head = run_workload(args.config, args.steps, args.warmup)
-    traffic = MEASURED_TRAFFIC_BYTES.get(args.config)
+    traffic = measured_traffic()
+    head = run_workload(args.config, args.steps, args.warmup, host_costs=True)
     line = {
         "metric": "algbw_GBps", "value": head["algbw_GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"int32": "i32", "uint8": "u8", "float32": "f32", "bfloat16": "bf16", "float16": "f16"}[head["dtype"]],
         "data": "synthetic", "config": {"workload": head["workload"], "virtual_ranks": head["ranks"], **head["geometry"]},
         "busbw_GBps": head["busbw_GBps"], "hbm_fraction": head["hbm_fraction"], "verified": head["verified"],
+        "timing": "every timed launch starts from restored inputs (restore untimed) and is bracketed by a device synchronisation on both sides"
+                  if head["inputs_restored_before_every_launch"] else "every timed launch is bracketed by a device synchronisation on both sides",
         "roofline": {"bound": "hbm", "achieved": round(head["algorithmic_bytes"] / (head["kernel_ms"] * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": head["roofline_frac_kernel"], "traffic": traffic,
-                     "kernel": "exec_kernel", "algorithmic_bytes_per_launch": head["algorithmic_bytes"], "kernel_ms": round(head["kernel_ms"], 5)},
+                     "unit": "GB/s", "frac": head["roofline_frac_kernel"], "traffic": traffic.get(args.config),
+                     "kernel": "exec_kernel", "algorithmic_bytes_per_launch": head["algorithmic_bytes"], "kernel_ms": round(head["kernel_ms"], 5),
+                     "kernel_ms_min": round(head["kernel_ms_min"], 5), "kernel_ms_max": round(head["kernel_ms_max"], 5),
+                     "kernel_ms_queued": round(head["kernel_ms_queued"], 5), "note": ROOFLINE_NOTE},
+        "host_us": head["host_us"],
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.config)
     if not args.no_others:
         line["others"] = {}
-        for key in ("c1", "c2", "c3", "c4", "c5"):
+        for key in sorted(WORKLOADS):
             if key == args.config:
                 continue
-            r = run_workload(key, max(5, args.steps // 2), args.warmup)
+            r = run_workload(key, max(5, args.steps // 2), args.warmup, host_costs=key in ("c4", "c5"))
             line["others"][key] = {k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items() if k != "geometry"}
             line["others"][key].update(r["geometry"])
-            line["others"][key]["traffic"] = MEASURED_TRAFFIC_BYTES.get(key)
+            line["others"][key]["traffic"] = traffic.get(key)
     print(json.dumps(line))
 
 

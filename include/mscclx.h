@@ -13,8 +13,14 @@
  * tables and their device copies) and never frees caller memory.
  * Errors: 0 on success, a negative mscclx_error otherwise; mscclx_last_error() returns the text of
  * the calling thread's last failure.  No exception crosses the ABI.
- * Threading: a plan is not thread-safe; launches are stream-ordered; at most one launch of a plan
- * may be in flight.
+ * Threading: a plan is not thread-safe; launches are stream-ordered; launches of one plan must all
+ * go to the same stream, and bind/configure only while none is in flight.
+ * Residency: a launch is one grid of workgroups that wait for each other, sized at configure time to
+ * what an otherwise idle GPU keeps resident.  The stream must therefore have the GPU to itself for
+ * the duration of a launch: a kernel of another stream that occupies compute units can keep part of
+ * the grid from starting, and the part that runs then waits until the in-kernel watchdog ends the
+ * launch with MSCCLX_ERR_TIMEOUT (never a hang).  mscclx_config.workgroups caps the grid for callers
+ * that share the GPU on purpose.
  */
 #ifndef MSCCLX_H
 #define MSCCLX_H
@@ -26,7 +32,7 @@
 extern "C" {
 #endif
 
-#define MSCCLX_VERSION 2
+#define MSCCLX_VERSION 3
 
 typedef enum {
   MSCCLX_OK = 0,
@@ -37,7 +43,9 @@ typedef enum {
   MSCCLX_ERR_HIP = -5,         /* a HIP runtime call failed                                      */
   MSCCLX_ERR_TIMEOUT = -6,     /* the in-kernel watchdog expired while a step was waiting        */
   MSCCLX_ERR_STATE = -7,       /* call order violated (launch before bind, ...)                  */
-  MSCCLX_ERR_UNSUPPORTED = -8
+  MSCCLX_ERR_UNSUPPORTED = -8,
+  MSCCLX_ERR_ABORTED = -9,     /* mscclx_plan_abort ended the launch                              */
+  MSCCLX_ERR_ALIASED = -10     /* rank buffers overlap in memory but the plan reads payloads in place */
 } mscclx_error;
 
 /* <step type=...>: msccl/language/ir.py:69-83 (the 'd' and 'st' members are never emitted). */
@@ -158,7 +166,10 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
 
 /* Attaches device memory: in/out/scratch[r] are rank r's buffers of i/o/s_chunks * chunk_bytes
  * bytes (may be NULL where the extent is 0; in == out aliasing is the caller's choice, as with an
- * in-place NCCL call).  Uploads the plan tables to the current device and clears the workspace. */
+ * in-place NCCL call; buffers that overlap in memory need a plan configured with staging=1, else
+ * MSCCLX_ERR_ALIASED).  Uploads the plan tables to the current device and clears the workspace.
+ * Binding again after a launch has been waited for (new buffers, same geometry) re-uses the
+ * device-side allocations: one upload of the tables, no allocation. */
 int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void* const* scratch,
                      void* workspace, size_t workspace_bytes);
 
@@ -166,6 +177,14 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
 int mscclx_plan_launch(mscclx_plan* plan, void* stream);
 /* Waits for `stream` and reports how the last launch ended. */
 int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status);
+/* The same without blocking: 1 while work is still queued or running on `stream` (a watchdog report
+ * that has already arrived is copied to `status`), else what mscclx_plan_wait would return. */
+int mscclx_plan_poll(mscclx_plan* plan, void* stream, mscclx_status* status);
+/* Asks the running launch (and any launch of this plan queued behind it) to give up: every
+ * workgroup sees the request while it polls and leaves, every wave exits normally.  Returns once
+ * the request is on the device; mscclx_plan_wait then returns MSCCLX_ERR_ABORTED, the rank buffers
+ * hold partial results, and the next launch re-arms the counters. */
+int mscclx_plan_abort(mscclx_plan* plan);
 /* Times `iters` back-to-back launches with HIP events on `stream`; ms_out[i] = duration of launch i. */
 int mscclx_plan_time(mscclx_plan* plan, void* stream, int32_t iters, float* ms_out);
 

@@ -41,38 +41,47 @@ static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll, bool fold) {
   }
 }
 
-struct DeviceState {
-  int device = -1;
-  DevTb* tbs = nullptr;
-  DevOp* ops = nullptr;
-  DevConn* conns = nullptr;
-  uint32_t* extra_deps = nullptr;
+// Everything the kernel reads about the program, packed into one block of bytes that is uploaded in
+// one copy: threadblocks | steps | folded dependencies | connections | hosting table.
+struct DeviceImage {
+  std::vector<unsigned char> bytes;
+  size_t off_tbs = 0, off_ops = 0, off_extras = 0, off_conns = 0, off_hosting = 0;
+  size_t hosting_wg_words = 0, hosting_ctx_words = 0;
   std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
   std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
-  int32_t* hosting = nullptr;            // wg_begin | ctx_tb | ctx_slice
+  kernel_fn kernel = nullptr;
+};
+
+struct DeviceState {
+  int device = -1;
+  bool ready = false;                    // every table is uploaded and the workspace is armed
+  unsigned char* tables = nullptr;       // device copy of DeviceImage::bytes
+  size_t tables_capacity = 0;
+  DeviceImage image;                     // (bytes are dropped after the upload)
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
-  kernel_fn kernel = nullptr;
-  bool dirty = false;  // counters must be cleared before the next launch (after a failed launch)
+  bool dirty = false;  // counters must be cleared before the next launch (after a failed or aborted launch)
+  bool abort_requested = false;
+  hipStream_t side = nullptr;            // for the host's abort request while the launch stream is busy
+  unsigned long long* abort_word_host = nullptr;  // pinned source of that request
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   unsigned long long* prof = nullptr;  // MSCCLX_PROFILE builds: kProfWords words per workgroup
 };
 
 void destroy_device_state(DeviceState* d) {
   if (!d) return;
-  if (d->tbs) (void)hipFree(d->tbs);
-  if (d->ops) (void)hipFree(d->ops);
-  if (d->conns) (void)hipFree(d->conns);
-  if (d->extra_deps) (void)hipFree(d->extra_deps);
-  if (d->hosting) (void)hipFree(d->hosting);
+  if (d->tables) (void)hipFree(d->tables);
+  if (d->prof) (void)hipFree(d->prof);
   if (d->host_status) (void)hipHostFree(d->host_status);
+  if (d->abort_word_host) (void)hipHostFree(d->abort_word_host);
+  if (d->side) (void)hipStreamDestroy(d->side);
   if (d->ev0) (void)hipEventDestroy(d->ev0);
   if (d->ev1) (void)hipEventDestroy(d->ev1);
   delete d;
 }
 
 // A nop that nobody depends on and that is not its threadblock's last step can be folded into the
-// step after it (mscclx_plan_bind).
+// step after it (build_image).
 static bool has_foldable_nops(const mscclx_plan& plan) {
   for (const Tb& tb : plan.tbs)
     for (int o = tb.op_begin; o + 1 < tb.op_end; ++o)
@@ -95,105 +104,55 @@ static int query_capacity(kernel_fn k, int* num_cus, int capacity[4]) {
   return MSCCLX_OK;
 }
 
-}  // namespace mscclx
-
-using namespace mscclx;
-
-extern "C" {
-
-int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, int32_t redop, const mscclx_config* cfg_in, mscclx_info* info) {
-  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
-  mscclx_config cfg = {};
-  if (cfg_in) cfg = *cfg_in;
-  if (dtype < 0 || dtype >= MSCCLX_NUM_DTYPES) return fail(MSCCLX_ERR_INVALID_ARG, "unknown dtype");
-  if (redop < 0 || redop >= MSCCLX_NUM_REDOPS) return fail(MSCCLX_ERR_INVALID_ARG, "unknown reduction");
-  const int elem = dtype_size(dtype);
-  if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
-  const bool vec = chunk_bytes % 16 == 0;
-  int num_cus = 256;
-  int capacity[4];
-  if (cfg.max_workgroups > 0) {
-    for (int i = 0; i < 4; ++i) capacity[i] = cfg.max_workgroups;
-  } else {
-    const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
-    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, vec && !ll && has_foldable_nops(*plan)), &num_cus, capacity);
-    if (rc) return rc;
-  }
-  Geometry g;
-  const uint64_t fifo_budget = 4ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes
-  int rc = decide_geometry(*plan, chunk_bytes, dtype, cfg, num_cus, capacity, fifo_budget, &g);
-  if (rc) return rc;
-  plan->geo = std::move(g);
-  const Geometry& gg = plan->geo;
-  plan->chunk_bytes = chunk_bytes;
-  plan->dtype = dtype;
-  plan->redop = redop;
-  plan->timeout_ms = cfg.timeout_ms > 0 ? cfg.timeout_ms : 10000;
-  plan->configured = true;
-  if (plan->dev) { destroy_device_state(plan->dev); plan->dev = nullptr; }
-  if (info) {
-    const Geometry& g = gg;
-    info->workgroups = g.workgroups;
-    info->max_hosted = g.max_hosted;
-    info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
-    info->threads = g.threads;
-    info->slices = g.slices;
-    info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);
-    info->fifo_depth = g.depth;
-    info->passes = g.passes;
-    info->connections = (int32_t)plan->conns.size();
-    info->vector_path = g.vector_path;
-    info->zero_copy_messages = 0;
-    info->staged_messages = 0;
-    for (const Op& op : plan->ops)
-      if (is_send_type(op.type)) ((!g.staging && op.zero_copy) ? info->zero_copy_messages : info->staged_messages)++;
-    info->workspace_bytes = g.workspace_bytes;
-    info->algorithmic_units = plan->algorithmic_units;
-  }
-  return MSCCLX_OK;
-}
-
-int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void* const* scratch, void* workspace, size_t workspace_bytes) {
-  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
-  if (!plan->configured) return fail(MSCCLX_ERR_STATE, "configure the plan before binding buffers");
-  const Geometry& g = plan->geo;
-  if (!workspace || workspace_bytes < g.workspace_bytes)
-    return fail(MSCCLX_ERR_CAPACITY, "workspace of " + std::to_string(workspace_bytes) + " bytes given, " + std::to_string(g.workspace_bytes) + " needed");
-  if ((uintptr_t)workspace % 256) return fail(MSCCLX_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
-  std::vector<void*> bufs((size_t)plan->nranks * 3, nullptr);
+// The caller's rank buffers as one table [rank][i, o, s]; refuses what the kernels cannot address.
+static int collect_buffers(const mscclx_plan& plan, void* const* in, void* const* out, void* const* scratch, std::vector<void*>* bufs_out) {
+  const Geometry& g = plan.geo;
+  std::vector<void*> bufs((size_t)plan.nranks * 3, nullptr);
   void* const* tables[3] = {in, out, scratch};
-  for (int r = 0; r < plan->nranks; ++r)
+  for (int r = 0; r < plan.nranks; ++r)
     for (int b = 0; b < 3; ++b) {
       void* ptr = tables[b] ? tables[b][r] : nullptr;
-      if (plan->rank_chunks[(size_t)r * 3 + b] > 0) {
+      if (plan.rank_chunks[(size_t)r * 3 + b] > 0) {
         if (!ptr) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer " + "ios"[b] + " is used by the algorithm but NULL was given");
         if (g.vector_path && (uintptr_t)ptr % 16) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffers must be 16-byte aligned");
-        if ((uintptr_t)ptr % dtype_size(plan->dtype)) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer not aligned to its element type");
+        if ((uintptr_t)ptr % dtype_size(plan.dtype)) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer not aligned to its element type");
       }
       bufs[(size_t)r * 3 + b] = ptr;
     }
-
   if (!g.staging) {
     // reading payloads in place assumes that distinct buffers are distinct memory
     std::vector<std::pair<uintptr_t, uintptr_t>> spans;
-    for (int r = 0; r < plan->nranks; ++r)
+    for (int r = 0; r < plan.nranks; ++r)
       for (int b = 0; b < 3; ++b) {
-        const size_t len = (size_t)plan->rank_chunks[(size_t)r * 3 + b] * plan->chunk_bytes;
+        const size_t len = (size_t)plan.rank_chunks[(size_t)r * 3 + b] * plan.chunk_bytes;
         if (len) spans.push_back({(uintptr_t)bufs[(size_t)r * 3 + b], (uintptr_t)bufs[(size_t)r * 3 + b] + len});
       }
     std::sort(spans.begin(), spans.end());
     for (size_t k = 1; k < spans.size(); ++k)
       if (spans[k].first < spans[k - 1].second)
-        return fail(MSCCLX_ERR_INVALID_ARG, "rank buffers overlap in memory; configure the plan with staging=1 for aliased buffers");
+        return fail(MSCCLX_ERR_ALIASED, "rank buffers overlap in memory; configure the plan with staging=1 for aliased buffers");
   }
-  if (plan->dev) { destroy_device_state(plan->dev); plan->dev = nullptr; }
-  DeviceState* d = new DeviceState();
-  plan->dev = d;
-  HIP_TRY(hipGetDevice(&d->device));
-  const bool fold = g.vector_path && !g.ll && has_foldable_nops(*plan);
-  d->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0, fold);
-  if (!d->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
+  bufs_out->swap(bufs);
+  return MSCCLX_OK;
+}
 
+template <typename T>
+static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<T>& v, size_t at_least = 1) {
+  const size_t off = (bytes.size() + 255) / 256 * 256;
+  const size_t n = std::max(v.size(), at_least);
+  bytes.resize(off + n * sizeof(T), 0);
+  if (!v.empty()) std::memcpy(bytes.data() + off, v.data(), v.size() * sizeof(T));
+  return off;
+}
+
+// The device's tables for the configured geometry and these buffers.  Pure host work.
+static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bufs, DeviceImage* img) {
+  const mscclx_plan* plan = &plan_ref;
+  const Geometry& g = plan->geo;
+  const bool fold = g.vector_path && !g.ll && has_foldable_nops(*plan);
+  img->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0, fold);
+  if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
+  DeviceImage* d = img;
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
   std::vector<DevTb> htb(ntb);
   std::vector<DevOp> hop(nop);
@@ -335,61 +294,39 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
     hop.swap(fused);
     d->dev_ir_step.swap(fused_ir);
   }
-  const size_t ndev = hop.size();
-  HIP_TRY(hipMalloc((void**)&d->tbs, sizeof(DevTb) * (ntb ? ntb : 1)));
-  HIP_TRY(hipMalloc((void**)&d->ops, sizeof(DevOp) * (ndev ? ndev : 1)));
-  HIP_TRY(hipMalloc((void**)&d->extra_deps, sizeof(uint32_t) * (extras.empty() ? kExtraDepWords : extras.size())));
-  if (!extras.empty()) HIP_TRY(hipMemcpy(d->extra_deps, extras.data(), sizeof(uint32_t) * extras.size(), hipMemcpyHostToDevice));
-  HIP_TRY(hipMalloc((void**)&d->conns, sizeof(DevConn) * hcn.size()));
-  HIP_TRY(hipMemcpy(d->tbs, htb.data(), sizeof(DevTb) * ntb, hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(d->ops, hop.data(), sizeof(DevOp) * ndev, hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(d->conns, hcn.data(), sizeof(DevConn) * hcn.size(), hipMemcpyHostToDevice));
-  {
-    std::vector<int32_t> table(g.wg_begin);
-    table.insert(table.end(), g.ctx_tb.begin(), g.ctx_tb.end());
-    table.insert(table.end(), g.ctx_slice.begin(), g.ctx_slice.end());
-    HIP_TRY(hipMalloc((void**)&d->hosting, sizeof(int32_t) * table.size()));
-    HIP_TRY(hipMemcpy(d->hosting, table.data(), sizeof(int32_t) * table.size(), hipMemcpyHostToDevice));
-  }
-  HIP_TRY(hipHostMalloc((void**)&d->host_status, sizeof(mscclx_status), hipHostMallocDefault));
-  std::memset(d->host_status, 0, sizeof(mscclx_status));
-  d->workspace = (unsigned char*)workspace;
-  // both counter areas; LL: the slots too, so that no line of whatever the memory held carries a flag
-  HIP_TRY(hipMemset(d->workspace, 0, g.ll ? g.workspace_bytes : g.fifo_byte_off));
-  HIP_TRY(hipDeviceSynchronize());
-  HIP_TRY(hipEventCreate(&d->ev0));
-  HIP_TRY(hipEventCreate(&d->ev1));
-#ifdef MSCCLX_PROFILE
-  HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * kProfWords * g.workgroups));
-  HIP_TRY(hipMemset(d->prof, 0, sizeof(unsigned long long) * kProfWords * g.workgroups));
-#endif
+  std::vector<int32_t> hosting(g.wg_begin);
+  hosting.insert(hosting.end(), g.ctx_tb.begin(), g.ctx_tb.end());
+  hosting.insert(hosting.end(), g.ctx_slice.begin(), g.ctx_slice.end());
+  img->hosting_wg_words = g.wg_begin.size();
+  img->hosting_ctx_words = g.ctx_tb.size();
+  img->bytes.clear();
+  img->off_tbs = append_table(img->bytes, htb);
+  img->off_ops = append_table(img->bytes, hop);
+  img->off_extras = append_table(img->bytes, extras, kExtraDepWords);
+  img->off_conns = append_table(img->bytes, hcn);
+  img->off_hosting = append_table(img->bytes, hosting);
   return MSCCLX_OK;
 }
 
-int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
-  if (!plan || !plan->dev || !plan->dev->kernel) return fail(MSCCLX_ERR_STATE, "bind buffers before launching");
-  DeviceState* d = plan->dev;
-  const Geometry& g = plan->geo;
-  hipStream_t s = (hipStream_t)stream;
-  if (d->dirty) {  // the previous launch gave up half-way: its counters mean nothing
-    HIP_TRY(hipStreamSynchronize(s));
-    HIP_TRY(hipMemset(d->workspace, 0, g.ll ? g.workspace_bytes : g.fifo_byte_off));  // LL: launches count from 0 again, old lines must go
-    HIP_TRY(hipDeviceSynchronize());
-    d->dirty = false;
-  }
+// Kernel arguments for tables at `tables` (a device copy of img.bytes) and a workspace.
+static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img, const unsigned char* tables, unsigned char* workspace,
+                                mscclx_status* status, unsigned long long* prof) {
+  const Geometry& g = plan.geo;
   KernelParams kp;
-  kp.tbs = d->tbs; kp.ops = d->ops; kp.conns = d->conns; kp.extra_deps = d->extra_deps;
-  unsigned long long* sync = (unsigned long long*)d->workspace;
-  kp.sync_base = sync;
+  kp.tbs = (const DevTb*)(tables + img.off_tbs);
+  kp.ops = (const DevOp*)(tables + img.off_ops);
+  kp.conns = (const DevConn*)(tables + img.off_conns);
+  kp.extra_deps = (const uint32_t*)(tables + img.off_extras);
+  kp.sync_base = (unsigned long long*)workspace;
   kp.sync_cur = kp.sync_nxt = nullptr;
   kp.sync_words = g.sync_words;
-  kp.fifo = d->workspace + g.fifo_byte_off;
-  kp.host_status = d->host_status;
-  kp.prof = d->prof;
+  kp.fifo = workspace + g.fifo_byte_off;
+  kp.host_status = status;
+  kp.prof = prof;
   kp.chunk_units = g.chunk_units;
   kp.slice_fifo_units = g.slice_fifo_units;
   kp.sync_slice_words = g.sync_slice_words;
-  kp.timeout_ticks = (uint64_t)plan->timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
+  kp.timeout_ticks = (uint64_t)plan.timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
   kp.slice_grain = g.slice_grain;
   {  // groups of about sqrt(workgroups), at most kFinishGroups of them
@@ -398,31 +335,178 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
     per = std::max<uint32_t>(per, ((uint32_t)g.workgroups + kFinishGroups - 1) / kFinishGroups);
     kp.finish_group = per;
   }
-  kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan->tbs.size(); kp.nconns = (int)plan->conns.size();
-  kp.wg_begin = d->hosting;
-  kp.ctx_tb = d->hosting + g.wg_begin.size();
-  kp.ctx_slice = kp.ctx_tb + g.ctx_tb.size();
-  const unsigned grid = (unsigned)g.workgroups;
-  hipLaunchKernelGGL(d->kernel, dim3(grid), dim3(g.threads), 0, s, kp);
+  kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan.tbs.size(); kp.nconns = (int)plan.conns.size();
+  kp.wg_begin = (const int32_t*)(tables + img.off_hosting);
+  kp.ctx_tb = kp.wg_begin + img.hosting_wg_words;
+  kp.ctx_slice = kp.ctx_tb + img.hosting_ctx_words;
+  return kp;
+}
+
+// Bytes of the workspace that must read zero before the first launch: both counter areas; LL: the
+// slots too, so that no line of whatever the memory held carries a flag.
+static size_t armed_bytes(const Geometry& g) { return g.ll ? g.workspace_bytes : g.fifo_byte_off; }
+
+// How a finished launch ended, as the IR counts steps.
+static int report_status(const mscclx_plan& plan, const DeviceImage& img, mscclx_status st, mscclx_status* status_out) {
+  if (st.code != MSCCLX_OK && st.tb >= 0 && (size_t)st.tb < img.dev_op_begin.size()) {
+    // the kernel counts the steps of its own list, in which runs of nops are folded: report the IR's step
+    const size_t at = (size_t)img.dev_op_begin[(size_t)st.tb] + (size_t)std::max(st.step, 0);
+    if (at < img.dev_ir_step.size()) st.step = img.dev_ir_step[at];
+  }
+  if (status_out) *status_out = st;
+  if (st.code == MSCCLX_OK) return MSCCLX_OK;
+  if (st.tb < 0 || (size_t)st.tb >= plan.tbs.size()) return fail(st.code, "the launch failed (no step was named)");
+  const Tb& tb = plan.tbs[(size_t)st.tb];
+  static const char* what[] = {"its dependency", "an incoming message", "a free slot on its outgoing connection", "?"};
+  return fail(st.code, "watchdog: rank " + std::to_string(tb.rank) + " tb " + std::to_string(tb.local_id) + " step " + std::to_string(st.step) +
+                           " (slice " + std::to_string(st.slice) + ", pass " + std::to_string(st.pass) + ") waited more than " +
+                           std::to_string(plan.timeout_ms) + " ms for " + what[st.waiting_on & 3]);
+}
+
+}  // namespace mscclx
+
+using namespace mscclx;
+
+extern "C" {
+
+int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, int32_t redop, const mscclx_config* cfg_in, mscclx_info* info) {
+  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
+  mscclx_config cfg = {};
+  if (cfg_in) cfg = *cfg_in;
+  if (dtype < 0 || dtype >= MSCCLX_NUM_DTYPES) return fail(MSCCLX_ERR_INVALID_ARG, "unknown dtype");
+  if (redop < 0 || redop >= MSCCLX_NUM_REDOPS) return fail(MSCCLX_ERR_INVALID_ARG, "unknown reduction");
+  const int elem = dtype_size(dtype);
+  if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
+  const bool vec = chunk_bytes % 16 == 0;
+  int num_cus = 256;
+  int capacity[4];
+  if (cfg.max_workgroups > 0) {
+    for (int i = 0; i < 4; ++i) capacity[i] = cfg.max_workgroups;
+  } else {
+    const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
+    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, vec && !ll && has_foldable_nops(*plan)), &num_cus, capacity);
+    if (rc) return rc;
+  }
+  Geometry g;
+  const uint64_t fifo_budget = 4ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes
+  int rc = decide_geometry(*plan, chunk_bytes, dtype, cfg, num_cus, capacity, fifo_budget, &g);
+  if (rc) return rc;
+  plan->geo = std::move(g);
+  const Geometry& gg = plan->geo;
+  plan->chunk_bytes = chunk_bytes;
+  plan->dtype = dtype;
+  plan->redop = redop;
+  plan->timeout_ms = cfg.timeout_ms > 0 ? cfg.timeout_ms : 10000;
+  plan->configured = true;
+  if (plan->dev) { destroy_device_state(plan->dev); plan->dev = nullptr; }
+  if (info) {
+    const Geometry& g = gg;
+    info->workgroups = g.workgroups;
+    info->max_hosted = g.max_hosted;
+    info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
+    info->threads = g.threads;
+    info->slices = g.slices;
+    info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);
+    info->fifo_depth = g.depth;
+    info->passes = g.passes;
+    info->connections = (int32_t)plan->conns.size();
+    info->vector_path = g.vector_path;
+    info->zero_copy_messages = 0;
+    info->staged_messages = 0;
+    for (const Op& op : plan->ops)
+      if (is_send_type(op.type)) ((!g.staging && op.zero_copy) ? info->zero_copy_messages : info->staged_messages)++;
+    info->workspace_bytes = g.workspace_bytes;
+    info->algorithmic_units = plan->algorithmic_units;
+  }
+  return MSCCLX_OK;
+}
+
+int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void* const* scratch, void* workspace, size_t workspace_bytes) {
+  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
+  if (!plan->configured) return fail(MSCCLX_ERR_STATE, "configure the plan before binding buffers");
+  const Geometry& g = plan->geo;
+  if (!workspace || workspace_bytes < g.workspace_bytes)
+    return fail(MSCCLX_ERR_CAPACITY, "workspace of " + std::to_string(workspace_bytes) + " bytes given, " + std::to_string(g.workspace_bytes) + " needed");
+  if ((uintptr_t)workspace % 256) return fail(MSCCLX_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
+  std::vector<void*> bufs;
+  int rc = collect_buffers(*plan, in, out, scratch, &bufs);
+  if (rc) return rc;
+  DeviceImage img;
+  rc = build_image(*plan, bufs, &img);
+  if (rc) return rc;
+
+  // The plan keeps its device state across binds of the same geometry (configure drops it): a new
+  // set of buffers then costs one upload of the tables.  The state is built aside and handed to the
+  // plan only when every call has succeeded, so a failed bind leaves nothing a launch could use.
+  int device = -1;
+  HIP_TRY(hipGetDevice(&device));
+  DeviceState* d = plan->dev;
+  plan->dev = nullptr;
+  if (d && (d->device != device || d->tables_capacity < img.bytes.size())) { destroy_device_state(d); d = nullptr; }
+  struct Guard {  // frees the state unless it is handed over
+    DeviceState* d;
+    ~Guard() { if (d) destroy_device_state(d); }
+  } guard{d};
+  const bool fresh = d == nullptr;
+  if (fresh) {
+    d = guard.d = new DeviceState();
+    d->device = device;
+    HIP_TRY(hipMalloc((void**)&d->tables, img.bytes.size()));
+    d->tables_capacity = img.bytes.size();
+    HIP_TRY(hipHostMalloc((void**)&d->host_status, sizeof(mscclx_status), hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc((void**)&d->abort_word_host, sizeof(unsigned long long), hipHostMallocDefault));
+    *d->abort_word_host = 1ull;
+    HIP_TRY(hipStreamCreateWithFlags(&d->side, hipStreamNonBlocking));
+    HIP_TRY(hipEventCreate(&d->ev0));
+    HIP_TRY(hipEventCreate(&d->ev1));
+#ifdef MSCCLX_PROFILE
+    HIP_TRY(hipMalloc((void**)&d->prof, sizeof(unsigned long long) * kProfWords * g.workgroups));
+    HIP_TRY(hipMemset(d->prof, 0, sizeof(unsigned long long) * kProfWords * g.workgroups));
+#endif
+  }
+  d->ready = false;
+  HIP_TRY(hipMemcpy(d->tables, img.bytes.data(), img.bytes.size(), hipMemcpyHostToDevice));
+  std::memset(d->host_status, 0, sizeof(mscclx_status));
+  if (fresh || d->dirty || d->workspace != (unsigned char*)workspace) {
+    HIP_TRY(hipMemset(workspace, 0, armed_bytes(g)));
+    HIP_TRY(hipDeviceSynchronize());
+    d->dirty = false;
+  }
+  d->workspace = (unsigned char*)workspace;
+  d->abort_requested = false;
+  img.bytes.clear();
+  img.bytes.shrink_to_fit();
+  d->image = std::move(img);
+  d->ready = true;
+  plan->dev = d;
+  guard.d = nullptr;
+  return MSCCLX_OK;
+}
+
+int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
+  if (!plan || !plan->dev || !plan->dev->ready) return fail(MSCCLX_ERR_STATE, "bind buffers before launching");
+  DeviceState* d = plan->dev;
+  const Geometry& g = plan->geo;
+  hipStream_t s = (hipStream_t)stream;
+  if (d->dirty) {  // the previous launch gave up half-way: its counters mean nothing
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipStreamSynchronize(d->side));
+    HIP_TRY(hipMemset(d->workspace, 0, armed_bytes(g)));  // LL: launches count from 0 again, old lines must go
+    HIP_TRY(hipDeviceSynchronize());
+    std::memset(d->host_status, 0, sizeof(mscclx_status));
+    d->dirty = false;
+    d->abort_requested = false;
+  }
+  const KernelParams kp = make_params(*plan, d->image, d->tables, d->workspace, d->host_status, d->prof);
+  hipLaunchKernelGGL(d->image.kernel, dim3((unsigned)g.workgroups), dim3(g.threads), 0, s, kp);
   HIP_TRY(hipGetLastError());
   return MSCCLX_OK;
 }
 
-int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
-  if (!plan || !plan->dev) return fail(MSCCLX_ERR_STATE, "nothing was launched");
+// How the launches so far ended, once the stream has drained.
+static int finish_wait(mscclx_plan* plan, mscclx_status* status) {
   DeviceState* d = plan->dev;
-  hipError_t e = hipStreamSynchronize((hipStream_t)stream);
-  if (e != hipSuccess) {
-    d->dirty = true;
-    return fail(MSCCLX_ERR_HIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(e));
-  }
   mscclx_status st = *d->host_status;
-  if (st.code != MSCCLX_OK && st.tb >= 0 && (size_t)st.tb < d->dev_op_begin.size()) {
-    // the kernel counts the steps of its own list, in which runs of nops are folded: report the IR's step
-    const size_t at = (size_t)d->dev_op_begin[(size_t)st.tb] + (size_t)std::max(st.step, 0);
-    if (at < d->dev_ir_step.size()) st.step = d->dev_ir_step[at];
-  }
-  if (status) *status = st;
 #ifdef MSCCLX_PROFILE
   if (d->prof && getenv("MSCCLX_PROFILE_DUMP")) {
     const size_t nwg = plan->geo.workgroups;
@@ -476,21 +560,62 @@ int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
     }
   }
 #endif
+  if (d->abort_requested) {
+    d->dirty = true;
+    if (status) { *status = st; status->code = MSCCLX_ERR_ABORTED; }
+    std::memset(d->host_status, 0, sizeof(mscclx_status));
+    return fail(MSCCLX_ERR_ABORTED, "the launch was aborted by mscclx_plan_abort; the rank buffers hold partial results");
+  }
   if (st.code != MSCCLX_OK) {
     d->dirty = true;
-    const Tb& tb = plan->tbs[st.tb];
-    static const char* what[] = {"its dependency", "an incoming message", "a free slot on its outgoing connection", "?"};
-    std::string msg = "watchdog: rank " + std::to_string(tb.rank) + " tb " + std::to_string(tb.local_id) + " step " + std::to_string(st.step) +
-                      " (slice " + std::to_string(st.slice) + ", pass " + std::to_string(st.pass) + ") waited more than " +
-                      std::to_string(plan->timeout_ms) + " ms for " + what[st.waiting_on & 3];
     std::memset(d->host_status, 0, sizeof(mscclx_status));
-    return fail(st.code, msg);
   }
+  return report_status(*plan, d->image, st, status);
+}
+
+int mscclx_plan_wait(mscclx_plan* plan, void* stream, mscclx_status* status) {
+  if (!plan || !plan->dev || !plan->dev->ready) return fail(MSCCLX_ERR_STATE, "nothing was launched");
+  DeviceState* d = plan->dev;
+  hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+  if (e != hipSuccess) {
+    d->dirty = true;
+    return fail(MSCCLX_ERR_HIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(e));
+  }
+  return finish_wait(plan, status);
+}
+
+int mscclx_plan_poll(mscclx_plan* plan, void* stream, mscclx_status* status) {
+  if (!plan || !plan->dev || !plan->dev->ready) return fail(MSCCLX_ERR_STATE, "nothing was launched");
+  DeviceState* d = plan->dev;
+  hipError_t e = hipStreamQuery((hipStream_t)stream);
+  if (e == hipErrorNotReady) {
+    if (status) *status = *d->host_status;  // a watchdog report shows here before the kernel has drained
+    return 1;
+  }
+  if (e != hipSuccess) {
+    d->dirty = true;
+    return fail(MSCCLX_ERR_HIP, std::string("hipStreamQuery: ") + hipGetErrorString(e));
+  }
+  return finish_wait(plan, status);
+}
+
+int mscclx_plan_abort(mscclx_plan* plan) {
+  if (!plan || !plan->dev || !plan->dev->ready) return fail(MSCCLX_ERR_STATE, "nothing was launched");
+  DeviceState* d = plan->dev;
+  const Geometry& g = plan->geo;
+  // Raise the abort word of both counter areas (which one the running launch uses is known to the
+  // device only) from a stream of the library's own: the launch stream is busy with the kernel.
+  d->abort_requested = true;
+  unsigned long long* base = (unsigned long long*)d->workspace;
+  for (int area = 0; area < 2; ++area)
+    HIP_TRY(hipMemcpyAsync(base + kControlWords + (uint64_t)area * g.sync_words, d->abort_word_host, sizeof(unsigned long long),
+                           hipMemcpyHostToDevice, d->side));
+  HIP_TRY(hipStreamSynchronize(d->side));
   return MSCCLX_OK;
 }
 
 int mscclx_plan_time(mscclx_plan* plan, void* stream, int32_t iters, float* ms_out) {
-  if (!plan || !plan->dev) return fail(MSCCLX_ERR_STATE, "bind buffers before timing");
+  if (!plan || !plan->dev || !plan->dev->ready) return fail(MSCCLX_ERR_STATE, "bind buffers before timing");
   if (iters <= 0 || !ms_out) return fail(MSCCLX_ERR_INVALID_ARG, "bad argument");
   DeviceState* d = plan->dev;
   hipStream_t s = (hipStream_t)stream;

@@ -727,6 +727,7 @@ __device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, 
   Hosted h;
   Context c;
   init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+  unsigned busy_rounds = 0;
   while (c.active) {
 #ifdef MSCCLX_PROFILE
     const u64 prof_t0 = wall_clock64();
@@ -767,6 +768,7 @@ __device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, 
 #ifdef MSCCLX_PROFILE
     const u64 prof_t1 = wall_clock64();
 #endif
+    if (__builtin_expect((++busy_rounds & 0x3fu) == 0, 0) && first_lane(writer ? load_counter(abort_word) : 0) != 0) return false;  // a host's abort request
     if (c.moves) do_move<R, VEC, LL>(c.m, p, epoch, c.rseq, c.sseq, h.tb, c.step, h.slice, c.pass);
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
@@ -841,6 +843,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
   int cursor = 0;
+  unsigned busy_rounds = 0;
 
   // A workgroup of one wave needs neither LDS nor a barrier to hand the chosen step to its threads:
   // they are the lanes of the polling wave, and take the operands from the chosen lane's registers.
@@ -881,6 +884,13 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
         if (movers) {
           const u64 from_cursor = movers & ~((cursor >= 64) ? ~0ull : ((1ull << cursor) - 1ull));
           choice = __ffsll((long long)(from_cursor ? from_cursor : movers)) - 1;
+          // a workgroup that always finds work never reaches the idle branch below: it looks at the
+          // abort word once in 64 moves, so that a host's abort request ends it too
+          if (__builtin_expect((++busy_rounds & 0x3fu) == 0, 0)) {
+            bool stop = false;
+            if (lane == 0) stop = load_counter(abort_word) != 0;
+            if (__any(stop)) choice = -3;
+          }
         } else if (!__any(c.active)) {
           choice = -1;  // every hosted context has run to its end
         } else if (__any(progressed)) {

@@ -15,9 +15,9 @@ CSRC_DIR = os.path.normpath(os.path.join(_HERE, "..", "..", "csrc"))
 LIB_PATH = os.path.join(CSRC_DIR, "libmscclx.so")
 
 OK = 0
-ERR_INVALID_ARG, ERR_BAD_IR, ERR_DEADLOCK, ERR_CAPACITY, ERR_HIP, ERR_TIMEOUT, ERR_STATE, ERR_UNSUPPORTED = range(-1, -9, -1)
+ERR_INVALID_ARG, ERR_BAD_IR, ERR_DEADLOCK, ERR_CAPACITY, ERR_HIP, ERR_TIMEOUT, ERR_STATE, ERR_UNSUPPORTED, ERR_ABORTED, ERR_ALIASED = range(-1, -11, -1)
 ERROR_NAMES = {0: "OK", -1: "INVALID_ARG", -2: "BAD_IR", -3: "DEADLOCK", -4: "CAPACITY", -5: "HIP", -6: "TIMEOUT",
-               -7: "STATE", -8: "UNSUPPORTED"}
+               -7: "STATE", -8: "UNSUPPORTED", -9: "ABORTED", -10: "ALIASED"}
 
 DTYPE_CODES = {"uint8": 0, "int8": 1, "int32": 2, "uint32": 3, "int64": 4, "uint64": 5,
                "float16": 6, "bfloat16": 7, "float32": 8, "float64": 9}
@@ -30,7 +30,7 @@ PROTOCOL_CODES = {"auto": 0, "simple": 1, "ll": 2, "Simple": 1, "LL": 2}
 EXPORTED_SYMBOLS = (
     "mscclx_version", "mscclx_last_error", "mscclx_plan_create", "mscclx_plan_destroy", "mscclx_plan_simulate",
     "mscclx_plan_min_fifo_depth", "mscclx_plan_algorithmic_units", "mscclx_plan_configure", "mscclx_plan_bind",
-    "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_time",
+    "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_poll", "mscclx_plan_abort", "mscclx_plan_time",
 )
 
 
@@ -103,9 +103,12 @@ def load_library(path=None):
     lib.mscclx_plan_bind.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, ctypes.c_size_t]
     lib.mscclx_plan_launch.argtypes = [vp, vp]
     lib.mscclx_plan_wait.argtypes = [vp, vp, ctypes.POINTER(Status)]
+    lib.mscclx_plan_poll.argtypes = [vp, vp, ctypes.POINTER(Status)]
+    lib.mscclx_plan_abort.argtypes = [vp]
     lib.mscclx_plan_time.argtypes = [vp, vp, i32, ctypes.POINTER(ctypes.c_float)]
     for name in ("mscclx_plan_create", "mscclx_plan_destroy", "mscclx_plan_simulate", "mscclx_plan_min_fifo_depth",
-                 "mscclx_plan_configure", "mscclx_plan_bind", "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_time"):
+                 "mscclx_plan_configure", "mscclx_plan_bind", "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_poll",
+                 "mscclx_plan_abort", "mscclx_plan_time"):
         getattr(lib, name).restype = ctypes.c_int
     if path is None:
         _lib = lib
@@ -175,6 +178,15 @@ class Plan:
         st = Status()
         _check(self.lib, self.lib.mscclx_plan_wait(self.handle, ctypes.c_void_p(stream or None), ctypes.byref(st)))
         return st
+
+    def poll(self, stream=0):
+        """(running, status): running is True while the launch stream still has work."""
+        st = Status()
+        rc = _check(self.lib, self.lib.mscclx_plan_poll(self.handle, ctypes.c_void_p(stream or None), ctypes.byref(st)))
+        return rc == 1, st
+
+    def abort(self):
+        _check(self.lib, self.lib.mscclx_plan_abort(self.handle))
 
     def time(self, iters, stream=0):
         ms = (ctypes.c_float * iters)()

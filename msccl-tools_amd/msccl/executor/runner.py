@@ -8,9 +8,11 @@ output chunks [r*cf, (r+1)*cf)).
 """
 from __future__ import annotations
 
+import time
+
 import torch
 
-from .binding import DTYPE_SIZES, MscclxError, Plan
+from .binding import DTYPE_SIZES, ERR_ALIASED, MscclxError, Plan
 from .ir_tables import AlgoTables, parse_algo_xml
 
 _TORCH_NAMES = {torch.uint8: "uint8", torch.int8: "int8", torch.int32: "int32", torch.int64: "int64",
@@ -43,6 +45,7 @@ class Executor:
         self._scratch = None
         self._workspace = None
         self._bound = None
+        self.host_seconds = {}   # host time of the last configure / bind call into the library
 
     # -- geometry ---------------------------------------------------------------------------------
     def setup(self, chunk_bytes, dtype, redop="sum", **knobs):
@@ -59,7 +62,9 @@ class Executor:
         self.chunk_bytes = int(chunk_bytes)
         self._setup_args = (chunk_bytes, dtype, redop, dict(knobs))
         with torch.cuda.device(self.device):
+            t0 = time.perf_counter()
             self.info = self.plan.configure(self.chunk_bytes, self.dtype, redop, **knobs)
+            self.host_seconds["configure"] = time.perf_counter() - t0
             t = self.tables
             self._scratch = [torch.empty(int(t.rank_chunks[r, 2]) * self.chunk_bytes, dtype=torch.uint8, device=self.device)
                              if t.rank_chunks[r, 2] else None for r in range(t.ngpus)]
@@ -99,9 +104,11 @@ class Executor:
         scr = [0 if s is None else s.data_ptr() for s in self._scratch]
         try:
             with torch.cuda.device(self.device):
+                t0 = time.perf_counter()
                 self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
+                self.host_seconds["bind"] = time.perf_counter() - t0
         except MscclxError as e:
-            if "overlap" not in e.message:
+            if e.code != ERR_ALIASED:
                 raise
             # the caller aliases buffers the IR names separately (an in-place call): payloads can no
             # longer be read in place, so every message goes through a FIFO slot
@@ -125,6 +132,16 @@ class Executor:
     def wait(self):
         with torch.cuda.device(self.device):
             return self.plan.wait(self._stream())
+
+    def poll(self):
+        """True while the launch is still running (non-blocking); raises like wait() once it has failed."""
+        with torch.cuda.device(self.device):
+            return self.plan.poll(self._stream())[0]
+
+    def abort(self):
+        """Ask the running launch to give up; wait() then raises MscclxError(ABORTED)."""
+        with torch.cuda.device(self.device):
+            self.plan.abort()
 
     def run(self, inputs, outputs):
         self.bind(inputs, outputs)

@@ -20,7 +20,7 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
     assert declared == set(EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(mscclx_lib, name), name
-    assert mscclx_lib.mscclx_version() == 2
+    assert mscclx_lib.mscclx_version() == 3
 
 
 def test_struct_layouts_match_header():

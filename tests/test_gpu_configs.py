@@ -178,23 +178,74 @@ def test_chunks_beyond_4_gib():
 
 
 def test_aliased_buffers_fall_back_to_staging():
-    """An in-place call aliases the 'i' and 'o' buffers the IR names separately; reading payloads in
-    place is then unsound, bind refuses it and the runner re-plans with staging."""
-    from msccl.executor import Executor
-    xml = golden_util.load("alltoall_allpairs_4r")
-    E = 1024
+    """An in-place call on an out-of-place algorithm aliases buffers the IR names separately: here every
+    rank's 'i' is chunk r of its own 'o' (NCCL's in-place all-gather convention) on an out-of-place
+    ring all-gather whose copy threadblock moves i[0] to o[r].  Reading payloads in place assumes
+    distinct memory, so bind refuses with ALIASED and the runner re-plans with every message staged;
+    the aliased run must still deliver the concatenation, and on a program where aliasing makes a
+    receive overwrite what a send of the same rank still has to read, nothing but the refusal is promised."""
+    import ir_samples
+    from msccl.executor import Executor, MscclxError
+    from msccl.executor.binding import ERR_ALIASED
+    n, E = 5, 3000
+    xml = ir_samples.ncclize_style_allgather_xml(n)
+    rng = np.random.default_rng(77)
+    x = [rng.integers(-2 ** 31, 2 ** 31, E, dtype=np.int64).astype(np.int32) for _ in range(n)]
+    want = np.concatenate(x)
     ex = Executor(xml)
     ex.setup(E * 4, "int32", protocol="simple")
     assert ex.info.zero_copy_messages > 0
-    n = 4
-    bufs = [torch.arange(n * E, dtype=torch.int32, device="cuda:0") + 100000 * r for r in range(n)]
-    shadow = [b.clone() for b in bufs]
     outs = [torch.zeros(n * E, dtype=torch.int32, device="cuda:0") for _ in range(n)]
-    ex.run(shadow, outs)                       # out of place: the reference result
+    ins = [outs[r][r * E:(r + 1) * E] for r in range(n)]        # same memory as o[r]
+    for r in range(n):
+        ins[r].copy_(torch.from_numpy(x[r]))
+    with pytest.raises(MscclxError) as e:                        # the C ABI itself refuses ...
+        ex.plan.bind([t.data_ptr() for t in ins], [t.data_ptr() for t in outs], [0] * n, ex._workspace.data_ptr(), ex._workspace.numel())
+    assert e.value.code == ERR_ALIASED
+    print("case: aliased all-gather, staged", flush=True)
+    ex.run(ins, outs)                                            # ... and the runner falls back to staging
+    assert ex.info.zero_copy_messages == 0 and ex.info.staged_messages > 0
+    torch.cuda.synchronize()
+    for r in range(n):
+        assert np.array_equal(outs[r].cpu().numpy(), want), r
+    # the same data out of place, payloads read in place: the same result
     ex2 = Executor(xml)
     ex2.setup(E * 4, "int32", protocol="simple")
-    ex2.bind(bufs, [b[: n * E] for b in bufs])  # same memory for 'i' and 'o'
-    assert ex2.info.zero_copy_messages == 0 and ex2.info.staged_messages > 0
+    outs2 = [torch.zeros(n * E, dtype=torch.int32, device="cuda:0") for _ in range(n)]
+    ex2.run([torch.from_numpy(v).cuda() for v in x], outs2)
+    assert ex2.info.zero_copy_messages > 0
+    for r in range(n):
+        assert torch.equal(outs2[r], outs[r]), r
+
+
+def test_rebind_new_buffers_same_plan():
+    """Binding a second and third set of buffers to a configured plan re-uses the device-side state
+    (one upload of the tables); every set must get its own, correct result, and going back to the
+    first set must work too."""
+    import ir_samples
+    from msccl.executor import Executor, collective_buffers
+    xml = ir_samples.allpairs_allreduce_xml(4)
+    algo = oi.parse_xml(xml)
+    E = 3000
+    ex = Executor(xml)
+    ex.setup(E * 4, "float32")
+    sets = []
+    for k in range(3):
+        rng = np.random.default_rng(500 + k)
+        x = [(rng.random(4 * E, dtype=np.float32) * 2 - 1) for _ in range(4)]
+        ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+        want = oc.place_inputs(algo, x, E, "float32")
+        oi.Interpreter(algo).run(want, E, "float32")
+        sets.append((x, ins, outs, res, want))
+    print("case: rebind", flush=True)
+    for k in (0, 1, 2, 0):
+        x, ins, outs, res, want = sets[k]
+        for r in range(4):
+            ins[r].copy_(torch.from_numpy(x[r]))
+        ex.run(ins, outs)
+        torch.cuda.synchronize()
+        for r in range(4):
+            assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (k, r)
 
 
 def test_init_to_run_flow(capsys):

@@ -317,6 +317,76 @@ def test_watchdog_names_the_ir_step_of_folded_nops():
     assert torch.equal(out[:nbytes], x) and torch.equal(out[nbytes:], x)
 
 
+def test_poll_does_not_block():
+    """mscclx_plan_poll: 'running' while the launch is under way, then the launch's result."""
+    import time
+    from msccl.executor import Executor, collective_buffers
+    xml = ir_samples.slow_producer_xml(24)
+    nbytes = 64 << 20
+    ex = Executor(xml)
+    ex.setup(nbytes, "uint8", slices=1, piece_bytes=nbytes)   # one workgroup makes the 24 copies: tens of milliseconds
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    torch.cuda.synchronize()
+    print("case: poll", flush=True)
+    ex.launch()
+    t0 = time.perf_counter()
+    first = ex.poll()
+    dt_first = time.perf_counter() - t0
+    polls = 1
+    while ex.poll():
+        polls += 1
+        time.sleep(0.001)
+        assert time.perf_counter() - t0 < 30
+    assert first and dt_first < 0.005, (first, dt_first)         # came back at once, with the launch still running
+    assert not ex.poll()                                         # finished: stays finished, no error
+    assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
+    print(f"polled {polls} times in {(time.perf_counter() - t0) * 1e3:.1f} ms", flush=True)
+
+
+def test_abort_from_the_host():
+    """mscclx_plan_abort ends a launch that still has a long way to go: every workgroup leaves by
+    itself, wait() reports ABORTED well before the launch could have finished, and the same binding
+    then runs to completion with the right result (the counters are re-armed)."""
+    import time
+    from msccl.executor import Executor, MscclxError, collective_buffers
+    from msccl.executor.binding import ERR_ABORTED
+    ncopies = 200
+    xml = ir_samples.slow_producer_xml(ncopies)
+    nbytes = 64 << 20
+    ex = Executor(xml)
+    ex.setup(nbytes, "uint8", slices=1, piece_bytes=nbytes)
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    torch.cuda.synchronize()
+    print("case: full run for reference", flush=True)
+    t0 = time.perf_counter()
+    ex.launch()
+    ex.wait()
+    full = time.perf_counter() - t0
+    assert torch.equal(outs[1].cpu(), x[0])
+    outs[1].zero_()
+    torch.cuda.synchronize()
+    print(f"case: abort (a full run takes {full * 1e3:.1f} ms)", flush=True)
+    t0 = time.perf_counter()
+    ex.launch()
+    assert ex.poll()
+    ex.abort()
+    with pytest.raises(MscclxError) as e:
+        ex.wait()
+    aborted = time.perf_counter() - t0
+    assert e.value.code == ERR_ABORTED
+    # the receiver gave up at once; the producer finishes the copy it is in (1/200 of the run) and leaves
+    assert aborted < 0.5 * full, (aborted, full)
+    assert not torch.equal(outs[1].cpu(), x[0])                  # the message never arrived
+    print(f"aborted after {aborted * 1e3:.1f} ms; relaunching", flush=True)
+    ex.launch()
+    ex.wait()
+    assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
+
+
 @pytest.mark.parametrize("threads", [0, 64])
 def test_watchdog_in_ll_mode(threads):
     """Flag-in-data lines, one context per workgroup (threads=64: a workgroup of one wave, which runs

