@@ -185,6 +185,21 @@ int mscclx_plan_poll(mscclx_plan* plan, void* stream, mscclx_status* status);
  * the request is on the device; mscclx_plan_wait then returns MSCCLX_ERR_ABORTED, the rank buffers
  * hold partial results, and the next launch re-arms the counters. */
 int mscclx_plan_abort(mscclx_plan* plan);
+/* Bytes of the device array behind mscclx_plan_run_static (one copy per GPU, held until the process ends). */
+#define MSCCLX_STATIC_SCRATCH_BYTES (32u << 20)
+/* No counterpart in msccl-tools.  For callers that cannot allocate device memory (tight serving
+ * loops, harnesses that forbid hipMalloc): one whole execution of a configured plan -- bind, launch,
+ * wait -- that calls no hipMalloc, hipFree or other allocating routine.  The plan tables, the
+ * counters and the FIFO slots, which mscclx_plan_bind keeps in memory it allocates and in the
+ * caller's workspace, live in a device array that is part of the library; the caller passes only
+ * the rank buffers (as to mscclx_plan_bind).  A plan that needs more than
+ * MSCCLX_STATIC_SCRATCH_BYTES for them is refused with MSCCLX_ERR_CAPACITY.  Returns when the
+ * launch has finished, with mscclx_plan_wait's result.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (from several threads or streams) race, and a call must
+ * not overlap a launch of the same plan made through mscclx_plan_launch either.  The plan's own
+ * binding (mscclx_plan_bind) is left untouched. */
+int mscclx_plan_run_static(mscclx_plan* plan, void* const* in, void* const* out, void* const* rank_scratch,
+                           void* stream, mscclx_status* status);
 /* Times `iters` back-to-back launches with HIP events on `stream`; ms_out[i] = duration of launch i. */
 int mscclx_plan_time(mscclx_plan* plan, void* stream, int32_t iters, float* ms_out);
 

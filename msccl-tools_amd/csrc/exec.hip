@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <utility>
 #include <string>
 #include <vector>
@@ -24,6 +25,7 @@ namespace mscclx {
 // host: kernel table, configure, bind, launch
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
 kernel_fn pick_kernel_group_0(int dtype, int op, bool vec, bool ll, bool fold);
 kernel_fn pick_kernel_group_1(int dtype, int op, bool vec, bool ll, bool fold);
@@ -363,6 +365,43 @@ static int report_status(const mscclx_plan& plan, const DeviceImage& img, mscclx
                            std::to_string(plan.timeout_ms) + " ms for " + what[st.waiting_on & 3]);
 }
 
+// ------------------------------------------------------------------------------------------------
+// mscclx_plan_run_static: one execution whose tables, counters and FIFO slots live in a device array
+// of the library's own, so that the call allocates nothing.
+// ------------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)MSCCLX_STATIC_SCRATCH_BYTES;
+constexpr size_t kStaticStatusBytes = 256;  // the launch's mscclx_status sits in front of the tables
+static_assert(sizeof(mscclx_status) <= kStaticStatusBytes, "status block");
+// In host code this name only stands for the symbol; the array's device address (one per GPU, each
+// GPU holds its own copy) comes from hipGetSymbolAddress and is kept in g_static_ptr.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static unsigned char* g_static_ptr[kMaxDevices] = {};
+static std::mutex g_static_mutex;
+
+// The calling thread's current device and the address of that device's copy of `scratch`.
+static int static_scratch(unsigned char** ptr_out) {
+  int device = -1;
+  HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(MSCCLX_ERR_UNSUPPORTED, "device ordinal beyond " + std::to_string(kMaxDevices - 1));
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[device]) {
+    unsigned char* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr || (uintptr_t)ptr % 256) return fail(MSCCLX_ERR_HIP, "hipGetSymbolAddress returned an unusable address for the static scratch array");
+    g_static_ptr[device] = ptr;
+  }
+  *ptr_out = g_static_ptr[device];
+  return MSCCLX_OK;
+}
+
+// (not hipMemsetAsync: a memset node recorded into a HIP graph has replayed wrongly on this platform)
+__global__ void __launch_bounds__(256) zero_fill_kernel(u32x4* dst, size_t n16) {
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = zero;
+}
+
 }  // namespace mscclx
 
 using namespace mscclx;
@@ -612,6 +651,42 @@ int mscclx_plan_abort(mscclx_plan* plan) {
                            hipMemcpyHostToDevice, d->side));
   HIP_TRY(hipStreamSynchronize(d->side));
   return MSCCLX_OK;
+}
+
+int mscclx_plan_run_static(mscclx_plan* plan, void* const* in, void* const* out, void* const* rank_scratch, void* stream, mscclx_status* status) {
+  if (!plan) return fail(MSCCLX_ERR_INVALID_ARG, "null plan");
+  if (!plan->configured) return fail(MSCCLX_ERR_STATE, "configure the plan before running it");
+  const Geometry& g = plan->geo;
+  std::vector<void*> bufs;
+  int rc = collect_buffers(*plan, in, out, rank_scratch, &bufs);
+  if (rc) return rc;
+  DeviceImage img;
+  rc = build_image(*plan, bufs, &img);
+  if (rc) return rc;
+  // layout inside the array: status | tables | workspace (control block, counters, FIFO slots)
+  const size_t tables_off = kStaticStatusBytes;
+  const size_t workspace_off = (tables_off + img.bytes.size() + 255) / 256 * 256;
+  const size_t need = workspace_off + g.workspace_bytes;
+  if (need > kStaticScratchBytes)
+    return fail(MSCCLX_ERR_CAPACITY, "this plan needs " + std::to_string(need) + " bytes of tables, counters and FIFO slots; mscclx_plan_run_static has " +
+                                         std::to_string(kStaticScratchBytes) + " (MSCCLX_STATIC_SCRATCH_BYTES): use mscclx_plan_bind with a workspace of the caller's");
+  unsigned char* base = nullptr;
+  rc = static_scratch(&base);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  // whatever the previous call left: the status, the counters (LL: the slots too) must read zero
+  const size_t clear_to = workspace_off + armed_bytes(g);
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(256), dim3(256), 0, s, (u32x4*)base, kStaticStatusBytes / 16);
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, (u32x4*)(base + workspace_off), (clear_to - workspace_off + 15) / 16);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpyAsync(base + tables_off, img.bytes.data(), img.bytes.size(), hipMemcpyHostToDevice, s));
+  const KernelParams kp = make_params(*plan, img, base + tables_off, base + workspace_off, (mscclx_status*)base, nullptr);
+  hipLaunchKernelGGL(img.kernel, dim3((unsigned)g.workgroups), dim3(g.threads), 0, s, kp);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipStreamSynchronize(s));
+  mscclx_status st;
+  HIP_TRY(hipMemcpy(&st, base, sizeof st, hipMemcpyDeviceToHost));
+  return report_status(*plan, img, st, status);
 }
 
 int mscclx_plan_time(mscclx_plan* plan, void* stream, int32_t iters, float* ms_out) {

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "mscclx_version", "mscclx_last_error", "mscclx_plan_create", "mscclx_plan_destroy", "mscclx_plan_simulate",
     "mscclx_plan_min_fifo_depth", "mscclx_plan_algorithmic_units", "mscclx_plan_configure", "mscclx_plan_bind",
     "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_poll", "mscclx_plan_abort", "mscclx_plan_time",
+    "mscclx_plan_run_static",
 )
 
 
@@ -106,6 +107,8 @@ def load_library(path=None):
     lib.mscclx_plan_poll.argtypes = [vp, vp, ctypes.POINTER(Status)]
     lib.mscclx_plan_abort.argtypes = [vp]
     lib.mscclx_plan_time.argtypes = [vp, vp, i32, ctypes.POINTER(ctypes.c_float)]
+    lib.mscclx_plan_run_static.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, ctypes.POINTER(Status)]
+    lib.mscclx_plan_run_static.restype = ctypes.c_int
     for name in ("mscclx_plan_create", "mscclx_plan_destroy", "mscclx_plan_simulate", "mscclx_plan_min_fifo_depth",
                  "mscclx_plan_configure", "mscclx_plan_bind", "mscclx_plan_launch", "mscclx_plan_wait", "mscclx_plan_poll",
                  "mscclx_plan_abort", "mscclx_plan_time"):
@@ -170,6 +173,15 @@ class Plan:
         arr = lambda ptrs: (ctypes.c_void_p * n)(*[ctypes.c_void_p(p or None) for p in ptrs])
         _check(self.lib, self.lib.mscclx_plan_bind(self.handle, arr(in_ptrs), arr(out_ptrs), arr(scratch_ptrs),
                                                   ctypes.c_void_p(workspace_ptr), workspace_bytes))
+
+    def run_static(self, in_ptrs, out_ptrs, scratch_ptrs, stream=0):
+        """One whole execution out of the library's static device array (no allocation)."""
+        n = self.tables.ngpus
+        arr = lambda ptrs: (ctypes.c_void_p * n)(*[ctypes.c_void_p(p or None) for p in ptrs])
+        st = Status()
+        _check(self.lib, self.lib.mscclx_plan_run_static(self.handle, arr(in_ptrs), arr(out_ptrs), arr(scratch_ptrs),
+                                                        ctypes.c_void_p(stream or None), ctypes.byref(st)))
+        return st
 
     def launch(self, stream=0):
         _check(self.lib, self.lib.mscclx_plan_launch(self.handle, ctypes.c_void_p(stream or None)))

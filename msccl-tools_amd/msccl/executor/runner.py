@@ -149,6 +149,18 @@ class Executor:
         self.wait()
         return outputs
 
+    def run_static(self, inputs, outputs):
+        """One whole execution that allocates nothing on the device: tables, counters and FIFO slots
+        sit in the library's own static device array (mscclx_plan_run_static).  Refused with CAPACITY
+        when the plan needs more than that array holds.  Leaves the binding of run()/launch() alone."""
+        if self.info is None:
+            raise RuntimeError("call setup() first")
+        ins = self._check_buffers(inputs, 0, "input")
+        outs = self._check_buffers(outputs, 1, "output")
+        scr = [0 if s is None else s.data_ptr() for s in self._scratch]
+        with torch.cuda.device(self.device):
+            return self.plan.run_static(ins, outs, scr, self._stream())
+
     def time(self, iters):
         """Per-launch GPU time in ms (HIP events around each launch on the current stream)."""
         with torch.cuda.device(self.device):

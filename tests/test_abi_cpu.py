@@ -233,3 +233,15 @@ def test_geometry_between_the_benchmark_sizes(mscclx_lib):
         w = WORKLOADS[key].scaled(nbytes)
         i = Plan(parse_algo_xml(WORKLOADS[key].build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.threads, i.slices, i.piece_bytes) == expect, (key, nbytes, (i.threads, i.slices, i.piece_bytes))
+
+
+def test_run_static_refuses_an_oversized_plan_before_touching_the_gpu(mscclx_lib):
+    """The size check of mscclx_plan_run_static is host arithmetic: a plan whose tables, counters and
+    FIFO slots exceed MSCCLX_STATIC_SCRATCH_BYTES is refused with CAPACITY before any HIP call."""
+    t = parse_algo_xml(ir_samples.ring_allreduce_xml(8, 2))
+    p = Plan(t)
+    p.configure(4 << 20, "float32", staging=1, max_workgroups=512)
+    fake = [0x10000000 + r * (1 << 28) for r in range(t.ngpus)]      # never dereferenced
+    with pytest.raises(MscclxError) as e:
+        p.run_static(fake, [0] * t.ngpus, [0] * t.ngpus)
+    assert e.value.code == binding.ERR_CAPACITY and "MSCCLX_STATIC_SCRATCH_BYTES" in e.value.message
