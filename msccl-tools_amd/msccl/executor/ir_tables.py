@@ -64,6 +64,24 @@ def _int(elem, name, default=None):
         raise IRError(f"<{elem.tag} {name}={v!r}> is not an integer") from None
 
 
+_LOCAL_SRC = {OP_CODES[k] for k in ("s", "cpy", "re")}
+_LOCAL_DST = {OP_CODES[k] for k in ("r", "rcs", "rrs", "rrc", "rrcs", "cpy", "re")}
+
+
+def _scratch_behind_output(row, o_chunks):
+    """ncclize(use_scratch=False) writes a rank's scratch references as output offsets past the
+    output's own chunks ("scratch at the end of output", msccl/ncclize.py:690-697) while still
+    declaring o_chunks and s_chunks separately.  Such a local reference is taken back to the
+    scratch buffer, so the caller's output buffer keeps the size the collective gives it.  (On 's'
+    and receive steps the other side's location is informational and is left alone.)"""
+    ty, sb, so, db, do, cnt, depid, deps, hasdep = row
+    if ty in _LOCAL_SRC and sb == BUF_CODES["o"] and so >= o_chunks:
+        sb, so = BUF_CODES["s"], so - o_chunks
+    if ty in _LOCAL_DST and db == BUF_CODES["o"] and do >= o_chunks:
+        db, do = BUF_CODES["s"], do - o_chunks
+    return (ty, sb, so, db, do, cnt, depid, deps, hasdep)
+
+
 def parse_algo_xml(text):
     """Parse one <algo> document into AlgoTables."""
     try:
@@ -111,6 +129,9 @@ def parse_algo_xml(text):
                 op_rows.append((OP_CODES[ty], BUF_CODES[sb], _int(st, "srcoff", -1), BUF_CODES[db], _int(st, "dstoff", -1),
                                 _int(st, "cnt", 1 if ty != "nop" else 0), _int(st, "depid", -1), _int(st, "deps", -1),
                                 _int(st, "hasdep", 0)))
+            if rank_chunks[r, 2] > 0:
+                for k in range(begin, len(op_rows)):
+                    op_rows[k] = _scratch_behind_output(op_rows[k], int(rank_chunks[r, 1]))
             tb_rows.append((r, _int(t, "send"), _int(t, "recv"), _int(t, "chan"), begin, len(op_rows)))
     return AlgoTables(
         name=root.get("name", ""), proto=root.get("proto", "Simple"), coll=root.get("coll", "custom"),

@@ -65,6 +65,10 @@ WORKLOADS = {
                    128 << 20, 64, lambda: _catalog().two_level_allreduce(8, 4, instances=2)),
     "c5": Workload("c5", 5, "small-message ring AllReduce, 64 ranks, one chunk per ring slot; fp16 256 KiB/rank", "allreduce", 64,
                    "float16", 256 << 10, 64, lambda: _catalog().ring_allreduce(64, channels=1, instances=1)),
+    # the other reading of "chunk factor 1" for the 64-rank configuration: the buffer is ONE chunk
+    "c5_chain": Workload("c5_chain", 5, "small-message chain AllReduce, 64 ranks, one 256 KiB chunk on a 63-hop reduce chain and a 63-hop "
+                         "broadcast chain; fp16 256 KiB/rank", "allreduce", 64, "float16", 256 << 10, 1,
+                         lambda: _catalog().chain_allreduce(64)),
 }
 
 

@@ -28,6 +28,18 @@ def ring_allreduce(num_ranks, channels=1, instances=1, protocol="Simple"):
     return _finish(prog)
 
 
+def chain_allreduce(num_ranks, instances=1, protocol="Simple"):
+    """AllReduce(n, 1, inplace): the whole buffer is ONE chunk, reduced along a chain of n-1 hops and
+    handed on along n-1 more (msccl/programs/allreduce_chain.py) -- what "chunk factor 1" means when
+    msccl-tools' registry passes it as the collective's chunk count (autosynth/registry.py:65-66,75-76)."""
+    from msccl.programs.allreduce_chain import allreduce_chain
+    prog = MSCCLProgram("allreduce_chain", fully_connected(num_ranks), AllReduce(num_ranks, 1, True), instances, protocol=protocol,
+                        threadblock_policy=ThreadblockPolicy.manual)
+    with prog:
+        allreduce_chain(num_ranks)
+    return _finish(prog)
+
+
 def ring_allgather(num_ranks, channels=1, instances=1, protocol="Simple"):
     """examples/mscclang/allgather_ring.py:13-26: AllGather(n, 1, inplace), manual threadblocks."""
     from msccl.programs.allgather_ring import allgather_ring

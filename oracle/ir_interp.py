@@ -22,6 +22,10 @@ msccl-tools checkout):
   `deps`:                                                       ir.py:235-262,380-391.
 * Connections are FIFOs per (sender rank, receiver rank, channel); sends and matching receives
   occur in the same order:                                      msccl/language/passes.py:31-55.
+* ncclize documents: on 's' the destination and on 'r'/'rrc' the source name the OTHER rank's
+  location (msccl/ncclize.py:532-535) and take no part in execution; a receive into a slot that
+  already holds data is an 'rrc' (ncclize.py:390-400); copies sit in a threadblock of their own,
+  which may be empty (ncclize.py:621-626).
 
 Parity pinning.  The reference holds no execution vectors for this path (its tests are
 symbolic), so this interpreter is pinned by what the mathematics fixes: closed forms of the
@@ -76,7 +80,11 @@ def bf16_bits_to_f32(b):
 
 
 def _reduce(a, b, dtype, redop):
-    """Element-wise a (+) b in the buffer dtype."""
+    """Element-wise a (+) b in the buffer dtype.  max and min of floating-point data are C's
+    fmax / fmin: a NaN operand counts as missing and the other operand is the result (NaN only if
+    both are) -- the semantics of the fmaxf / fminf the collective runtimes of the NCCL family
+    reduce with, and of the device code here; sum and prod propagate NaN as IEEE addition and
+    multiplication do."""
     if dtype == "bfloat16":
         fa, fb = bf16_bits_to_f32(a), bf16_bits_to_f32(b)
         with np.errstate(all="ignore"):
@@ -85,9 +93,9 @@ def _reduce(a, b, dtype, redop):
             elif redop == "prod":
                 r = fa * fb
             elif redop == "max":
-                r = np.maximum(fa, fb)
+                r = np.fmax(fa, fb)
             elif redop == "min":
-                r = np.minimum(fa, fb)
+                r = np.fmin(fa, fb)
             else:
                 raise ValueError(redop)
         return f32_to_bf16_bits(r)
@@ -97,9 +105,9 @@ def _reduce(a, b, dtype, redop):
         if redop == "prod":
             return a * b
         if redop == "max":
-            return np.maximum(a, b)
+            return np.fmax(a, b)
         if redop == "min":
-            return np.minimum(a, b)
+            return np.fmin(a, b)
     raise ValueError(redop)
 
 
@@ -146,8 +154,15 @@ def parse_xml(text):
         for t in g.findall("tb"):
             tb = Tb(int(t.get("id")), int(t.get("send")), int(t.get("recv")), int(t.get("chan")))
             for st in t.findall("step"):
-                tb.steps.append(Step(int(st.get("s")), st.get("type"), st.get("srcbuf"), int(st.get("srcoff")),
-                                     st.get("dstbuf"), int(st.get("dstoff")), int(st.get("cnt")),
+                ty = st.get("type")
+                sb, so, db, do = st.get("srcbuf"), int(st.get("srcoff")), st.get("dstbuf"), int(st.get("dstoff"))
+                # ncclize(use_scratch=False) addresses a rank's scratch as output chunks past o_chunks
+                # (msccl/ncclize.py:690-697, "scratch at the end of output"): local references only
+                if gpu.s_chunks and ty in ("s", "cpy", "re") and sb == "o" and so >= gpu.o_chunks:
+                    sb, so = "s", so - gpu.o_chunks
+                if gpu.s_chunks and ty in RECV_TYPES + ("cpy", "re") and db == "o" and do >= gpu.o_chunks:
+                    db, do = "s", do - gpu.o_chunks
+                tb.steps.append(Step(int(st.get("s")), ty, sb, so, db, do, int(st.get("cnt")),
                                      int(st.get("depid")), int(st.get("deps")), int(st.get("hasdep"))))
             gpu.tbs.append(tb)
         a.gpus.append(gpu)

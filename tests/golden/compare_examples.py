@@ -32,7 +32,8 @@ EXAMPLES = [
     ("alltoall_a100_three_step.py", [3, 4, 1]), ("alltoall_a100_two_step.py", [2, 4]), ("alltoall_allpairs.py", [4, 2]),
     ("alltonext_backward.py", [2, 1]), ("alltonext_forward.py", [2, 1]), ("hierarchical_allreduce.py", [4, 2, 1]),
     ("hierarchical_allreduce.py", [4, 2, 2, "--schedule", "manual"]), ("pipeline_a100_allpairs.py", [8, 1]),
-    ("pipeline_a100_ring.py", [8, 2, 1]), ("reducegather.py", [8, 2]), ("allreduce_dgx1.py", [1, 1]), ("allreduce_ndv2.py", [1]),
+    ("pipeline_a100_ring.py", [8, 2, 1]), ("reducegather.py", [8, 2]), ("simple/allgather_ring.py", []), ("simple/allreduce_ring.py", [8, 2]),
+    ("simple/custom_collective.py", []), ("allreduce_dgx1.py", [1, 1]), ("allreduce_ndv2.py", [1]),
 ]
 
 

@@ -42,8 +42,9 @@ def normalise(xml):
     return xml.replace(" />", "/>").strip() + "\n"
 
 
-def from_example(script, argv):
-    """Run an examples/mscclang script as __main__ and capture the XML it prints."""
+def from_example(script, argv, which=0):
+    """Run an examples/mscclang script as __main__ and capture the XML it prints (the `which`-th
+    document, for scripts that print several)."""
     old = sys.argv
     sys.argv = [script] + [str(a) for a in argv]
     buf = io.StringIO()
@@ -53,7 +54,8 @@ def from_example(script, argv):
     finally:
         sys.argv = old
     text = buf.getvalue()
-    return normalise(text[text.index("<algo"):text.index("</algo>") + len("</algo>")])
+    docs = [d[:d.index("</algo>") + len("</algo>")] for d in text.split("<algo")[1:]]
+    return normalise("<algo" + docs[which])
 
 
 def from_program(build):
@@ -75,6 +77,17 @@ def main():
         with MSCCLProgram("allreduce_ring", fully_connected(n), AllReduce(n, n, True), instances,
                           threadblock_policy=ThreadblockPolicy.manual):
             allreduce_ring(n, channels)
+            assert Check()
+            XML()
+
+    def chain(n):
+        # this repository's msccl/programs/allreduce_chain.py, through msccl-tools' compiler
+        from msccl.language import chunk, Buffer
+        with MSCCLProgram("allreduce_chain", fully_connected(n), AllReduce(n, 1, True), 1, threadblock_policy=ThreadblockPolicy.manual):
+            for hop in range(n - 1):
+                chunk(hop + 1, Buffer.input, 0).reduce(chunk(hop, Buffer.input, 0), ch=0, recvtb=0, sendtb=0)
+            for hop in range(-1, n - 2):
+                chunk(hop % n, Buffer.input, 0).copy(hop + 1, Buffer.input, 0, ch=0, recvtb=0, sendtb=0)
             assert Check()
             XML()
 
@@ -110,6 +123,13 @@ def main():
         "c4_hierarchical_allreduce_8x4_2inst_auto": lambda: from_example("hierarchical_allreduce.py", [8, 4, 2]),
         "c4_hierarchical_allreduce_4x2_1inst_manual": lambda: from_example("hierarchical_allreduce.py", [4, 2, 1, "--schedule", "manual"]),
         "c5_allreduce_ring_64r_1ch_1inst": lambda: from_program(lambda: ring(64, 1, 1)),
+        "c5_allreduce_chain_64r": lambda: from_program(lambda: chain(64)),
+        "simple_allgather_ring_4r_auto": lambda: from_example("simple/allgather_ring.py", []),
+        "simple_allreduce_ring_8r_2inst_auto": lambda: from_example("simple/allreduce_ring.py", [8, 2]),
+        "simple_custom_collective_3r_fanout": lambda: from_example("simple/custom_collective.py", [], which=0),
+        "simple_custom_collective_3r_relay": lambda: from_example("simple/custom_collective.py", [], which=1),
+        "allreduce_a100_allpairs_v2_8r": lambda: from_example("allreduce_a100_allpairs_v2.py", [8, 1]),
+        "alltoall_a100_three_step_3x4_example": lambda: from_example("alltoall_a100_three_step.py", [3, 4, 1]),
         "allreduce_ring_8r_4ch_8inst": lambda: from_program(lambda: ring(8, 4, 8)),
         "allreduce_allpairs_8r_2inst": lambda: from_program(lambda: allpairs(8, 2)),
         "alltoall_three_step_3x4": lambda: from_program(lambda: three_step(3, 4)),

@@ -203,6 +203,7 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
         "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
         "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed
+        "c5_chain": (1024, 128, 16, 16384, 1, 1),
     }
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)

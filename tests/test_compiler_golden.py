@@ -23,12 +23,13 @@ PROGRAMS = {
     "c4_hierarchical_allreduce_8x4_2inst_auto": lambda: catalog.two_level_allreduce(8, 4, 2),
     "c4_hierarchical_allreduce_4x2_1inst_manual": lambda: catalog.two_level_allreduce(4, 2, 1, schedule="manual"),
     "c5_allreduce_ring_64r_1ch_1inst": lambda: catalog.ring_allreduce(64, 1, 1),
+    "c5_allreduce_chain_64r": lambda: catalog.chain_allreduce(64),
     "allreduce_ring_8r_4ch_8inst": lambda: catalog.ring_allreduce(8, 4, 8),
     "allreduce_allpairs_8r_2inst": lambda: catalog.allpairs_allreduce(8, 2, protocol="LL"),
     "alltoall_three_step_3x4": lambda: catalog.three_step_alltoall(3, 4),
 }
 BYTE_IDENTICAL = ["c1_allreduce_ring_8r_1ch_1inst", "c2_allgather_ring_8r_1ch_4inst", "c4_hierarchical_allreduce_8x4_2inst_auto",
-                  "c4_hierarchical_allreduce_4x2_1inst_manual", "c5_allreduce_ring_64r_1ch_1inst", "allreduce_ring_8r_4ch_8inst"]
+                  "c4_hierarchical_allreduce_4x2_1inst_manual", "c5_allreduce_ring_64r_1ch_1inst", "c5_allreduce_chain_64r", "allreduce_ring_8r_4ch_8inst"]
 
 
 def _anonymous(xml):

@@ -19,7 +19,7 @@ from test_gpu_parity import to_numpy, to_torch
 
 pytestmark = pytest.mark.gpu
 
-REDUCED = {"c1": 8 * 4 * 5000, "c2": 4 * 4 * 30000, "c3": 16 * 70000, "c4": 64 * 2 * 3000, "c5": 64 * 2 * 2048}
+REDUCED = {"c1": 8 * 4 * 5000, "c2": 4 * 4 * 30000, "c3": 16 * 70000, "c4": 64 * 2 * 3000, "c5": 64 * 2 * 2048, "c5_chain": 2 * 30000}
 
 
 def device_run(xml, w, inputs_np, **knobs):
@@ -63,9 +63,10 @@ def test_config_reduced_size_vs_oracle(key, source, mode):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
 
 
-@pytest.mark.parametrize("name", golden_util.names())
+@pytest.mark.parametrize("name", golden_util.names() + golden_util.ncclize_names())
 def test_reference_emitted_programs_vs_oracle(name):
-    """Every program msccl-tools' compiler emitted for the fixtures, whatever its collective: all
+    """Every program msccl-tools' compiler (tests/golden/reference_xml) and its second emitter, ncclize
+    (tests/golden/ncclize_xml), emitted for the fixtures, whatever its collective: all
     three buffers of every rank start from the same random bits on both sides and must end equal,
     with payloads read in place, with everything staged, and with flag-in-data lines."""
     from msccl.executor import Executor
@@ -93,6 +94,26 @@ def test_reference_emitted_programs_vs_oracle(name):
             for b in "ios":
                 if want[r][b].size:
                     assert np.array_equal(got[b].cpu().numpy().view(np.uint32), want[r][b].view(np.uint32)), (name, r, b, mode)
+
+
+@pytest.mark.parametrize("name", golden_util.ncclize_names())
+def test_ncclize_emitted_programs_match_their_send_lists_on_device(name):
+    """The documents ncclize emitted, on the device, against what their hand-written send lists mean
+    (no interpreter in between): 32-bit integers, ragged chunks, automatic geometry."""
+    from msccl.executor import Executor
+    from test_configs_oracle import _ncclize_case, _ncclize_expected
+    E = 2501
+    algo, x = _ncclize_case(name, E, seed=21)
+    ex = Executor(golden_util.load(name))
+    print(f"case: {name} closed form", flush=True)
+    ex.setup(E * 4, "int32")
+    ins = [torch.from_numpy(v).cuda() if v.size else None for v in x]
+    outs = [torch.zeros(g.o_chunks * E, dtype=torch.int32, device="cuda") if g.o_chunks else None for g in algo.gpus]
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    for r, (buf, want) in _ncclize_expected(name, algo, x, E).items():
+        got = (outs if buf == "o" else ins)[r].cpu().numpy()
+        assert np.array_equal(got[:want.size], want), (name, r)
 
 
 def torch_fold(order, operands):

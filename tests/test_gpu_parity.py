@@ -107,6 +107,41 @@ def test_ring_allreduce_redops(dtype, redop, protocol):
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "float64"])
+@pytest.mark.parametrize("redop", ["max", "min", "sum"])
+def test_nan_operands(dtype, redop):
+    """max and min drop a NaN operand (fmax / fmin, as the oracle does), sum propagates it: a quarter of
+    every rank's elements are quiet NaNs, at places that differ from rank to rank, so chunks meet NaN
+    against number, number against NaN and NaN against NaN along the ring."""
+    from msccl.executor import Executor, collective_buffers
+    n, E = 4, 2048
+    xml = ir_samples.ring_allreduce_xml(n)
+    algo = oi.parse_xml(xml)
+    x = make_inputs(n, n * E, dtype, seed=90)
+    rng = np.random.default_rng(91)
+    for r in range(n):
+        holes = rng.random(n * E) < 0.25
+        if dtype == "bfloat16":
+            x[r][holes] = 0x7FC0
+        else:
+            x[r][holes] = np.nan
+    want = oc.place_inputs(algo, x, E, dtype)
+    oi.Interpreter(algo).run(want, E, dtype, redop)
+    ex = Executor(xml)
+    print(f"case: NaN operands dtype={dtype} redop={redop}", flush=True)
+    ex.setup(E * oi.DTYPES[dtype]().itemsize, dtype, redop)
+    ins, outs, _ = collective_buffers(ex.tables, E * oi.DTYPES[dtype]().itemsize, dtype, inputs=[to_torch(v, dtype) for v in x])
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    as_float = (lambda v: oi.bf16_bits_to_f32(v)) if dtype == "bfloat16" else (lambda v: v)
+    for r in range(n):
+        got, ref = to_numpy(ins[r], dtype), want[r]["i"]
+        gn, rn = np.isnan(as_float(got)), np.isnan(as_float(ref))
+        assert np.array_equal(gn, rn), (r, int(gn.sum()), int(rn.sum()))           # NaN exactly where the oracle has NaN
+        assert 0 < rn.sum() < rn.size
+        assert np.array_equal(got[~rn].view(np.uint8), ref[~rn].view(np.uint8)), r  # and the same bits everywhere else
+
+
 @pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("n,inst", [(2, 1), (8, 4), (5, 2)])
 def test_ring_allgather(n, inst, protocol):

@@ -190,3 +190,19 @@ def test_ncclize_style_allreduce():
     want = (x[0] + x[1]) + x[2]
     for r in range(3):
         assert np.array_equal(outs[r].view(np.uint32), want.view(np.uint32))
+
+
+def test_max_min_drop_nan_like_fmax():
+    """max/min treat a NaN operand as missing (fmax/fmin), on every floating-point type; sum keeps it."""
+    nan = np.float32(np.nan)
+    a = np.array([1.0, nan, -2.0, nan], np.float32)
+    b = np.array([nan, 3.0, -5.0, nan], np.float32)
+    for dtype, conv, back in (("float32", lambda v: v, lambda v: v), ("float64", lambda v: v.astype(np.float64), lambda v: v),
+                              ("float16", lambda v: v.astype(np.float16), lambda v: v),
+                              ("bfloat16", oi.f32_to_bf16_bits, oi.bf16_bits_to_f32)):
+        mx = back(oi._reduce(conv(a), conv(b), dtype, "max")).astype(np.float64)
+        mn = back(oi._reduce(conv(a), conv(b), dtype, "min")).astype(np.float64)
+        assert mx[:3].tolist() == [1.0, 3.0, -2.0] and np.isnan(mx[3]), dtype
+        assert mn[:3].tolist() == [1.0, 3.0, -5.0] and np.isnan(mn[3]), dtype
+        sm = back(oi._reduce(conv(a), conv(b), dtype, "sum")).astype(np.float64)
+        assert np.isnan(sm[[0, 1, 3]]).all() and sm[2] == -7.0, dtype

@@ -56,12 +56,12 @@ def test_registered_allreduce_allpairs(capsys):
     assert types[1] == types[2] == 8 * 7 * 2 * 2
 
 
-def test_catalog_builds_the_five_workloads():
+def test_catalog_builds_the_workloads():
     from msccl.executor.workloads import WORKLOADS
-    expect = {"c1": (8, 8, 120), "c2": (8, 32, 256), "c3": (16, 256, 624), "c4": (32, 1920, 4480), "c5": (64, 64, 8128)}
+    expect = {"c1": (8, 8, 120), "c2": (8, 32, 256), "c3": (16, 256, 624), "c4": (32, 1920, 4480), "c5": (64, 64, 8128), "c5_chain": (64, 64, 127)}
     for key, w in WORKLOADS.items():
         t = parse_algo_xml(w.build())
         assert (t.ngpus, t.ntbs, t.nops) == expect[key], key
         assert t.algorithmic_units() * w.chunk_bytes == {"c1": 5 * 7 * (1 << 20), "c2": 2 * 7 * 8 * (32 << 20),
                                                          "c3": 3 * 16 * (64 << 20), "c4": 5 * 31 * (128 << 20),
-                                                         "c5": 5 * 63 * (256 << 10)}[key]
+                                                         "c5": 5 * 63 * (256 << 10), "c5_chain": 5 * 63 * (256 << 10)}[key]
