@@ -104,7 +104,7 @@ typedef struct {
   int32_t slices;      /* independent copies of the program, each on a 1/slices part of every chunk */
   int32_t piece_bytes; /* bytes of one chunk moved per step per pass of the step list            */
   int32_t fifo_depth;  /* messages a connection can hold                                         */
-  int32_t threads;     /* threads per workgroup: 64, 128, 256 or 512                             */
+  int32_t threads;     /* threads per workgroup: 64, 128, 256, 512 or 1024                       */
   int32_t timeout_ms;  /* in-kernel watchdog; default 10000                                      */
   int32_t max_workgroups; /* cap on resident workgroups assumed when no device is queried (tests) */
   int32_t staging;     /* 0: a receiver reads a payload in place where that is provably safe; 1: always stage in FIFO slots */
@@ -126,6 +126,8 @@ typedef struct {
   int32_t staged_messages;
   int32_t max_hosted;  /* most contexts any workgroup hosts                         */
   int32_t protocol;    /* MSCCLX_PROTO_SIMPLE or MSCCLX_PROTO_LL                    */
+  int32_t waiting_ratio_x100; /* 100 * threadblocks * depth of the dataflow / moving steps: 100 = every threadblock always has work (a ring) */
+  int32_t dataflow_depth;     /* moving steps on the longest chain through step order, dependencies and messages */
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

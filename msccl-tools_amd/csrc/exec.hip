@@ -91,14 +91,14 @@ static bool has_foldable_nops(const mscclx_plan& plan) {
   return false;
 }
 
-static int query_capacity(kernel_fn k, int* num_cus, int capacity[4]) {
+static int query_capacity(kernel_fn k, int* num_cus, int capacity[kThreadChoices]) {
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, dev));
   *num_cus = prop.multiProcessorCount;
-  const int threads[4] = {64, 128, 256, 512};
-  for (int i = 0; i < 4; ++i) {
+  const int threads[kThreadChoices] = {64, 128, 256, 512, 1024};
+  for (int i = 0; i < kThreadChoices; ++i) {
     int per_cu = 0;
     HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, threads[i], 0));
     capacity[i] = per_cu * prop.multiProcessorCount;
@@ -418,9 +418,9 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
   const bool vec = chunk_bytes % 16 == 0;
   int num_cus = 256;
-  int capacity[4];
+  int capacity[kThreadChoices];
   if (cfg.max_workgroups > 0) {
-    for (int i = 0; i < 4; ++i) capacity[i] = cfg.max_workgroups;
+    for (int i = 0; i < kThreadChoices; ++i) capacity[i] = cfg.max_workgroups;
   } else {
     const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
     int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, vec && !ll && has_foldable_nops(*plan)), &num_cus, capacity);
@@ -443,6 +443,8 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     info->workgroups = g.workgroups;
     info->max_hosted = g.max_hosted;
     info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
+    info->waiting_ratio_x100 = (int32_t)std::min(2.0e9, g.waiting_ratio * 100.0 + 0.5);
+    info->dataflow_depth = g.dataflow_depth;
     info->threads = g.threads;
     info->slices = g.slices;
     info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);

@@ -795,7 +795,7 @@ __device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, 
 // FOLD: steps may carry the dependencies of nop steps folded into them (a kernel of its own, so that
 // programs without such steps do not pay for the check in the poll loop).
 template <class R, bool VEC, bool LL, bool FOLD = false>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
   static_assert(VEC || !LL, "LL lines carry 16-byte units");
   constexpr int EB = R::kElemBytes;
   constexpr uint64_t UB = VEC ? 16 : EB;

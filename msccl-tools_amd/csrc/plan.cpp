@@ -357,7 +357,7 @@ static int build_plan(const mscclx_plan_desc* d, mscclx_plan* p) {
 }
 
 static int thread_index(int threads) {
-  switch (threads) { case 64: return 0; case 128: return 1; case 256: return 2; case 512: return 3; default: return -1; }
+  switch (threads) { case 64: return 0; case 128: return 1; case 256: return 2; case 512: return 3; case 1024: return 4; default: return -1; }
 }
 
 // bytes a threadblock moves per chunk-sized unit of its steps, given which payloads are staged
@@ -456,7 +456,7 @@ static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t sli
 }
 
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
-                    int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out) {
+                    int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);
   if (!elem) return fail(MSCCLX_ERR_INVALID_ARG, "unknown dtype " + std::to_string(dtype));
   if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
@@ -484,10 +484,11 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     depth = std::max(depth, 2);
   }
   g.depth = depth;
+  g.waiting_ratio = waiting_ratio(plan, &g.dataflow_depth);
 
   // Slices are independent copies of the program on 1/slices of every chunk; they are what keeps
   // the chip busy while one copy waits on its dependency chain.
-  const int most_threads_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
+  const int most_threads_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + kThreadChoices);
   const int64_t host_limit = (int64_t)most_threads_capacity * kMaxHosted;
   if (ntbs > host_limit)
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
@@ -506,7 +507,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // pass k of a later one).  Candidates are scored on (1) and (2); (3) follows below.
       std::vector<uint64_t> works;
       for (const Tb& tb : plan.tbs) works.push_back(tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL));
-      const int most_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + 4);
+      const int most_capacity = *std::max_element(capacity_by_threads, capacity_by_threads + kThreadChoices);
       const int64_t lo = std::max<int64_t>(1, to_fill);
       const double wanted_per_wg = std::min(32.0, 4.0 * waiting_ratio(plan));
       // pieces of 16 KiB only where 32 KiB pieces leave less than a quarter of the contexts wanted in (2)
@@ -630,7 +631,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   // threads: enough to cover a piece with 8 16-byte loads per thread
   int threads = cfg.threads;
   if (threads) {
-    if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256 or 512");
+    if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256, 512 or 1024");
   } else {
     const uint64_t piece_bytes = piece_units * g.unit_bytes;
     threads = threads_for_piece(piece_bytes);

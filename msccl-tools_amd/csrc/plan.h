@@ -8,6 +8,8 @@
 
 namespace mscclx {
 
+constexpr int kThreadChoices = 5;  // workgroups of 64, 128, 256, 512 or 1024 threads
+
 // One <step>, plus what plan_create derives for it.
 struct Op {
   int32_t type, srcbuf, srcoff, dstbuf, dstoff, cnt, depid, deps, hasdep;
@@ -100,6 +102,8 @@ struct Geometry {
   int32_t max_hosted = 0;
   std::vector<int32_t> wg_begin, ctx_tb, ctx_slice;  // the hosting table
   int32_t passes = 0;
+  double waiting_ratio = 1.0;     // threadblocks x depth of the dataflow / moving steps
+  int32_t dataflow_depth = 1;
   uint64_t slice_fifo_units = 0;  // FIFO units one slice needs (all connections)
   uint64_t sync_words = 0;        // uint64 words of ONE synchronisation area (there are two)
   uint64_t sync_slice_words = 0;  // words per slice inside an area
@@ -192,6 +196,6 @@ int dtype_size(int dtype);
 int simulate(const mscclx_plan& plan, int depth);
 // Pure geometry decision (no HIP): max_wgs = resident workgroup capacity per thread count.
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
-                    int num_cus, const int capacity_by_threads[4], uint64_t fifo_budget_bytes, Geometry* out);
+                    int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out);
 void destroy_device_state(DeviceState* d);
 }  // namespace mscclx

@@ -65,6 +65,7 @@ class Info(ctypes.Structure):
                 ("connections", ctypes.c_int32), ("vector_path", ctypes.c_int32),
                 ("zero_copy_messages", ctypes.c_int32), ("staged_messages", ctypes.c_int32),
                 ("max_hosted", ctypes.c_int32), ("protocol", ctypes.c_int32),
+                ("waiting_ratio_x100", ctypes.c_int32), ("dataflow_depth", ctypes.c_int32),
                 ("workspace_bytes", ctypes.c_uint64), ("algorithmic_units", ctypes.c_uint64)]
 
     def as_dict(self):

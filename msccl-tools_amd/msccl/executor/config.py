@@ -50,9 +50,11 @@ def load_config(path=None):
 
 
 def select(algos, coll, nbytes, ngpus=None):
-    """First listed algorithm for collective `coll` whose window holds `nbytes`
-    (minBytes <= nbytes <= maxBytes), optionally with `ngpus` ranks; None if there is none."""
+    """First listed algorithm for collective `coll` whose window holds `nbytes`, optionally with
+    `ngpus` ranks; None if there is none.  Windows are half-open, minBytes <= nbytes < maxBytes, the
+    convention of the emitter: a single size n is written as (n, n + 1) and adjacent plans share
+    their boundary value (msccl/autosynth/__init__.py:57-68)."""
     for a in algos:
-        if a.tables.coll == str(coll) and a.min_bytes <= nbytes <= a.max_bytes and (ngpus is None or a.tables.ngpus == ngpus):
+        if a.tables.coll == str(coll) and a.min_bytes <= nbytes < a.max_bytes and (ngpus is None or a.tables.ngpus == ngpus):
             return a
     return None

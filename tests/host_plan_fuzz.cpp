@@ -22,7 +22,7 @@ static int run_once(int nranks, const std::vector<int32_t>& rc, const std::vecto
   (void)mscclx_plan_simulate(p, 0);
   (void)mscclx_plan_simulate(p, 2);
   (void)mscclx_plan_algorithmic_units(p);
-  const int capacity[4] = {4096, 2048, 1024, 512};
+  const int capacity[mscclx::kThreadChoices] = {4096, 2048, 1024, 512, 256};
   mscclx::Geometry g;
   for (int variant = 0; variant < variants; ++variant)  // 0 automatic, 1 LL lines, 2 explicit knobs with staging
   for (size_t chunk : {(size_t)4, (size_t)4096, (size_t)(1 << 20) + 16, (size_t)3 << 20}) {

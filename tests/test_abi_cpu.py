@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
 
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(binding.Config) == 48
-    assert ctypes.sizeof(binding.Info) == 64
+    assert ctypes.sizeof(binding.Info) == 72
     assert ctypes.sizeof(binding.Status) == 32
 
 

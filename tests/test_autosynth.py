@@ -112,6 +112,25 @@ def test_index_roundtrip_and_selection(capsys):
     assert algos[2].tables.nchunksperloop == 64 and algos[2].bytes_per_rank_to_chunk_bytes(1 << 20) == (1 << 20) // 64
 
 
+def test_selection_windows_are_half_open(capsys):
+    """A size on the boundary two plans share belongs to the upper one: windows are [minBytes, maxBytes),
+    the interval convention of msccl.init (msccl/autosynth/__init__.py:57-68,130-131)."""
+    msccl.init('mi355x', 1, ('allreduce', (0, None)))
+    capsys.readouterr()
+    algos = load_config()
+    windows = [(a.min_bytes, a.max_bytes, a.tables.nchunksperloop) for a in algos]
+    assert windows == [(0, 16000000, 64), (16000000, float("inf"), 32)]       # all-pairs below 16 MB, the ring from there on
+    assert select(algos, "allreduce", 15999999) is algos[0]
+    assert select(algos, "allreduce", 16000000) is algos[1]
+    # msccl.init treats a requested size the same way: exactly 16 MB asks for [16000000, 16000001), which only the ring's window meets
+    msccl.init('mi355x', 1, ('allreduce', 16000000))
+    capsys.readouterr()
+    assert [(a.min_bytes, a.max_bytes, a.tables.nchunksperloop) for a in load_config()] == [(16000000, float("inf"), 32)]
+    msccl.init('mi355x', 1, ('allreduce', 15999999))
+    capsys.readouterr()
+    assert [(a.min_bytes, a.max_bytes, a.tables.nchunksperloop) for a in load_config()] == [(0, 16000000, 64)]
+
+
 def test_ef_file_plan(tmp_path, capsys):
     import ir_samples
     f = tmp_path / "ring.xml"
