@@ -6,12 +6,23 @@
         ...
         XML(); Check()
 
-The user-facing names and their meaning follow msccl-tools' msccl/language/__init__.py:
-MSCCLProgram and its keyword arguments (:23-50), the symbolic effect of a copy (dst = src, :65-71)
-and of a reduce (dst = dst (+) src, :74-82), `lower()` (:107-126), `chunk`/`XML`/`Check`
-(:144-156) and `Ref.copy` / `Ref.reduce` / `split` / `group` (:171-254).
+The user-facing names and their meaning are msccl-tools' (msccl/language/__init__.py): MSCCLProgram
+and its keyword arguments (:23-50), what a copy (dst = src, :65-71) and a reduce (dst = dst (+) src,
+:74-82) do to the symbolic buffers, `lower()` (:107-126), `chunk` / `XML` / `Check` (:144-156) and
+`Ref.copy` / `Ref.reduce` / `split` / `group` (:171-254).
+
+How this module is put together is its own: a traced program is three things kept apart --
+
+* `SymbolicMemory`: what every slot of every rank's buffers holds (the collective's pre-condition
+  at first), with the collective's aliasing of in-place buffers applied where a location is named;
+* a list of `Transfer`s as the user issues them -- one record per `copy` / `reduce`, which
+  `MSCCLProgram.record` turns into the symbolic effect and into the instruction DAG's nodes (a local
+  instruction, or a send matched with its receive);
+* `LOWERING`, the ordered passes that take the instruction DAG to per-threadblock step lists.
 """
 from __future__ import annotations
+
+import dataclasses
 
 from msccl.language.ir import (Buffer, ChunkInstruction, ChunkRef, Gpu, Instruction, Op, Program, Threadblock,
                                ThreadblockPolicy, ir_to_xml)
@@ -21,99 +32,169 @@ from msccl.language.dag import InstructionDAG
 from msccl.language.scheduling import auto_assign_tbs, manual_assign_tbs, topo_sort_instrs, channel_assignment
 from msccl.language.checks import ScheduleError, check_dependency_cycles, check_threadblock_ordering
 
-_current_program = None
+PROTOCOLS = ("Simple", "LL", "LL128")
+
+# ---- the program being traced -------------------------------------------------------------------
+_active = []  # at most one entry: programs do not nest
 
 
-def _curr():
-    if _current_program is None:
+def active_program():
+    if not _active:
         raise RuntimeError("No Program in context")
-    return _current_program
+    return _active[0]
+
+
+# ---- symbolic state -------------------------------------------------------------------------------
+class SymbolicMemory:
+    """Per rank, per buffer, the symbolic chunk every slot holds.  Locations are always resolved
+    through the collective first, so that the two names of an aliased in-place buffer mean one slot."""
+
+    def __init__(self, collective):
+        self.collective = collective
+        self.buffers = collective.init_buffers()
+
+    def resolve(self, rank, buffer, index):
+        return self.collective.get_buffer_index(rank, buffer, index)
+
+    def slots(self, rank, buffer, index):
+        buffer, index = self.resolve(rank, buffer, index)
+        return self.buffers[rank][buffer], index
+
+    def populated_inputs(self, rank):
+        """Resolved (buffer, index) of every slot of the rank's input buffer, in order."""
+        return [self.resolve(rank, Buffer.input, k) for k in range(len(self.buffers[rank][Buffer.input]))]
+
+    def holds(self, rank, buffer, index):
+        return self.buffers[rank][buffer][index] is not None
+
+    def peek(self, rank, buffer, index, size=1):
+        store = self.buffers[rank][buffer]
+        return [store[index + k] if store and index + k < len(store) else None for k in range(size)]
+
+    def scratch(self, rank, name):
+        """The named scratch buffer of a rank, created on first use; standard buffers pass through."""
+        if name is not None and name not in self.buffers[rank]:
+            self.buffers[rank][name] = BufferSlice(Buffer.scratch, name)
+        return self.buffers[rank].get(name)
+
+    def overwrite(self, src, dst, size):
+        (sb, si), (db, di) = self.slots(*src), self.slots(*dst)
+        for k in range(size):
+            db[di + k] = sb[si + k]
+
+    def accumulate(self, src, dst, size):
+        (sb, si), (db, di) = self.slots(*src), self.slots(*dst)
+        for k in range(size):
+            db[di + k] = db[di + k].reduce(dst[0], sb[si + k])
+
+
+@dataclasses.dataclass(frozen=True)
+class Transfer:
+    """One `copy` or `reduce` as the user wrote it."""
+    reduces: bool
+    src: "Ref"
+    dst: "Ref"
+    sendtb: int = -1
+    recvtb: int = -1
+    ch: int = -1
+
+    @property
+    def local(self):
+        return self.src.rank == self.dst.rank
+
+
+# ---- lowering -----------------------------------------------------------------------------------
+def _fuse(prog, dag):
+    if prog.instr_fusion:
+        dag.optimize()
+
+
+def _assign_threadblocks(prog, dag):
+    (manual_assign_tbs if prog.threadblock_policy == ThreadblockPolicy.manual else auto_assign_tbs)(dag)
+
+
+def _verify(prog, dag):
+    if prog.check_xml:
+        check_dependency_cycles(dag.tbs)
+        check_threadblock_ordering(dag)
+
+
+# (name, pass over (program, instruction DAG)); `replicate` is where the per-rank Gpu objects appear
+LOWERING = (
+    ("normalise", lambda prog, dag: dag.convert_set_list()),
+    ("fuse", _fuse),
+    ("measure", lambda prog, dag: dag._complete_metadata()),
+    ("assign threadblocks", _assign_threadblocks),
+    ("order steps", lambda prog, dag: dag.lower_pt1(prog.instances)),
+    ("replicate", lambda prog, dag: dag.lower_pt2(prog.instances, prog.interleaved_replication)),
+    ("verify", _verify),
+)
 
 
 class MSCCLProgram:
     def __init__(self, name, topo, collective, instances, protocol="Simple", threadblock_policy=ThreadblockPolicy.auto,
                  interleaved_replication=True, instr_fusion=True, check_xml=True, dependence_nop=False):
-        assert protocol in ("Simple", "LL", "LL128"), f"Given protocol: {protocol}. Must be either Simple, LL, LL128"
-        self.name = name
-        self.topo = topo
-        self.collective = collective
+        assert protocol in PROTOCOLS, f"Given protocol: {protocol}. Must be either Simple, LL, LL128"
+        self.name, self.topo, self.collective, self.instances = name, topo, collective, instances
         self.num_ranks = topo.num_nodes()
-        self.instances = instances
         self.protocol = protocol
         self.threadblock_policy = threadblock_policy
         self.interleaved_replication = interleaved_replication
         self.instr_fusion = instr_fusion
         self.check_xml = check_xml
         self.dependence_nop = dependence_nop
-        self.buffers = collective.init_buffers()
+        self.memory = SymbolicMemory(collective)
+        self.buffers = self.memory.buffers  # (user collectives' check() reads prog.buffers)
+        self.transfers = []
         self.instr_dag = InstructionDAG(self.num_ranks, self.buffers)
         # every slot of every input buffer starts life written by a `start` pseudo-op
-        for r in range(self.num_ranks):
-            for k in range(len(self.buffers[r][Buffer.input])):
-                buffer, index = collective.get_buffer_index(r, Buffer.input, k)
-                self.instr_dag.add_start(r, buffer, index, self.get_ref(r, buffer, index, 1))
+        for rank in range(self.num_ranks):
+            for buffer, index in self.memory.populated_inputs(rank):
+                self.instr_dag.add_start(rank, buffer, index, Ref(rank, buffer, index, 1, self))
 
     def __enter__(self):
-        global _current_program
-        if _current_program is not None:
+        if _active:
             raise RuntimeError("There is already a MSCCL Program in context")
-        _current_program = self
+        _active.append(self)
         return self
 
     def __exit__(self, exc_type, exc_value, exc_traceback):
-        global _current_program
-        if _current_program is not self:
+        if not _active or _active[0] is not self:
             raise RuntimeError("This program is not currently in context")
-        _current_program = None
+        _active.clear()
 
-    # ---- symbolic execution ---------------------------------------------------------------------
-    def _slots(self, rank, buffer, index):
-        buffer, index = self.collective.get_buffer_index(rank, buffer, index)
-        return self.buffers[rank][buffer], index
-
-    def apply_send(self, src, src_buffer, src_index, dst, dst_buffer, dst_index, size):
-        sb, si = self._slots(src, src_buffer, src_index)
-        db, di = self._slots(dst, dst_buffer, dst_index)
-        for k in range(size):
-            db[di + k] = sb[si + k]
-
-    def apply_reduce(self, src, src_buffer, src_index, dst, dst_buffer, dst_index, size):
-        sb, si = self._slots(src, src_buffer, src_index)
-        db, di = self._slots(dst, dst_buffer, dst_index)
-        for k in range(size):
-            db[di + k] = db[di + k].reduce(dst, sb[si + k])
-
+    # ---- tracing ----------------------------------------------------------------------------------
     def get_ref(self, rank, buffer, index, size):
-        buffer, index = self.collective.get_buffer_index(rank, buffer, index)
+        buffer, index = self.memory.resolve(rank, buffer, index)
         return Ref(rank, buffer, index, size, self)
 
     def get_chunks(self, rank, buffer, index, size=1):
-        buf = self.buffers[rank][buffer]
-        return [buf[index + k] if buf and index + k < len(buf) else None for k in range(size)]
+        return self.memory.peek(rank, buffer, index, size)
 
-    def check_buffer_exists(self, rank, name):
-        if name is not None and name not in self.buffers[rank]:
-            self.buffers[rank][name] = BufferSlice(Buffer.scratch, name)
+    def record(self, t):
+        """Take one Transfer: it must follow a link of the topology; the symbolic buffers change;
+        the instruction DAG gets a local instruction, or a send and the receive that matches it."""
+        assert t.local or self.topo.link(t.src.rank, t.dst.rank), f"No link from {t.src.rank} to {t.dst.rank}"
+        src_at, dst_at = (t.src.rank, t.src.buffer, t.src.index), (t.dst.rank, t.dst.buffer, t.dst.index)
+        (self.memory.accumulate if t.reduces else self.memory.overwrite)(src_at, dst_at, t.dst.size)
+        self.transfers.append(t)
+        dag = self.instr_dag
+        if t.local:
+            (dag.add_reduce if t.reduces else dag.add_copy)(t.src.rank, t.src, t.dst, t.sendtb, t.ch)
+            return
+        send = dag.add_send(t.src.rank, t.src, t.dst, t.sendtb, t.ch)
+        receive = (dag.add_recv_reduce_copy if t.reduces else dag.add_recv)(t.dst.rank, t.src, t.dst, t.recvtb, t.ch, send)
+        send.recv_match = receive
 
     def check(self):
         return self.collective.check(self)
 
     # ---- lowering ---------------------------------------------------------------------------------
     def lower(self):
-        dag = self.instr_dag
-        dag.convert_set_list()
-        if self.instr_fusion:
-            dag.optimize()
-        dag._complete_metadata()
-        if self.threadblock_policy == ThreadblockPolicy.manual:
-            manual_assign_tbs(dag)
-        else:
-            auto_assign_tbs(dag)
-        dag.lower_pt1(self.instances)
-        gpus = dag.lower_pt2(self.instances, self.interleaved_replication)
-        if self.check_xml:
-            check_dependency_cycles(dag.tbs)
-            check_threadblock_ordering(dag)
+        gpus = None
+        for _stage, run in LOWERING:
+            out = run(self, self.instr_dag)
+            gpus = out if out is not None else gpus
         return Program(self.name, self.collective.name, self.collective.inplace, self.protocol, gpus)
 
     def generate_xml(self):
@@ -121,17 +202,16 @@ class MSCCLProgram:
 
 
 def chunk(rank, buffer, index, size=1):
-    if _curr().buffers[rank][buffer][index] is None:
-        return None
-    return _curr().get_ref(rank, buffer, index, size)
+    prog = active_program()
+    return prog.get_ref(rank, buffer, index, size) if prog.memory.holds(rank, buffer, index) else None
 
 
 def XML():
-    print(_curr().generate_xml())
+    print(active_program().generate_xml())
 
 
 def Check():
-    return _curr().check()
+    return active_program().check()
 
 
 class Ref(ChunkRef):
@@ -141,21 +221,21 @@ class Ref(ChunkRef):
         super().__init__(rank, buffer, index, size)
         self.prog = prog
 
+    def _key(self):
+        return (self.rank, self.buffer, self.index, self.size)
+
     def __eq__(self, other):
-        return (isinstance(other, ChunkRef) and (self.rank, self.buffer, self.index, self.size) ==
-                (other.rank, other.buffer, other.index, other.size))
+        return isinstance(other, ChunkRef) and self._key() == (other.rank, other.buffer, other.index, other.size)
 
     def __hash__(self):
-        return hash((self.rank, self.buffer, self.index, self.size))
+        return hash(self._key())
 
     def __repr__(self):
         return f"Ref(Buffer:{self.buffer}, Index:{self.index}, Size:{self.size}, Rank:{self.rank})"
 
-    def _end(self):
+    @property
+    def end(self):
         return self.index + self.size
-
-    def _get_chunk(self, index):
-        return self.prog.buffers[self.rank][self.buffer][index]
 
     def split(self, num):
         assert self.size % num == 0, f"Trying to split a chunk of {self.size} elements into {num} parts"
@@ -166,63 +246,56 @@ class Ref(ChunkRef):
         assert self.rank == other.rank, f"Trying to concatenate chunks on ranks {self.rank} and {other.rank}"
         assert self.buffer == other.buffer, f"Trying to concatenate chunks in {self.buffer} and {other.buffer}"
         first = min(self.index, other.index)
-        return Ref(self.rank, self.buffer, first, max(self._end(), other._end()) - first, self.prog)
+        return Ref(self.rank, self.buffer, first, max(self.end, other.end) - first, self.prog)
+
+    def _destination(self, dst, buffer, index):
+        """Where a copy to rank `dst` lands: the same place when nothing is said, the end of a
+        scratch buffer named without an index, else as given -- then through the collective's aliasing
+        (as seen from the SENDING rank, which is how msccl-tools resolves it, language/__init__.py:203)."""
+        memory = self.prog.memory
+        store = memory.scratch(dst, buffer)
+        if index == -1 and buffer is None:
+            buffer, index = self.buffer, self.index
+        elif index == -1 and buffer is not Buffer.input and buffer is not Buffer.output:
+            index = store.instance_size()
+        buffer, index = memory.resolve(self.rank, buffer, index)
+        return self.prog.get_ref(dst, buffer, index, self.size)
 
     def copy(self, dst, buffer=None, index=-1, sendtb=-1, recvtb=-1, ch=-1):
-        """Copy these chunks to rank `dst` at (buffer, index); returns the destination handle.
-        Without buffer and index the chunks keep their place; a scratch buffer named without an
-        index is appended to."""
-        prog = self.prog
-        prog.check_buffer_exists(dst, buffer)
-        if index == -1 and buffer is None:
-            index, buffer = self.index, self.buffer
-        elif index == -1 and buffer is not Buffer.input and buffer is not Buffer.output:
-            index = prog.buffers[dst][buffer].instance_size()
-        buffer, index = prog.collective.get_buffer_index(self.rank, buffer, index)
-        assert prog.topo.link(self.rank, dst) or dst == self.rank, f"No link from {self.rank} to {dst}"
-        target = prog.get_ref(dst, buffer, index, self.size)
+        """Copy these chunks to rank `dst` at (buffer, index); returns the destination handle
+        (None when source and destination are the same place)."""
+        target = self._destination(dst, buffer, index)
         if target == self:
             return None
-        prog.apply_send(self.rank, self.buffer, self.index, dst, buffer, index, self.size)
-        if dst != self.rank:
-            send = prog.instr_dag.add_send(self.rank, self, target, sendtb, ch)
-            recv = prog.instr_dag.add_recv(dst, self, target, recvtb, ch, send)
-            send.recv_match = recv
-        else:
-            prog.instr_dag.add_copy(self.rank, self, target, sendtb, ch)
+        self.prog.record(Transfer(False, self, target, sendtb, recvtb, ch))
         return target
 
     def reduce(self, other_chunkref, sendtb=-1, recvtb=-1, ch=-1):
         """self = self (+) other; returns self."""
-        prog = self.prog
-        dst, src = self.rank, other_chunkref.rank
-        assert prog.topo.link(src, dst) or src == dst, f"No link from {src} to {dst}"
-        prog.apply_reduce(src, other_chunkref.buffer, other_chunkref.index, dst, self.buffer, self.index, self.size)
-        if src != dst:
-            send = prog.instr_dag.add_send(src, other_chunkref, self, sendtb, ch)
-            recv = prog.instr_dag.add_recv_reduce_copy(dst, other_chunkref, self, recvtb, ch, send)
-            send.recv_match = recv
-        else:
-            prog.instr_dag.add_reduce(src, other_chunkref, self, sendtb, ch)
+        self.prog.record(Transfer(True, other_chunkref, self, sendtb, recvtb, ch))
         return self
 
+    # ---- what the symbolic chunk at a position of this handle says about itself --------------------
+    def _symbolic(self, index):
+        return self.prog.buffers[self.rank][self.buffer][self.index + index]
+
     def get_origin_index(self, index=0):
-        return self._get_chunk(index + self.index).origin_index
+        return self._symbolic(index).origin_index
 
     def get_origin_rank(self, index=0):
-        return self._get_chunk(index + self.index).origin_rank
+        return self._symbolic(index).origin_rank
 
     def get_dst_index(self, index=0):
-        return self._get_chunk(index + self.index).dst_index
+        return self._symbolic(index).dst_index
 
     def get_dst_rank(self, index=0):
-        return self._get_chunk(index + self.index).dst_rank
+        return self._symbolic(index).dst_rank
 
     def print_chunk_info(self, index=0):
-        print(self._get_chunk(index + self.index))
+        print(self._symbolic(index))
 
 
 __all__ = ["Buffer", "ChunkInstruction", "ChunkRef", "Gpu", "Instruction", "Op", "Program", "Threadblock", "ThreadblockPolicy",
            "ir_to_xml", "Chunk", "ReduceChunk", "BufferSlice", "InstructionDAG", "MSCCLProgram", "Ref", "chunk", "XML", "Check",
            "ScheduleError", "auto_assign_tbs", "manual_assign_tbs", "topo_sort_instrs", "channel_assignment",
-           "check_dependency_cycles", "check_threadblock_ordering"]
+           "check_dependency_cycles", "check_threadblock_ordering", "SymbolicMemory", "Transfer", "LOWERING", "active_program"]
