@@ -322,14 +322,38 @@ __device__ __forceinline__ u64 load_counter(const u64* p) { return __hip_atomic_
 __device__ __forceinline__ void publish(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 __device__ __forceinline__ u64 first_lane(u64 v) {  // the first lane's value, as a value the compiler knows to be the same in all lanes
-  return ((u64)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) | (u64)__builtin_amdgcn_readfirstlane((uint32_t)v);
+  // (the builtin returns int: each half goes through uint32_t, or a low half with its top bit set would
+  // sign-extend over the high half -- harmless for counters, fatal for addresses)
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)), lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  return ((u64)hi << 32) | (u64)lo;
 }
 
 __device__ __forceinline__ uint32_t lane_value(uint32_t v, int l) { return (uint32_t)__builtin_amdgcn_readlane((int)v, l); }  // l: the same in all lanes
 __device__ __forceinline__ u64 lane_value(u64 v, int l) { return ((u64)lane_value((uint32_t)(v >> 32), l) << 32) | (u64)lane_value((uint32_t)v, l); }
 
+// Values that are the same in all lanes but that the compiler holds in vector registers (anything
+// loaded from memory the kernel also writes): taken into scalar registers, so that addresses and
+// buffer descriptors built from them are scalar too -- a descriptor in vector registers costs a
+// loop of a dozen instructions around every load and store that uses it.
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t uniform(uint64_t v) { return (uint64_t)first_lane((u64)v); }
+__device__ __forceinline__ DevOp uniform(const DevOp& o) {
+  DevOp r;
+  r.word = uniform(o.word); r.dep_tb = uniform(o.dep_tb); r.dep_step = uniform(o.dep_step); r.dep_nops = uniform(o.dep_nops);
+  r.extra = uniform(o.extra); r.steps = uniform(o.steps);
+  r.src_addr = uniform(o.src_addr); r.dst_addr = uniform(o.dst_addr); r.in_addr = uniform(o.in_addr);
+  return r;
+}
+
 __device__ __forceinline__ bool is_recv(int t) { return t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS; }
 __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS; }
+
+// Between two polls of the same address.  It is more than a courtesy to the memory system: the
+// compiler treats a buffer load as a function of its arguments and takes a re-load with unchanged
+// arguments out of a loop that has nothing with a side effect in it -- the loop would then spin on
+// a register.  The pause is such a side effect.
+#define MSCCLX_POLL_PAUSE() __builtin_amdgcn_s_sleep(1)
 
 // ------------------------------------------------------------------------------------------------
 // LL lines.  One unit (16 payload bytes d0..d3) occupies 32 bytes of a slot: {d0,f,d1,f}{d2,f,d3,f}.
@@ -350,9 +374,9 @@ struct LLWatch {
 };
 
 // (arguments by value: a struct handed to a function that is not inlined would have to live in memory)
-__device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int tb, int step, int slice, u64 pass) {
+__device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int tb, int step, int slice, u64 pass, int waiting_on = 1) {
   if (atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
-    hs->tb = tb; hs->step = step; hs->slice = slice; hs->pass = (int64_t)pass; hs->waiting_on = 1;
+    hs->tb = tb; hs->step = step; hs->slice = slice; hs->pass = (int64_t)pass; hs->waiting_on = waiting_on;
     __threadfence_system();
     __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
@@ -388,6 +412,7 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
       for (;;) {
         const bool ok_a = ll_valid(a0, a1, fin), ok_b = ib >= n || ll_valid(b0, b1, fin);
         if (ok_a && ok_b) break;
+        MSCCLX_POLL_PAUSE();
         if (!ok_a) { a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)); a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16)); }
         if (!ok_b) { b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)); b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16)); }
         if ((++spins & 0x7fu) == 0) {
@@ -710,81 +735,171 @@ __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, ui
   }
 }
 
-// LL, one context on a workgroup of one wave: the wave runs the context with all its lanes.  Every
-// value of the bookkeeping is then the same in all lanes, so it lives in scalar registers and runs
-// on the scalar unit; there is no hand-over through LDS and no barrier, and the lanes go straight
-// from one message's lines to the next one's.  This is the shape of latency-bound programs (small
-// pieces, as many workgroups as contexts).  Measured on a 64-rank ring all-reduce of 2 KiB pieces it
-// takes 15% off the LL time; with the counter protocol it gains nothing (a hop is then bound by the
-// memory round trips of payload, acknowledgement and counter, not by instructions), so that
-// protocol always runs hosted.  Returns false if the launch was given up.
-template <class R, bool VEC, bool LL>
-__device__ __forceinline__ bool run_solo(const KernelParams& p, uint32_t epoch, int ctx, unsigned long long* prof4) {
-  constexpr int EB = R::kElemBytes;
-  constexpr int UB = VEC ? 16 : EB;
-  const bool writer = threadIdx.x == 0;
+// What a wait of run_chain does once in 64 polls: look at the abort word and at the clock.  Returns
+// the time the wait began (to be handed in again), or ~0 when the wait must be abandoned -- the
+// launch is lost, by this wait's own expiry (which it reports) or by somebody else's.
+__device__ __noinline__ u64 chain_slow_check(u64* abort_word, mscclx_status* hs, u64 timeout_ticks, u64 since, int tb, int step, int slice, u64 pass, int waiting_on) {
+  if (load_counter(abort_word) != 0) return ~0ull;
+  const u64 now = wall_clock64();
+  if (!since) return now;
+  if (now - since > timeout_ticks) {
+    ll_give_up(abort_word, hs, tb, step, slice, pass, waiting_on);
+    return ~0ull;
+  }
+  return since;
+}
+
+// LL, one context on a workgroup of one wave: the wave runs the context with all its lanes.  This is
+// the shape of latency-bound programs (small pieces, as many workgroups as contexts), where a launch
+// takes as long as the instructions and round trips of the longest chain of steps: a ring of one-wave
+// workgroups that does nothing but poll lines, add and store lines makes a round in 0.7 to 1.1 us
+// on MI355X (512 workgroups, 512-byte messages), and every instruction added to the loop shows.  So
+// this loop is written for that case and nothing else: every value of the bookkeeping is the same
+// in all lanes and is kept in scalar registers (`uniform`), so that addresses and buffer descriptors
+// are scalar; a step's state is a handful of running numbers; the table entry of the step after is
+// asked for before the wait for this step's message; the local operand and the outgoing
+// connection's tail are loaded together with the message's lines and looked at when the lines are
+// there; stores are waited for only where a flag announces them (lines announce themselves, and the
+// counter that frees the incoming slot only says that its lines were read).
+template <class R>
+__device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch, int ctx) {
+  typedef Access<16> A;
+  constexpr int XL = MSCCLX_AUX_LD, XP = (int)(0x80000000u | MSCCLX_AUX), XF = MSCCLX_AUX, XS = MSCCLX_AUX_ST, XN = MSCCLX_AUX_ST_FINAL;
+  const uint32_t lane = threadIdx.x;
+  const bool writer = lane == 0;
   u64* const abort_word = p.sync_cur;
   Hosted h;
-  Context c;
-  init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
-  unsigned busy_rounds = 0;
-  while (c.active) {
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t0 = wall_clock64();
-#endif
-    {  // wait until the step may start.  LL: not for the message itself -- the lines are retried by the threads that read them
-      const bool watch1 = c.w1 && !LL;
+  {
+    Context first;
+    init_context<true, R::kElemBytes, true>(h, first, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+    if (!first.active) return;
+  }
+  const DevOp* const ops = p.ops + uniform(h.op_begin);
+  const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
+  unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
+  const u64* const flags = p.sync_cur + uniform(h.flags);
+  const u64* const out_tail = p.sync_cur + uniform(h.tail_in);  // what the receiver of the outgoing connection has consumed
+  u64* const in_tail = p.sync_cur + uniform(h.tail_out);        // what this context has consumed of the incoming connection
+  u64* const my_flag = p.sync_cur + uniform(h.my_flag);
+  const uint32_t piece = p.piece_units, depth = (uint32_t)p.depth, nops = (uint32_t)uniform(h.nops), npasses = uniform(h.npasses);
+  const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
+  const int my_tb = uniform(h.tb), my_slice = uniform(h.slice);
+  uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
+  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice));
+  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice) * 16;
+  DevOp op = uniform(ops[0]);
+  for (;;) {
+    const DevOp after = ops[step + 1 == nops ? 0 : step + 1];  // (a table nobody writes: it arrives while the wave waits)
+    const int t = (int)(op.word & 15u);
+    const uint32_t cnt = op.word >> kOpCntShift;
+    const uint32_t n = left < piece ? left : piece;
+    bool lost = false;
+    if (op.dep_tb >= 0) {  // a step of another threadblock of this rank must have finished
+      const u64* const flag = flags + (uint32_t)op.dep_tb * kSyncStrideWords;
+      const u64 want = (u64)pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1;
       unsigned spins = 0;
-      u64 deadline = 0;
-      bool armed = false;
-      for (;;) {
-        // one lane asks memory, the wave shares the answers
-        u64 l0 = 0, l1 = 0, l2 = 0;
-        if (writer) {
-          if (c.w0) l0 = load_counter(c.w0);
-          if (watch1) l1 = load_counter(c.w1);
-          if (c.w2) l2 = load_counter(c.w2);
-        }
-        const u64 v0 = first_lane(l0), v1 = first_lane(l1), v2 = first_lane(l2);
-        const int what = (c.w0 && v0 < c.t0) ? 0 : (watch1 && v1 < c.t1) ? 1 : (c.w2 && v2 < c.t2) ? 2 : -1;
-        if (what < 0) break;
-        __builtin_amdgcn_s_sleep(1);
+      u64 since = 0;
+      while (uniform((uint64_t)load_counter(flag)) < want) {
+        MSCCLX_POLL_PAUSE();
         if ((++spins & 0x3fu) == 0) {
-          const u64 now = wall_clock64();
-          if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
-          if (load_counter(abort_word) != 0) return false;
-          if (now > deadline) {
-            if (writer && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
-              mscclx_status* hs = p.host_status;
-              hs->tb = h.tb; hs->step = c.step; hs->slice = h.slice; hs->pass = (int64_t)c.pass; hs->waiting_on = what;
-              __threadfence_system();
-              __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-            }
-            return false;
-          }
+          since = uniform((uint64_t)chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 0));
+          if (since == ~0ull) return;
         }
       }
     }
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t1 = wall_clock64();
-#endif
-    if (__builtin_expect((++busy_rounds & 0x3fu) == 0, 0) && first_lane(writer ? load_counter(abort_word) : 0) != 0) return false;  // a host's abort request
-    if (c.moves) do_move<R, VEC, LL>(c.m, p, epoch, c.rseq, c.sseq, h.tb, c.step, h.slice, c.pass);
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t2 = wall_clock64();
-#endif
-    const DevOp next = fetch_next_op(c, h, p);
-    if (c.moves) __builtin_amdgcn_s_waitcnt(0);  // this wave's stores are acknowledged: the counters may announce them
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t3 = wall_clock64();
-#endif
-    finish_step<UB, LL>(c, h, p, epoch, next, writer);
-#ifdef MSCCLX_PROFILE
-    const u64 prof_t4 = wall_clock64();
-    prof4[0] += prof_t1 - prof_t0; prof4[1] += prof_t2 - prof_t1; prof4[2] += prof_t3 - prof_t2; prof4[3] += prof_t4 - prof_t3;
-#endif
+    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(abort_word)) != 0) return;  // a host's abort request, a lost launch
+    const bool rcv = is_recv(t), snd = is_send(t);
+    const bool has_b = t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE;
+    const bool to_local = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
+    const bool nt = (op.word & kOpNtStore) != 0;
+    const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
+    const bool gated = snd && sseq >= depth;
+    const u64 gate_target = (u64)sseq + 1 - depth;
+    for (uint32_t row = 0; row < cnt; ++row) {
+      const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_ring + rslot + (u64)row * n * kLLUnitBytes, n * kLLUnitBytes);
+      const __amdgpu_buffer_rsrc_t rout = make_rsrc(out_ring + sslot + (u64)row * n * kLLUnitBytes, n * kLLUnitBytes);
+      const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)(op.src_addr + off + (u64)row * row_stride), n * 16);
+      const __amdgpu_buffer_rsrc_t rdst = make_rsrc((const void*)(op.dst_addr + off + (u64)row * row_stride), n * 16);
+      for (uint32_t base = 0; base < n; base += 128) {  // two units per lane at a time
+        const uint32_t i0 = base + lane, i1 = i0 + 64;
+        u32x4 a0 = {}, a1 = {}, b0 = {}, b1 = {}, x0 = {}, x1 = {}, y0 = {}, y1 = {};
+        if (rcv) {
+          a0 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes)); a1 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes + 16));
+          b0 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes)); b1 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes + 16));
+        } else if (t != MSCCLX_OP_NOP) {
+          x0 = A::template ld<XL>(rsrc, (int)(i0 * 16)); x1 = A::template ld<XL>(rsrc, (int)(i1 * 16));
+        }
+        if (has_b) { y0 = A::template ld<XL>(rdst, (int)(i0 * 16)); y1 = A::template ld<XL>(rdst, (int)(i1 * 16)); }
+        const bool first_of_step = row == 0 && base == 0;
+        u64 gate_seen = (gated && first_of_step) ? load_counter(out_tail) : ~0ull;
+        if (rcv) {
+          unsigned spins = 0;
+          u64 since = 0;
+          for (;;) {
+            const bool ok0 = i0 >= n || ll_valid(a0, a1, fin), ok1 = i1 >= n || ll_valid(b0, b1, fin);
+            if (ok0 && ok1) break;
+            MSCCLX_POLL_PAUSE();
+            if (!ok0) { a0 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes)); a1 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes + 16)); }
+            if (!ok1) { b0 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes)); b1 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes + 16)); }
+            if ((++spins & 0x3fu) == 0) {
+              since = chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 1);
+              if (since == ~0ull) { lost = true; break; }
+            }
+          }
+          x0 = u32x4{a0.x, a0.z, a1.x, a1.z};
+          x1 = u32x4{b0.x, b0.z, b1.x, b1.z};
+        }
+        if (has_b) { x0 = R::combine(y0, x0); x1 = R::combine(y1, x1); }
+        if (gated && first_of_step) {  // the slot may still be being read
+          unsigned spins = 0;
+          u64 since = 0;
+          while (gate_seen < gate_target && !lost) {
+            MSCCLX_POLL_PAUSE();
+            gate_seen = load_counter(out_tail);
+            if ((++spins & 0x3fu) == 0) {
+              since = chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 2);
+              if (since == ~0ull) lost = true;
+            }
+          }
+        }
+        if (__builtin_amdgcn_ballot_w64(lost) != 0) return;  // (the same decision in all lanes)
+        if (snd) {  // the forwarded lines first: the next rank is waiting for them
+          A::template st<XF>(rout, (int)(i0 * kLLUnitBytes), u32x4{x0.x, fout, x0.y, fout});
+          A::template st<XF>(rout, (int)(i0 * kLLUnitBytes + 16), u32x4{x0.z, fout, x0.w, fout});
+          A::template st<XF>(rout, (int)(i1 * kLLUnitBytes), u32x4{x1.x, fout, x1.y, fout});
+          A::template st<XF>(rout, (int)(i1 * kLLUnitBytes + 16), u32x4{x1.z, fout, x1.w, fout});
+        }
+        if (to_local) {
+          if (nt) { A::template st<XN>(rdst, (int)(i0 * 16), x0); A::template st<XN>(rdst, (int)(i1 * 16), x1); }
+          else { A::template st<XS>(rdst, (int)(i0 * 16), x0); A::template st<XS>(rdst, (int)(i1 * 16), x1); }
+        }
+      }
+    }
+    if (rcv) {
+      if (writer) publish(in_tail, (u64)rseq + 1);
+      ++rseq;
+      rslot += in_slot_bytes;
+      if (rslot == in_wrap) rslot = 0;
+    }
+    if (snd) {
+      ++sseq;
+      sslot += out_slot_bytes;
+      if (sslot == out_wrap) sslot = 0;
+    }
+    ++count;  // = pass * steps of the IR + IR step + 1 (nothing is folded under LL)
+    if (op.word & kOpHasdep) {
+      __builtin_amdgcn_s_waitcnt(0);
+      if (writer) publish(my_flag, (u64)count);
+    }
+    if (++step == nops) {
+      step = 0;
+      left -= n;
+      off += (u64)piece * 16;
+      if (++pass >= npasses) break;
+    }
+    op = uniform(after);
   }
-  return true;
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -834,11 +949,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
   if (LL && hosted == 1 && blockDim.x == 64) {
-    unsigned long long prof4[4] = {0, 0, 0, 0};
-    run_solo<R, VEC, LL>(p, epoch, ctx_begin, prof4);
-#ifdef MSCCLX_PROFILE
-    prof_wait = prof4[0]; prof_move = prof4[1]; prof_ack = prof4[2]; prof_fin = prof4[3];
-#endif
+    if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin);
   } else {
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
