@@ -761,20 +761,149 @@ __device__ __noinline__ u64 chain_slow_check(u64* abort_word, mscclx_status* hs,
 // connection's tail are loaded together with the message's lines and looked at when the lines are
 // there; stores are waited for only where a flag announces them (lines announce themselves, and the
 // counter that frees the incoming slot only says that its lines were read).
-template <class R>
-__device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch, int ctx) {
+#ifdef MSCCLX_PROFILE
+#define MSCCLX_CHAIN_CLOCK(var) const u64 var = __builtin_amdgcn_s_memtime()
+#define MSCCLX_CHAIN_ADD(k, a, b) (prof_acc[k] += (b) - (a))
+#else
+#define MSCCLX_CHAIN_CLOCK(var)
+#define MSCCLX_CHAIN_ADD(k, a, b)
+#endif
+// What run_chain's waits need in order to give up, kept together so that a wait passes one reference.
+struct ChainWatch {
+  u64* abort_word;
+  mscclx_status* host_status;
+  u64 timeout_ticks;
+  int tb, slice;
+};
+
+// One round of a step of run_chain: units i0, i0 + 64, ... (U of them per lane) of one row of n units.
+// Returns false when the launch is lost (the same answer in all lanes).  gate: the counter that must
+// reach gate_target before the outgoing slot may be written, or null.
+template <class R, int U>
+__device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rout, const __amdgpu_buffer_rsrc_t rsrc,
+                                            const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool rcv, const bool snd,
+                                            const bool from_src, const bool has_b, const bool to_local, const bool nt, const uint32_t fin,
+                                            const uint32_t fout, const u64* gate, const u64 gate_target, const ChainWatch& watch, const int step,
+                                            const uint32_t pass, u64* prof_acc, u64& prof_mark, const u64 prof_floor) {
   typedef Access<16> A;
   constexpr int XL = MSCCLX_AUX_LD, XP = (int)(0x80000000u | MSCCLX_AUX), XF = MSCCLX_AUX, XS = MSCCLX_AUX_ST, XN = MSCCLX_AUX_ST_FINAL;
+  u32x4 lo[U], hi[U], x[U], y[U];
+  MSCCLX_CHAIN_CLOCK(prof_ld);
+#ifdef MSCCLX_PROFILE
+  prof_acc[3] += prof_ld - (prof_mark > prof_floor ? prof_mark : prof_floor);
+#endif
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t i = i0 + 64u * (uint32_t)u;
+    lo[u] = hi[u] = x[u] = y[u] = u32x4{0, 0, 0, 0};
+    if (rcv) {
+      lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
+      hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
+    } else if (from_src) {
+      x[u] = A::template ld<XL>(rsrc, (int)(i * 16));
+    }
+  }
+  if (has_b) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) y[u] = A::template ld<XL>(rdst, (int)((i0 + 64u * (uint32_t)u) * 16));
+  }
+  u64 gate_seen = gate ? load_counter(gate) : ~0ull;
+  bool lost = false;
+  if (rcv) {
+    unsigned spins = 0;
+    u64 since = 0;
+    for (;;) {
+      bool ok[U], all = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        ok[u] = i0 + 64u * (uint32_t)u >= n || ll_valid(lo[u], hi[u], fin);
+        all = all && ok[u];
+      }
+      if (all) break;
+      MSCCLX_POLL_PAUSE();
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (!ok[u]) {
+          const uint32_t i = i0 + 64u * (uint32_t)u;
+          lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
+          hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
+        }
+      if ((++spins & 0x3fu) == 0) {
+        since = chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 1);
+        if (since == ~0ull) { lost = true; break; }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = u32x4{lo[u].x, lo[u].z, hi[u].x, hi[u].z};
+  }
+  MSCCLX_CHAIN_CLOCK(prof_got);
+  MSCCLX_CHAIN_ADD(1, prof_ld, prof_got);
+  if (has_b) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = R::combine(y[u], x[u]);
+  }
+  if (gate) {  // the slot may still be being read
+    unsigned spins = 0;
+    u64 since = 0;
+    while (gate_seen < gate_target && !lost) {
+      MSCCLX_POLL_PAUSE();
+      gate_seen = load_counter(gate);
+      if ((++spins & 0x3fu) == 0) {
+        since = chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 2);
+        if (since == ~0ull) lost = true;
+      }
+    }
+  }
+  if (__builtin_amdgcn_ballot_w64(lost) != 0) return false;  // (the same decision in all lanes)
+  if (snd) {  // the forwarded lines first: the next rank is waiting for them
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + 64u * (uint32_t)u;
+      A::template st<XF>(rout, (int)(i * kLLUnitBytes), u32x4{x[u].x, fout, x[u].y, fout});
+      A::template st<XF>(rout, (int)(i * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
+    }
+  }
+  if (to_local) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + 64u * (uint32_t)u;
+      if (nt) A::template st<XN>(rdst, (int)(i * 16), x[u]);
+      else A::template st<XS>(rdst, (int)(i * 16), x[u]);
+    }
+  }
+#ifdef MSCCLX_PROFILE
+  prof_mark = __builtin_amdgcn_s_memtime();
+  prof_acc[2] += prof_mark - prof_got;
+#endif
+  return true;
+}
+
+// The step table seen through the constant address space: nothing on the device writes it, and a
+// step's entry then arrives in scalar registers with three scalar loads (a vector load would bring it
+// to every lane, to be carried back to scalar registers word by word).
+typedef const __attribute__((address_space(4))) DevOp* ConstOps;
+__device__ __forceinline__ DevOp fetch_step(ConstOps e) {  // (field by field: a struct cannot be copied out of another address space as a whole)
+  DevOp r;
+  r.word = e->word; r.dep_tb = e->dep_tb; r.dep_step = e->dep_step; r.dep_nops = e->dep_nops;
+  r.extra = e->extra; r.steps = e->steps;
+  r.src_addr = e->src_addr; r.dst_addr = e->dst_addr; r.in_addr = e->in_addr;
+  return r;
+}
+
+// (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for a dependency, 1 from the first
+// load of a message's lines until they are all there, 2 from there until the step's stores are issued,
+// 3 from there to the next step's first load, 4 in all)
+template <class R>
+__device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch, int ctx, u64* prof_acc = nullptr) {
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
-  u64* const abort_word = p.sync_cur;
   Hosted h;
   {
     Context first;
     init_context<true, R::kElemBytes, true>(h, first, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
     if (!first.active) return;
   }
-  const DevOp* const ops = p.ops + uniform(h.op_begin);
+  const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
   const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
   unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
   unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
@@ -784,17 +913,22 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   u64* const my_flag = p.sync_cur + uniform(h.my_flag);
   const uint32_t piece = p.piece_units, depth = (uint32_t)p.depth, nops = (uint32_t)uniform(h.nops), npasses = uniform(h.npasses);
   const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
-  const int my_tb = uniform(h.tb), my_slice = uniform(h.slice);
+  const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
   uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
-  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice));
-  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, my_slice) * 16;
-  DevOp op = uniform(ops[0]);
+  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice));
+  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice) * 16;
+  DevOp op = fetch_step(ops);
+  MSCCLX_CHAIN_CLOCK(prof_begin);
+  u64 prof_mark = 0;  // profiling builds: when the previous step's stores were issued
+#ifdef MSCCLX_PROFILE
+  prof_mark = prof_begin;
+#endif
   for (;;) {
-    const DevOp after = ops[step + 1 == nops ? 0 : step + 1];  // (a table nobody writes: it arrives while the wave waits)
+    const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+    MSCCLX_CHAIN_CLOCK(prof_dep0);
     const int t = (int)(op.word & 15u);
     const uint32_t cnt = op.word >> kOpCntShift;
     const uint32_t n = left < piece ? left : piece;
-    bool lost = false;
     if (op.dep_tb >= 0) {  // a step of another threadblock of this rank must have finished
       const u64* const flag = flags + (uint32_t)op.dep_tb * kSyncStrideWords;
       const u64 want = (u64)pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1;
@@ -803,77 +937,47 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       while (uniform((uint64_t)load_counter(flag)) < want) {
         MSCCLX_POLL_PAUSE();
         if ((++spins & 0x3fu) == 0) {
-          since = uniform((uint64_t)chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 0));
+          since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, (int)step, watch.slice, (u64)pass, 0));
           if (since == ~0ull) return;
         }
       }
     }
-    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(abort_word)) != 0) return;  // a host's abort request, a lost launch
+    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) return;  // a host's abort request, a lost launch
+    u64 prof_floor = 0;
+#ifdef MSCCLX_PROFILE
+    prof_floor = __builtin_amdgcn_s_memtime();
+    prof_acc[0] += prof_floor - prof_dep0;
+#endif
     const bool rcv = is_recv(t), snd = is_send(t);
+    const bool from_src = t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
     const bool has_b = t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE;
     const bool to_local = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
     const bool nt = (op.word & kOpNtStore) != 0;
     const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
-    const bool gated = snd && sseq >= depth;
+    const u64* gate = (snd && sseq >= depth) ? out_tail : nullptr;  // looked at in the step's first round only
     const u64 gate_target = (u64)sseq + 1 - depth;
-    for (uint32_t row = 0; row < cnt; ++row) {
-      const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_ring + rslot + (u64)row * n * kLLUnitBytes, n * kLLUnitBytes);
-      const __amdgpu_buffer_rsrc_t rout = make_rsrc(out_ring + sslot + (u64)row * n * kLLUnitBytes, n * kLLUnitBytes);
-      const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)(op.src_addr + off + (u64)row * row_stride), n * 16);
-      const __amdgpu_buffer_rsrc_t rdst = make_rsrc((const void*)(op.dst_addr + off + (u64)row * row_stride), n * 16);
-      for (uint32_t base = 0; base < n; base += 128) {  // two units per lane at a time
-        const uint32_t i0 = base + lane, i1 = i0 + 64;
-        u32x4 a0 = {}, a1 = {}, b0 = {}, b1 = {}, x0 = {}, x1 = {}, y0 = {}, y1 = {};
-        if (rcv) {
-          a0 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes)); a1 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes + 16));
-          b0 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes)); b1 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes + 16));
-        } else if (t != MSCCLX_OP_NOP) {
-          x0 = A::template ld<XL>(rsrc, (int)(i0 * 16)); x1 = A::template ld<XL>(rsrc, (int)(i1 * 16));
-        }
-        if (has_b) { y0 = A::template ld<XL>(rdst, (int)(i0 * 16)); y1 = A::template ld<XL>(rdst, (int)(i1 * 16)); }
-        const bool first_of_step = row == 0 && base == 0;
-        u64 gate_seen = (gated && first_of_step) ? load_counter(out_tail) : ~0ull;
-        if (rcv) {
-          unsigned spins = 0;
-          u64 since = 0;
-          for (;;) {
-            const bool ok0 = i0 >= n || ll_valid(a0, a1, fin), ok1 = i1 >= n || ll_valid(b0, b1, fin);
-            if (ok0 && ok1) break;
-            MSCCLX_POLL_PAUSE();
-            if (!ok0) { a0 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes)); a1 = A::template ld<XP>(rin, (int)(i0 * kLLUnitBytes + 16)); }
-            if (!ok1) { b0 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes)); b1 = A::template ld<XP>(rin, (int)(i1 * kLLUnitBytes + 16)); }
-            if ((++spins & 0x3fu) == 0) {
-              since = chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 1);
-              if (since == ~0ull) { lost = true; break; }
-            }
-          }
-          x0 = u32x4{a0.x, a0.z, a1.x, a1.z};
-          x1 = u32x4{b0.x, b0.z, b1.x, b1.z};
-        }
-        if (has_b) { x0 = R::combine(y0, x0); x1 = R::combine(y1, x1); }
-        if (gated && first_of_step) {  // the slot may still be being read
-          unsigned spins = 0;
-          u64 since = 0;
-          while (gate_seen < gate_target && !lost) {
-            MSCCLX_POLL_PAUSE();
-            gate_seen = load_counter(out_tail);
-            if ((++spins & 0x3fu) == 0) {
-              since = chain_slow_check(abort_word, p.host_status, p.timeout_ticks, since, my_tb, (int)step, my_slice, (u64)pass, 2);
-              if (since == ~0ull) lost = true;
-            }
+    // the step's rows: packed in the slots, a chunk apart in the rank's buffers
+    const unsigned char* in_row = in_ring + rslot;
+    unsigned char* out_row = out_ring + sslot;
+    u64 src_row = op.src_addr + off, dst_row = op.dst_addr + off;
+    const uint32_t row_line_bytes = n * kLLUnitBytes;
+    if (t != MSCCLX_OP_NOP) {
+      for (uint32_t row = 0; row < cnt; ++row) {
+        const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, row_line_bytes), rout = make_rsrc(out_row, row_line_bytes);
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, n * 16), rdst = make_rsrc((const void*)dst_row, n * 16);
+        if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
+          if (!chain_round<R, 1>(rin, rout, rsrc, rdst, lane, n, rcv, snd, from_src, has_b, to_local, nt, fin, fout, gate, gate_target, watch, (int)step, pass,
+                                 prof_acc, prof_mark, prof_floor)) return;
+          gate = nullptr;
+        } else {
+          for (uint32_t base = 0; base < n; base += 128) {
+            if (!chain_round<R, 2>(rin, rout, rsrc, rdst, base + lane, n, rcv, snd, from_src, has_b, to_local, nt, fin, fout, gate, gate_target, watch, (int)step,
+                                   pass, prof_acc, prof_mark, prof_floor)) return;
+            gate = nullptr;
           }
         }
-        if (__builtin_amdgcn_ballot_w64(lost) != 0) return;  // (the same decision in all lanes)
-        if (snd) {  // the forwarded lines first: the next rank is waiting for them
-          A::template st<XF>(rout, (int)(i0 * kLLUnitBytes), u32x4{x0.x, fout, x0.y, fout});
-          A::template st<XF>(rout, (int)(i0 * kLLUnitBytes + 16), u32x4{x0.z, fout, x0.w, fout});
-          A::template st<XF>(rout, (int)(i1 * kLLUnitBytes), u32x4{x1.x, fout, x1.y, fout});
-          A::template st<XF>(rout, (int)(i1 * kLLUnitBytes + 16), u32x4{x1.z, fout, x1.w, fout});
-        }
-        if (to_local) {
-          if (nt) { A::template st<XN>(rdst, (int)(i0 * 16), x0); A::template st<XN>(rdst, (int)(i1 * 16), x1); }
-          else { A::template st<XS>(rdst, (int)(i0 * 16), x0); A::template st<XS>(rdst, (int)(i1 * 16), x1); }
-        }
+        in_row += row_line_bytes; out_row += row_line_bytes;
+        src_row += row_stride; dst_row += row_stride;
       }
     }
     if (rcv) {
@@ -898,8 +1002,11 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       off += (u64)piece * 16;
       if (++pass >= npasses) break;
     }
-    op = uniform(after);
+    op = after;
   }
+#ifdef MSCCLX_PROFILE
+  prof_acc[4] = __builtin_amdgcn_s_memtime() - prof_begin;
+#endif
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -949,7 +1056,14 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
   if (LL && hosted == 1 && blockDim.x == 64) {
+#ifdef MSCCLX_PROFILE
+    u64 chain_acc[5] = {0, 0, 0, 0, 0};
+    if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin, chain_acc);
+    prof_fin = chain_acc[0]; prof_wait = chain_acc[1]; prof_move = chain_acc[2]; prof_ack = chain_acc[3];
+    if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
+#else
     if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin);
+#endif
   } else {
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
