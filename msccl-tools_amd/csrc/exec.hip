@@ -82,15 +82,6 @@ void destroy_device_state(DeviceState* d) {
   delete d;
 }
 
-// A nop that nobody depends on and that is not its threadblock's last step can be folded into the
-// step after it (build_image).
-static bool has_foldable_nops(const mscclx_plan& plan) {
-  for (const Tb& tb : plan.tbs)
-    for (int o = tb.op_begin; o + 1 < tb.op_end; ++o)
-      if (plan.ops[o].type == MSCCLX_OP_NOP && !plan.ops[o].hasdep) return true;
-  return false;
-}
-
 static int query_capacity(kernel_fn k, int* num_cus, int capacity[kThreadChoices]) {
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
@@ -423,8 +414,15 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     for (int i = 0; i < kThreadChoices; ++i) capacity[i] = cfg.max_workgroups;
   } else {
     const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
-    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, vec && !ll && has_foldable_nops(*plan)), &num_cus, capacity);
+    const bool fold = vec && !ll && has_foldable_nops(*plan);
+    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, fold), &num_cus, capacity);
     if (rc) return rc;
+    if (cfg.protocol == MSCCLX_PROTO_AUTO && vec && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
+      int other[kThreadChoices];
+      rc = query_capacity(pick_kernel(dtype, redop, true, true, false), &num_cus, other);
+      if (rc) return rc;
+      for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
+    }
   }
   Geometry g;
   const uint64_t fifo_budget = 4ull << 30;  // FIFO slots of staged messages; larger pieces are split into passes

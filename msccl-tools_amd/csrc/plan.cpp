@@ -455,6 +455,13 @@ static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t sli
   return largest ? (double)total / (double)wgs / (double)largest : 1.0;
 }
 
+bool has_foldable_nops(const mscclx_plan& plan) {
+  for (const Tb& tb : plan.tbs)
+    for (int o = tb.op_begin; o + 1 < tb.op_end; ++o)
+      if (plan.ops[o].type == MSCCLX_OP_NOP && !plan.ops[o].hasdep) return true;
+  return false;
+}
+
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);
@@ -493,6 +500,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (ntbs > host_limit)
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
   int64_t slices = cfg.slices;
+  bool lines = cfg.protocol == MSCCLX_PROTO_LL;  // flag-in-data lines instead of counters
   if (!slices) {
     const int64_t finest = (int64_t)(chunk_bytes / (32 * 1024));       // most slices of at least 32 KiB
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;  // fewest slices that give every compute unit a context or two
@@ -566,6 +574,27 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // (64-rank ring, 2 KiB chunks: 251 us with 8 slices of 256 bytes, 264 us with 4 of 512).
       // Only where that still is a workgroup or two per compute unit: more of them cost more than the hand-offs save.
       if (slices < 8 && chunk_bytes / 8 >= 128 && 8 * ntbs <= 2 * (int64_t)num_cus) slices = 8;
+      // Flag-in-data lines by themselves, where they win: a chain of hand-offs (8 or more deep) whose
+      // pieces can be cut down to 1 KiB -- one unit per lane of a one-wave workgroup, the shape the
+      // kernel's chain loop is written for -- with at most two such workgroups per compute unit, one
+      // context each.  There a hop takes 1.55 us against 2.1 us with counters (64-rank ring on
+      // 256 KiB per rank 198 against 262 us, 8-rank ring on 8 to 512 KiB per rank 30 against 35-38 us);
+      // with bigger pieces or more workgroups the doubled slot traffic and the staging of every
+      // message cost more than the hand-off saves (8-rank ring on 1 MiB: 38 us either way; on 2 MiB
+      // 59 against 40 us).  Programs whose nops can be folded keep the counters: folding, and chains
+      // of local reduces done as one step, are worth more there.  Only when every knob is automatic.
+      if (cfg.protocol == MSCCLX_PROTO_AUTO && g.vector_path && !cfg.staging && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups &&
+          depth_of_dataflow >= 8 && !has_foldable_nops(plan)) {
+        int64_t s = slices;
+        while (chunk_bytes / (uint64_t)s > 1024 && s * 2 * ntbs <= 2 * (int64_t)num_cus && (uint64_t)(s * 2) <= g.chunk_units) s *= 2;
+        int64_t most_msgs = 0;
+        for (const Conn& c : plan.conns) most_msgs = std::max<int64_t>(most_msgs, c.nmsg);
+        if (chunk_bytes / (uint64_t)s <= 1024 && s * ntbs <= 2 * (int64_t)num_cus && s * ntbs <= capacity_by_threads[thread_index(64)] &&
+            most_msgs < (1 << 22) - 1) {
+          slices = s;
+          lines = true;
+        }
+      }
     }
   }
   slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
@@ -593,10 +622,9 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   }
   piece_units = std::min(piece_units, longest_slice);
   // protocol: flag-in-data lines pay twice the slot traffic and stage every message to take the
-  // counter round trip out of a hand-off.  Chosen only on request: measured on MI355X a hop is bound
-  // as much by the receiving workgroup's own step-to-step time as by the hand-off, and reading
-  // payloads in place (which LL gives up) wins at every piece size tried.
-  g.ll = cfg.protocol == MSCCLX_PROTO_LL ? 1 : 0;
+  // counter round trip out of a hand-off.  On request, or where the rule for small chunks above
+  // found them faster; everywhere else reading payloads in place (which LL gives up) wins.
+  g.ll = lines ? 1 : 0;
   if (g.ll) g.staging = 1;
   const uint64_t fifo_unit_bytes = (uint64_t)g.unit_bytes * (g.ll ? 2 : 1);
   uint64_t slot_chunks = 0;  // FIFO units per slice per unit of piece

@@ -195,6 +195,9 @@ int dtype_size(int dtype);
 // Host dry run of one pass; returns MSCCLX_OK or MSCCLX_ERR_DEADLOCK (error text names a blocked step).
 int simulate(const mscclx_plan& plan, int depth);
 // Pure geometry decision (no HIP): max_wgs = resident workgroup capacity per thread count.
+// A nop that nobody depends on and that is not its threadblock's last step can be folded into the
+// step after it when the device tables are built; programs with such nops run on kernels of their own.
+bool has_foldable_nops(const mscclx_plan& plan);
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out);
 void destroy_device_state(DeviceState* d);

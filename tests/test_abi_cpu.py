@@ -7,6 +7,7 @@ import re
 import numpy as np
 import pytest
 
+import golden_util
 import ir_samples
 from msccl.executor import (EXPORTED_SYMBOLS, IRError, MscclxError, Plan, parse_algo_xml)
 from msccl.executor import binding
@@ -171,11 +172,20 @@ def test_zero_copy_analysis(mscclx_lib):
 
 
 def test_protocol_choice(mscclx_lib):
-    """Flag-in-data lines are used on request only, double the slot bytes and stage every message."""
+    """Flag-in-data lines double the slot bytes and stage every message.  They are used on request, and
+    by themselves only for a deep chain of hand-offs whose pieces can be cut to 1 KiB on at most two
+    one-wave workgroups per compute unit, with every other knob automatic."""
     p = Plan(parse_algo_xml(ir_samples.ring_allreduce_xml(8)))
-    for chunk in (8 << 20, 64 << 10):
+    for chunk in (8 << 20, 256 << 10):
         auto = p.configure(chunk, "float32", max_workgroups=2048)
         assert auto.protocol == binding.PROTOCOL_CODES["simple"] and auto.zero_copy_messages > 0
+    auto = p.configure(64 << 10, "float32", max_workgroups=2048)
+    assert auto.protocol == binding.PROTOCOL_CODES["ll"] and (auto.slices, auto.piece_bytes, auto.threads, auto.max_hosted) == (64, 1024, 64, 1)
+    for knobs in (dict(threads=64), dict(piece_bytes=1024), dict(workgroups=512), dict(staging=1), dict(protocol="simple")):
+        assert p.configure(64 << 10, "float32", max_workgroups=2048, **knobs).protocol == binding.PROTOCOL_CODES["simple"], knobs
+    # nops that can be folded into the next step are worth more than the lines: such programs keep the counters
+    allpairs = Plan(parse_algo_xml(golden_util.load("allreduce_a100_allpairs_8r")))
+    assert allpairs.configure(1024, "float32", max_workgroups=2048).protocol == binding.PROTOCOL_CODES["simple"]
     small = p.configure(64 << 10, "float32", max_workgroups=2048, protocol="ll")
     assert small.protocol == binding.PROTOCOL_CODES["ll"]
     assert small.zero_copy_messages == 0 and small.staged_messages == 8 * 14
@@ -202,12 +212,13 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
         "c2": (512, 512, 64, 131072, 1, 4),     # a ring is always busy: 4 contexts per workgroup, one pass
         "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
-        "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed
+        "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed, flag-in-data lines
         "c5_chain": (1024, 128, 16, 16384, 1, 1),
     }
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
+        assert i.protocol == binding.PROTOCOL_CODES["ll" if key == "c5" else "simple"], key
 
 
 def test_geometry_between_the_benchmark_sizes(mscclx_lib):
