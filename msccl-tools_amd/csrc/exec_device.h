@@ -1013,6 +1013,141 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
 #endif
 }
 
+// One round of a step of run_chain_counters: units i0, i0 + 64, ... (U per lane) of one row of n
+// units; out-of-range lanes load zeros and store nothing (the descriptors bound every access).
+template <class R, int U>
+__device__ __forceinline__ void chain_copy_round(const __amdgpu_buffer_rsrc_t ra, const __amdgpu_buffer_rsrc_t rb, const __amdgpu_buffer_rsrc_t rlocal,
+                                                 const __amdgpu_buffer_rsrc_t rslot, const uint32_t i0, const bool has_b, const bool to_local,
+                                                 const bool to_slot, const bool nt) {
+  typedef Access<16> A;
+  constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, XN = MSCCLX_AUX_ST_FINAL;
+  u32x4 x[U], y[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) x[u] = A::template ld<XL>(ra, (int)((i0 + 64u * (uint32_t)u) * 16));
+  if (has_b) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) y[u] = A::template ld<XL>(rb, (int)((i0 + 64u * (uint32_t)u) * 16));
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = R::combine(y[u], x[u]);
+  }
+  if (to_slot) {  // the forwarded copy first: the next rank is waiting for it
+#pragma unroll
+    for (int u = 0; u < U; ++u) A::template st<XS>(rslot, (int)((i0 + 64u * (uint32_t)u) * 16), x[u]);
+  }
+  if (to_local) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (nt) A::template st<XN>(rlocal, (int)((i0 + 64u * (uint32_t)u) * 16), x[u]);
+      else A::template st<XS>(rlocal, (int)((i0 + 64u * (uint32_t)u) * 16), x[u]);
+    }
+  }
+}
+
+// The counter protocol, one context on a workgroup of one wave: the same lean loop as run_chain for
+// programs whose messages are announced by counters and mostly read where the sender keeps them.  A
+// step waits for its (up to three) counters with one round of loads, moves its rows, waits until its
+// stores are acknowledged and announces them.  Steps, waits and counters are those of the hosted
+// path, so a workgroup running this loop can talk to workgroups running that one.
+template <class R>
+__device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ctx) {
+  const uint32_t lane = threadIdx.x;
+  const bool writer = lane == 0;
+  Hosted h;
+  {
+    Context first;
+    init_context<true, R::kElemBytes, false>(h, first, p, 0, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+    if (!first.active) return;
+  }
+  const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
+  const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
+  unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
+  const u64* const flags = p.sync_cur + uniform(h.flags);
+  const u64* const in_head = p.sync_cur + uniform(h.head_in);   // messages the sender of the incoming connection has announced
+  u64* const in_tail = p.sync_cur + uniform(h.tail_out);        // messages this context has consumed of them
+  u64* const out_head = p.sync_cur + uniform(h.head_out);       // messages this context has announced on the outgoing connection
+  const u64* const out_tail = p.sync_cur + uniform(h.tail_in);  // messages its receiver has consumed
+  u64* const my_flag = p.sync_cur + uniform(h.my_flag);
+  const uint32_t piece = p.piece_units, depth = (uint32_t)p.depth, nops = (uint32_t)uniform(h.nops), npasses = uniform(h.npasses);
+  const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
+  const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
+  uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
+  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice));
+  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice) * 16;
+  DevOp op = fetch_step(ops);
+  for (;;) {
+    const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+    const uint32_t t = op.word & 15u;
+    const uint32_t cnt = op.word >> kOpCntShift;
+    const uint32_t n = left < piece ? left : piece;
+    const uint32_t rcv_bit = (0x7cu >> t) & 1u, snd_bit = (0x5au >> t) & 1u;  // r rcs rrs rrc rrcs / s rcs rrs rrcs
+    static_assert(MSCCLX_OP_SEND == 1 && MSCCLX_OP_RECV == 2 && MSCCLX_OP_RCS == 3 && MSCCLX_OP_RRS == 4 && MSCCLX_OP_RRC == 5 && MSCCLX_OP_RRCS == 6,
+                  "the two masks above list the receiving and the sending step types by their codes");
+    {  // what the step waits for: a step of another threadblock, the incoming message, a free outgoing slot -- one round of loads for all
+      const u64* const w0 = op.dep_tb >= 0 ? flags + (uint32_t)op.dep_tb * kSyncStrideWords : nullptr;
+      const u64 t0 = (u64)pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1;
+      const u64* const w1 = rcv_bit ? in_head : nullptr;
+      const u64 t1 = (u64)rseq + 1;
+      const u64* const w2 = (snd_bit && sseq >= depth) ? out_tail : nullptr;
+      const u64 t2 = (u64)sseq + 1 - depth;
+      unsigned spins = 0;
+      u64 since = 0;
+      for (;;) {
+        const u64 v0 = w0 ? load_counter(w0) : 0, v1 = w1 ? load_counter(w1) : 0, v2 = w2 ? load_counter(w2) : 0;
+        const bool ok0 = !w0 || uniform((uint64_t)v0) >= t0, ok1 = !w1 || uniform((uint64_t)v1) >= t1, ok2 = !w2 || uniform((uint64_t)v2) >= t2;
+        if (ok0 && ok1 && ok2) break;
+        MSCCLX_POLL_PAUSE();
+        if ((++spins & 0x3fu) == 0) {
+          since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, (int)step, watch.slice, (u64)pass,
+                                                     !ok0 ? 0 : !ok1 ? 1 : 2));
+          if (since == ~0ull) return;
+        }
+      }
+    }
+    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) return;  // a host's abort request, a lost launch
+    const bool rcv = rcv_bit != 0;
+    const bool has_b = t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE;
+    const bool to_local = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
+    const bool to_slot = snd_bit && (op.word & kOpOutStaged);  // else the receiver reads the payload where this rank keeps it
+    const bool nt = (op.word & kOpNtStore) != 0;
+    if (to_local || to_slot) {
+      // the step's rows: packed in the slots, a chunk apart in rank buffers (the sender's too, when the payload is read in place)
+      const bool in_place = rcv && (op.word & kOpInPlace);
+      u64 a_row = rcv ? (in_place ? op.in_addr + off : (u64)(in_ring + rslot)) : op.src_addr + off;
+      const u64 a_stride = (rcv && !in_place) ? (u64)n * 16 : row_stride;
+      u64 local_row = op.dst_addr + off, slot_row = (u64)(out_ring + sslot);
+      const uint32_t row_bytes = n * 16;
+      for (uint32_t row = 0; row < cnt; ++row) {
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc((const void*)a_row, row_bytes), rlocal = make_rsrc((const void*)local_row, row_bytes);
+        const __amdgpu_buffer_rsrc_t rslot_out = make_rsrc((const void*)slot_row, row_bytes);
+        if (n <= 64) chain_copy_round<R, 1>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
+        else if (n <= 128) chain_copy_round<R, 2>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
+        else
+          for (uint32_t base = 0; base < n; base += 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
+        a_row += a_stride; local_row += row_stride; slot_row += row_bytes;
+      }
+      __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged: the counters below may announce them
+    }
+    if (snd_bit && writer) publish(out_head, (u64)sseq + 1);
+    if (rcv_bit && writer) publish(in_tail, (u64)rseq + 1);
+    rseq += rcv_bit;
+    rslot += in_slot_bytes & (0u - rcv_bit);
+    rslot = rslot == in_wrap ? 0u : rslot;
+    sseq += snd_bit;
+    sslot += out_slot_bytes & (0u - snd_bit);
+    sslot = sslot == out_wrap ? 0u : sslot;
+    ++count;  // = pass * steps of the IR + IR step + 1 (programs with folded steps do not come here)
+    if ((op.word & kOpHasdep) && writer) publish(my_flag, (u64)count);
+    if (++step == nops) {
+      step = 0;
+      left -= n;
+      off += (u64)piece * 16;
+      if (++pass >= npasses) break;
+    }
+    op = after;
+  }
+}
+
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
 // active context waits for (one round of loads covers all of them), finishes steps that move no data
 // on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
@@ -1068,6 +1203,8 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #else
     if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin);
 #endif
+  } else if (!LL && !FOLD && VEC && hosted == 1 && blockDim.x == 64) {
+    if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin);
   } else {
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
