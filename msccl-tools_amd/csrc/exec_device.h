@@ -822,6 +822,23 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
     u64 since = 0;
     while (!all_there()) {
       MSCCLX_POLL_PAUSE();
+      if (spins >= 2) {
+        // A long wait (the start of a pipeline, a rank far down a chain): asking for every line again
+        // and again costs memory traffic that the ranks at work pay for -- 4096 waiting waves ask for
+        // 16 MiB a round.  Watch the round's last line alone until it is there, then ask for all.
+        const uint32_t round_end = i0 - threadIdx.x + 64u * (uint32_t)U;
+        const int watched = (int)(((round_end < n ? round_end : n) - 1u) * kLLUnitBytes + 16u);
+        for (;;) {
+          const u32x4 w = A::template ld<XP>(rin, watched);
+          if (uniform(w.y) == fin && uniform(w.w) == fin) break;
+          MSCCLX_POLL_PAUSE();
+          if ((++spins & 0x3fu) == 0) {
+            since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 1));
+            if (since == ~0ull) { lost = true; break; }
+          }
+        }
+        if (lost) break;
+      }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t i = i0 + 64u * (uint32_t)u;
@@ -1122,8 +1139,9 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
         const __amdgpu_buffer_rsrc_t rslot_out = make_rsrc((const void*)slot_row, row_bytes);
         if (n <= 64) chain_copy_round<R, 1>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else if (n <= 128) chain_copy_round<R, 2>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
-        else
-          for (uint32_t base = 0; base < n; base += 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
+        else if (n <= 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
+        else  // (eight loads in flight per lane and operand, as the workgroup-wide mover has)
+          for (uint32_t base = 0; base < n; base += 512) chain_copy_round<R, 8>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
         a_row += a_stride; local_row += row_stride; slot_row += row_bytes;
       }
       __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged: the counters below may announce them

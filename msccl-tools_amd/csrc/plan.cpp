@@ -504,7 +504,17 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (!slices) {
     const int64_t finest = (int64_t)(chunk_bytes / (32 * 1024));       // most slices of at least 32 KiB
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;  // fewest slices that give every compute unit a context or two
-    if (finest >= 2 && finest >= to_fill) {
+    // A long chain of hand-offs with few bytes on each (a chain all-reduce passes one buffer through
+    // every rank) is bound by latency however big its chunks: about 2 us a hop against the bytes at
+    // 5 TB/s.  It goes the way of the small chunks below.
+    bool chain_bound = false;
+    {
+      uint64_t moved = 0;  // in chunks
+      for (const Tb& tb : plan.tbs) moved += tb_work(plan, tb, cfg.staging != 0 || cfg.protocol == MSCCLX_PROTO_LL);
+      const double data_us = (double)moved * (double)chunk_bytes / 5e6, chain_us = 2.0 * (double)g.dataflow_depth;
+      chain_bound = chain_us > 2.0 * data_us;
+    }
+    if (finest >= 2 && finest >= to_fill && !chain_bound) {
       // Slices of 32 KiB or more can give every compute unit a context.  Measured on MI355X (8 to 1920
       // threadblocks, 128 KiB to 64 MiB chunks), what matters is (1) that the contexts spread EVENLY
       // over the resident workgroups -- 7.5 contexts per workgroup on average means some host 8, and
@@ -549,8 +559,9 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // -- a fixed cost per workgroup launched, and one hand-off plus one small move for every step
       // on the longest chain of the program's dataflow.  More slices shrink the pieces but add
       // workgroups; the minimum is at slices = sqrt(b/a * depth * chunk / threadblocks).  With
-      // b/a = 6.25 per KiB (fitted on MI355X, workgroups of one wave) an 8-rank ring on 1 MiB comes
-      // out at 39 slices and a 64-rank ring on 256 KiB at 7; 32 and 8 measured best.  Threadblocks that
+      // b/a = 12.5 per KiB (fitted on MI355X, workgroups of one wave running the chain loops) an
+      // 8-rank ring on 1 MiB comes out at 53 slices and a 64-rank ring on 256 KiB at 10; 64 and 8
+      // measured best.  Threadblocks that
       // mostly wait for each other cost less than the fixed cost each: with waiting_ratio r the
       // minimum moves to sqrt(r) times as many slices (two-level all-reduce, r = 9.4, 16 KiB chunks:
       // 4 slices 78 us, 1 slice 86 us).
@@ -558,7 +569,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // r times that with pieces of 4 KiB or more.
       int32_t depth_of_dataflow = 1;
       const double ratio = waiting_ratio(plan, &depth_of_dataflow);
-      const double best = std::sqrt(ratio * 6.25 * (double)depth_of_dataflow * ((double)chunk_bytes / 1024.0) / (double)ntbs);
+      const double best = std::sqrt(ratio * 12.5 * (double)depth_of_dataflow * ((double)chunk_bytes / 1024.0) / (double)ntbs);
       const int64_t fill = (int64_t)std::ceil((double)to_fill * ratio);
       const int64_t most = std::max<int64_t>(1, std::max(std::min<int64_t>(std::max(finest, to_fill), (int64_t)(chunk_bytes / 512)),
                                                          std::min<int64_t>(std::max(finest, fill), (int64_t)(chunk_bytes / 4096))));

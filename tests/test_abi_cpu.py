@@ -208,12 +208,12 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
     MI355X: (workgroups, threads, slices, piece bytes, passes, most contexts on a workgroup)."""
     from msccl.executor.workloads import WORKLOADS
     want = {
-        "c1": (256, 64, 32, 4096, 1, 1),        # latency bound: few workgroups of one wave, 4 KiB pieces
+        "c1": (512, 64, 64, 2048, 1, 1),        # latency bound: two workgroups of one wave per compute unit, 2 KiB pieces
         "c2": (512, 512, 64, 131072, 1, 4),     # a ring is always busy: 4 contexts per workgroup, one pass
         "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
         "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed, flag-in-data lines
-        "c5_chain": (1024, 128, 16, 16384, 1, 1),
+        "c5_chain": (4096, 64, 64, 4096, 1, 1),  # one buffer through 64 ranks: latency bound however big the chunk, most contexts wait
     }
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
