@@ -111,7 +111,7 @@ def fold_orders(key):
     return None
 
 
-def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_costs=False):
+def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_costs=False, knobs=None):
     import torch
     from msccl.executor import Executor, collective_buffers, parse_algo_xml
     from msccl.executor.workloads import WORKLOADS, torch_input
@@ -124,7 +124,7 @@ def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_
     t0 = time.perf_counter()
     ex = Executor(tables, device=device)
     host["plan_create"] = time.perf_counter() - t0
-    info = ex.setup(w.chunk_bytes, w.dtype)
+    info = ex.setup(w.chunk_bytes, w.dtype, **(knobs or {}))
     host["configure"] = ex.host_seconds["configure"]
     x = [torch_input(w, r, device) for r in range(w.ranks)]
     ins, outs, res = collective_buffers(ex.tables, w.chunk_bytes, w.dtype, device=device, inputs=x)
@@ -248,6 +248,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
+    ap.add_argument("--knobs", default="", metavar="K=V,...", help="geometry of the headline workload instead of the automatic one, e.g. "
+                    "threads=1024,workgroups=256,piece_bytes=131072 (for experiments; the line then carries them in config.knobs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy baseline")
     ap.add_argument("--sweep", metavar="LO:HI", help="instead of the benchmark line: time the chosen algorithm on LO, 2*LO, ... HI bytes per "
                     "rank (same inputs, same timing; results not verified) and print one JSON line holding the list")
@@ -286,17 +288,21 @@ def main():
         print(json.dumps({"sweep": args.config, "workload": r["workload"].split(";")[0], "dtype": r["dtype"], "steps": args.steps, "rows": rows}))
         return
     traffic = measured_traffic()
-    head = run_workload(args.config, args.steps, args.warmup, host_costs=True)
+    knobs = {}
+    for kv in filter(None, args.knobs.split(",")):
+        k, _, v = kv.partition("=")
+        knobs[k] = v if k == "protocol" else int(v)
+    head = run_workload(args.config, args.steps, args.warmup, host_costs=True, knobs=knobs)
     line = {
         "metric": "algbw_GBps", "value": head["algbw_GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"int32": "i32", "uint8": "u8", "float32": "f32", "bfloat16": "bf16", "float16": "f16"}[head["dtype"]],
-        "data": "synthetic", "config": {"workload": head["workload"], "virtual_ranks": head["ranks"], **head["geometry"]},
+        "data": "synthetic", "config": {"workload": head["workload"], "virtual_ranks": head["ranks"], **head["geometry"], **({"knobs": knobs} if knobs else {})},
         "busbw_GBps": head["busbw_GBps"], "hbm_fraction": head["hbm_fraction"], "verified": head["verified"],
         "timing": "every timed launch starts from restored inputs (restore untimed) and is bracketed by a device synchronisation on both sides"
                   if head["inputs_restored_before_every_launch"] else "every timed launch is bracketed by a device synchronisation on both sides",
         "roofline": {"bound": "hbm", "achieved": round(head["algorithmic_bytes"] / (head["kernel_ms"] * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": head["roofline_frac_kernel"], "traffic": traffic.get(args.config),
+                     "unit": "GB/s", "frac": head["roofline_frac_kernel"], "traffic": None if knobs else traffic.get(args.config),
                      "kernel": "exec_kernel", "algorithmic_bytes_per_launch": head["algorithmic_bytes"], "kernel_ms": round(head["kernel_ms"], 5),
                      "kernel_ms_min": round(head["kernel_ms_min"], 5), "kernel_ms_max": round(head["kernel_ms_max"], 5),
                      "kernel_ms_queued": round(head["kernel_ms_queued"], 5), "note": ROOFLINE_NOTE},
