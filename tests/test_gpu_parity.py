@@ -101,7 +101,7 @@ def test_ring_allreduce_dtypes(dtype, protocol):
 
 @pytest.mark.parametrize("protocol", PROTOCOLS)
 @pytest.mark.parametrize("redop", ["prod", "max", "min"])
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "int32"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16", "int32"])
 def test_ring_allreduce_redops(dtype, redop, protocol):
     got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(4), 2048, dtype, redop=redop, protocol=protocol)
     assert_same(got, want)
