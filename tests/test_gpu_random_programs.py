@@ -1,0 +1,76 @@
+"""Random MSCCLang programs on the device: whatever well-formed MSCCL-IR the compiler emits for a random
+sequence of copies and reduces (tests/random_programs.py) -- fused step types in combinations no
+shipped program has, scratch buffers, chains of dependencies, two instances -- must leave in every
+buffer of every rank, scratch included, the bits the interpreter leaves, however the messages cross
+the connections."""
+import numpy as np
+import pytest
+import torch
+
+import random_programs as rp
+from msccl.executor import Executor, MscclxError, Plan, binding, parse_algo_xml
+from oracle import ir_interp as oi
+
+pytestmark = pytest.mark.gpu
+
+# fused (one seed in seven is refused as malformed and skipped), every seed below 400 whose program has an `rrs`, and unfused
+CASES = [(seed, True) for seed in range(48)] + [(seed, True) for seed in (216, 270, 319)] + [(seed, False) for seed in range(12)]
+MODES = {"in-place": dict(protocol="simple", staging=0), "staged": dict(protocol="simple", staging=1), "ll": dict(protocol="ll")}
+ELEMS = 1000  # 4000-byte chunks: the 16-byte vector path
+
+
+def races(algo, elems=8):
+    """Does what the program leaves behind depend on how its threadblocks interleave?  (Random
+    interleavings of the interpreter, with unbounded and with two-deep connections.)  Such IR has no
+    result to compare a device with."""
+    rng = np.random.default_rng(7)
+    init = [{b: rng.standard_normal(n * elems).astype(np.float32) for b, n in (("i", g.i_chunks), ("o", g.o_chunks), ("s", g.s_chunks))} for g in algo.gpus]
+    outcomes = set()
+    for schedule, seed, depth in [("fifo", 0, None)] + [("random", k, None) for k in range(12)] + [("random", k, 2) for k in range(6)]:
+        bufs = [{b: v.copy() for b, v in d.items()} for d in init]
+        try:
+            oi.Interpreter(algo, schedule, seed, depth).run(bufs, elems, "float32")
+        except oi.Deadlock:
+            continue  # (two-deep connections may be too shallow for the program: the device picks its own depth)
+        outcomes.add(b"".join(bufs[r][b].tobytes() for r in range(len(bufs)) for b in "ios"))
+    return len(outcomes) > 1
+
+
+@pytest.mark.parametrize("seed,fusion", CASES)
+def test_random_program_vs_interpreter(seed, fusion):
+    xml = rp.random_program(seed, fusion)[0]
+    tables = parse_algo_xml(xml)
+    try:
+        Plan(tables)
+    except MscclxError as e:
+        assert e.code == binding.ERR_BAD_IR
+        pytest.skip("msccl-tools' fusion leaves this program with unmatched sends and receives")
+    algo = oi.parse_xml(xml)
+    rng = np.random.default_rng(2000 + seed)
+    init = [{b: rng.standard_normal(n * ELEMS).astype(np.float32) for b, n in (("i", g.i_chunks), ("o", g.o_chunks), ("s", g.s_chunks))} for g in algo.gpus]
+    want = [{b: v.copy() for b, v in d.items()} for d in init]
+    try:
+        oi.Interpreter(algo).run(want, ELEMS, "float32")
+    except oi.Deadlock:
+        with pytest.raises(MscclxError) as e:  # the host's dry run must find it too, before anything is launched
+            Executor(tables).setup(ELEMS * 4, "float32")
+        assert e.value.code == binding.ERR_DEADLOCK
+        return
+    if races(algo):
+        pytest.skip("msccl-tools' fusion leaves this program with a race: the interpreter's result depends on the interleaving")
+    for mode, knobs in sorted(MODES.items()):
+        ex = Executor(tables)
+        print(f"case: random program seed={seed} fusion={fusion} mode={mode}", flush=True)
+        ex.setup(ELEMS * 4, "float32", **knobs)
+        ins = [torch.from_numpy(d["i"]).cuda() if d["i"].size else None for d in init]
+        outs = [torch.from_numpy(d["o"]).cuda() if d["o"].size else None for d in init]
+        for r, d in enumerate(init):
+            if d["s"].size:
+                ex._scratch[r].view(torch.float32).copy_(torch.from_numpy(d["s"]))
+        ex.run(ins, outs)
+        torch.cuda.synchronize()
+        for r in range(algo.ngpus):
+            got = {"i": ins[r], "o": outs[r], "s": None if ex._scratch[r] is None else ex._scratch[r].view(torch.float32)}
+            for b in "ios":
+                if want[r][b].size:
+                    assert np.array_equal(got[b].cpu().numpy().view(np.uint32), want[r][b].view(np.uint32)), (seed, fusion, mode, r, b)
