@@ -15,7 +15,11 @@ pytestmark = pytest.mark.gpu
 
 # fused (one seed in seven is refused as malformed and skipped), every seed below 400 whose program has an `rrs`, and unfused
 CASES = [(seed, True) for seed in range(48)] + [(seed, True) for seed in (216, 270, 319)] + [(seed, False) for seed in range(12)]
-MODES = {"in-place": dict(protocol="simple", staging=0), "staged": dict(protocol="simple", staging=1), "ll": dict(protocol="ll")}
+# the automatic geometry (one-wave workgroups with one context each at this size) in the three message modes, and the
+# general path: a few workgroups of several waves that host all the contexts between them
+MODES = {"in-place": dict(protocol="simple", staging=0), "staged": dict(protocol="simple", staging=1), "ll": dict(protocol="ll"),
+         "in-place, hosted": dict(protocol="simple", staging=0, workgroups=6, threads=128, slices=2),
+         "ll, hosted": dict(protocol="ll", workgroups=5, threads=256, slices=2)}
 ELEMS = 1000  # 4000-byte chunks: the 16-byte vector path
 
 
