@@ -28,6 +28,12 @@
 // scheme only relies on 8-byte accesses being indivisible.  Free slots are still granted through the
 // tail counters.
 //
+// Chain loops.  A workgroup of one wave that hosts one context -- the geometry of every latency-bound
+// launch -- leaves the hosting machinery: the wave runs its context with all its lanes in a loop
+// written for that case (run_chain for lines, run_chain_counters for counters), with the bookkeeping
+// in scalar registers.  Same steps, same counters, same slots: such a workgroup talks to workgroups
+// that run the general loop.
+//
 // A workgroup that makes no progress for the watchdog period raises the area's abort word; all
 // other workgroups see it while they poll, and every wave leaves the kernel.
 #pragma once
