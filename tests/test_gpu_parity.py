@@ -25,7 +25,7 @@ def make_inputs(n, elems, dtype, seed):
             out.append(oi.f32_to_bf16_bits(rng.standard_normal(elems, dtype=np.float32)))
         else:
             info = np.iinfo(oi.DTYPES[dtype])
-            out.append(rng.integers(info.min, info.max, elems, dtype=np.int64, endpoint=True).astype(oi.DTYPES[dtype]))
+            out.append(rng.integers(info.min, info.max, elems, dtype=oi.DTYPES[dtype], endpoint=True))
     return out
 
 
@@ -93,7 +93,7 @@ def test_fusion_chain_f32(protocol):
 
 
 @pytest.mark.parametrize("protocol", PROTOCOLS)
-@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "int32", "uint8", "float64", "int64", "int8"])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "int32", "uint8", "float64", "int64", "int8", "uint32", "uint64"])
 def test_ring_allreduce_dtypes(dtype, protocol):
     got, want, _, _ = run_both(ir_samples.ring_allreduce_xml(8), 4096, dtype, protocol=protocol)
     assert_same(got, want)
