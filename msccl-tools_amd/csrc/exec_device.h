@@ -1072,7 +1072,7 @@ __device__ __forceinline__ void chain_copy_round(const __amdgpu_buffer_rsrc_t ra
 // stores are acknowledged and announces them.  Steps, waits and counters are those of the hosted
 // path, so a workgroup running this loop can talk to workgroups running that one.
 template <class R>
-__device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ctx) {
+__device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ctx, u64* prof_acc = nullptr) {
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
   Hosted h;
@@ -1098,7 +1098,11 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice));
   u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice) * 16;
   DevOp op = fetch_step(ops);
+  // (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for the step's counters, 1 moving its rows,
+  // 2 waiting for the stores' acknowledgement, 3 on the bookkeeping between steps, 4 in all)
+  MSCCLX_CHAIN_CLOCK(prof_begin);
   for (;;) {
+    MSCCLX_CHAIN_CLOCK(prof_top);
     const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
     const uint32_t t = op.word & 15u;
     const uint32_t cnt = op.word >> kOpCntShift;
@@ -1128,6 +1132,8 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       }
     }
     if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) return;  // a host's abort request, a lost launch
+    MSCCLX_CHAIN_CLOCK(prof_ready);
+    MSCCLX_CHAIN_ADD(0, prof_top, prof_ready);
     const bool rcv = rcv_bit != 0;
     const bool has_b = t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE;
     const bool to_local = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
@@ -1150,8 +1156,13 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
           for (uint32_t base = 0; base < n; base += 512) chain_copy_round<R, 8>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
         a_row += a_stride; local_row += row_stride; slot_row += row_bytes;
       }
+      MSCCLX_CHAIN_CLOCK(prof_issued);
+      MSCCLX_CHAIN_ADD(1, prof_ready, prof_issued);
       __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged: the counters below may announce them
+      MSCCLX_CHAIN_CLOCK(prof_acked);
+      MSCCLX_CHAIN_ADD(2, prof_issued, prof_acked);
     }
+    MSCCLX_CHAIN_CLOCK(prof_moved);
     if (snd_bit && writer) publish(out_head, (u64)sseq + 1);
     if (rcv_bit && writer) publish(in_tail, (u64)rseq + 1);
     rseq += rcv_bit;
@@ -1169,7 +1180,13 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       if (++pass >= npasses) break;
     }
     op = after;
+#ifdef MSCCLX_PROFILE
+    prof_acc[3] += __builtin_amdgcn_s_memtime() - prof_moved;
+#endif
   }
+#ifdef MSCCLX_PROFILE
+  prof_acc[4] = __builtin_amdgcn_s_memtime() - prof_begin;
+#endif
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -1228,7 +1245,14 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin);
 #endif
   } else if (!LL && !FOLD && VEC && hosted == 1 && blockDim.x == 64) {
+#ifdef MSCCLX_PROFILE
+    u64 chain_acc[5] = {0, 0, 0, 0, 0};
+    if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin, chain_acc);
+    prof_wait = chain_acc[0]; prof_move = chain_acc[1]; prof_ack = chain_acc[2]; prof_fin = chain_acc[3];
+    if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
+#else
     if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin);
+#endif
   } else {
   if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
