@@ -23,7 +23,8 @@ which matters for the two latency-bound workloads (a launch on an idle GPU pays 
 metric/value: algbw in GB/s (nccl-tests convention, S / t).  "roofline": algorithmic bytes per launch
 / mean launch duration against the 8 TB/s HBM peak.  "cpu_baseline": the NumPy interpreter of the
 same IR on this box's host cores (reported, not a target).  "host_us": what a caller pays on the host
-for plan creation, configuration, binding and launching.
+for plan creation, configuration, binding and launching.  "roofline.streaming_reference": what torch's own
+copy and add kernels reach on the same box over 1 GiB arrays (read + write bytes), a yardstick beside the peak.
 """
 import argparse
 import json
@@ -54,6 +55,31 @@ def measured_traffic():
     for key, val in re.findall(r"^\s*(c\d) traffic = (\d+) bytes per launch", text, re.M):
         out[key] = int(val)
     return out
+
+
+def streaming_reference():
+    """What dependency-free streaming kernels reach on this box, read + write bytes over HIP-event time:
+    torch's device copy and its bf16 add (2 reads : 1 write) over 1 GiB arrays, median of 7 after 3 warm-ups.
+    A yardstick next to the 8 TB/s peak, not part of the executor."""
+    import torch
+    n = 1 << 30
+    a = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
+    b = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
+    c = torch.empty_like(a)
+    a16, b16, c16 = (t.view(torch.bfloat16) for t in (a, b, c))
+
+    def median_us(fn):
+        ts = []
+        for it in range(10):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); fn(); e1.record(); torch.cuda.synchronize()
+            if it >= 3:
+                ts.append(e0.elapsed_time(e1) * 1e3)
+        return sorted(ts)[len(ts) // 2]
+    copy_us = median_us(lambda: c.copy_(a))
+    add_us = median_us(lambda: torch.add(a16, b16, out=c16))
+    return {"copy_GBps": round(2 * n / copy_us / 1e3, 1), "add_GBps": round(3 * n / add_us / 1e3, 1), "bytes_per_array": n,
+            "what": "torch copy_ and bf16 add on this box, read + write bytes / HIP-event time"}
 
 
 def ensure_built():
@@ -315,6 +341,7 @@ def main():
                      "kernel_ms_queued": round(head["kernel_ms_queued"], 5), "note": ROOFLINE_NOTE},
         "host_us": head["host_us"],
     }
+    line["roofline"]["streaming_reference"] = streaming_reference()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.config)
     if not args.no_others:
