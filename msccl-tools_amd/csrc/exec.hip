@@ -44,11 +44,11 @@ static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll, bool fold) {
 }
 
 // Everything the kernel reads about the program, packed into one block of bytes that is uploaded in
-// one copy: threadblocks | steps | folded dependencies | connections | hosting table.
+// one copy: threadblocks | steps | folded dependencies | connections | hosting table | context records.
 struct DeviceImage {
   std::vector<unsigned char> bytes;
-  size_t off_tbs = 0, off_ops = 0, off_extras = 0, off_conns = 0, off_hosting = 0;
-  size_t hosting_wg_words = 0, hosting_ctx_words = 0;
+  size_t off_tbs = 0, off_ops = 0, off_extras = 0, off_conns = 0, off_hosting = 0, off_ctxs = 0;
+  bool one_each = false;              // workgroup w hosts context w and no other
   std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
   std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
   kernel_fn kernel = nullptr;
@@ -287,17 +287,54 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
     hop.swap(fused);
     d->dev_ir_step.swap(fused_ir);
   }
+  // One record per hosted context, in hosting order: where its counters and slots are, its slice's bounds.
+  std::vector<DevCtx> ctxs(g.ctx_tb.size());
+  {
+    const uint64_t ub = g.unit_bytes, fb = g.ll ? (uint64_t)kLLUnitBytes : ub, slot_step = g.vector_path ? 16 : 1;
+    for (size_t k = 0; k < ctxs.size(); ++k) {
+      const int32_t tbi = g.ctx_tb[k], slice = g.ctx_slice[k];
+      const DevTb& tb = htb[(size_t)tbi];
+      DevCtx rec{};
+      Hosted& h = rec.h;
+      h.tb = tbi; h.slice = slice;
+      h.nops = tb.nops; h.op_begin = tb.op_begin;
+      const uint64_t u0 = slice_begin(g.chunk_units, g.slice_grain, g.slices, slice), u1 = slice_begin(g.chunk_units, g.slice_grain, g.slices, slice + 1);
+      h.npasses = (unsigned)((u1 - u0 + g.piece_units - 1) / g.piece_units);
+      const uint64_t slice_fifo = (uint64_t)slice * g.slice_fifo_units * fb;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
+      const uint64_t area = (uint64_t)kSyncHeaderWords + (uint64_t)slice * g.sync_slice_words;
+      const uint64_t heads = area + (uint64_t)ntb * kSyncStrideWords, tails = heads + (uint64_t)ncn * kSyncStrideWords;
+      if (tails + (uint64_t)ncn * kSyncStrideWords > 0xffffffffull) return fail(MSCCLX_ERR_CAPACITY, "counter area beyond 32-bit word indices");
+      h.flags = (uint32_t)area;
+      h.my_flag = (uint32_t)(area + (uint64_t)tbi * kSyncStrideWords);
+      auto slots_of = [&](int conn, uint32_t* first, uint32_t* slot_bytes, uint32_t* wrap) -> bool {
+        const uint64_t at = (slice_fifo + hcn[(size_t)conn].fifo_off * fb) / slot_step, bytes = (uint64_t)hcn[(size_t)conn].slot_units * fb;
+        if (at > 0xffffffffull || bytes * (uint64_t)g.depth > 0xffffffffull) return false;
+        *first = (uint32_t)at; *slot_bytes = (uint32_t)bytes; *wrap = (uint32_t)(bytes * (uint64_t)g.depth);
+        return true;
+      };
+      if (tb.recv_conn >= 0) {
+        if (!slots_of(tb.recv_conn, &h.in_slots, &h.in_slot_bytes, &h.in_wrap)) return fail(MSCCLX_ERR_CAPACITY, "FIFO region beyond 32-bit slot offsets");
+        h.head_in = (uint32_t)(heads + (uint64_t)tb.recv_conn * kSyncStrideWords); h.tail_out = (uint32_t)(tails + (uint64_t)tb.recv_conn * kSyncStrideWords);
+      }
+      if (tb.send_conn >= 0) {
+        if (!slots_of(tb.send_conn, &h.out_slots, &h.out_slot_bytes, &h.out_wrap)) return fail(MSCCLX_ERR_CAPACITY, "FIFO region beyond 32-bit slot offsets");
+        h.head_out = (uint32_t)(heads + (uint64_t)tb.send_conn * kSyncStrideWords); h.tail_in = (uint32_t)(tails + (uint64_t)tb.send_conn * kSyncStrideWords);
+      }
+      rec.left = (uint32_t)(u1 - u0);
+      rec.off = u0 * ub;
+      ctxs[k] = rec;
+    }
+  }
+  img->one_each = g.wg_begin.size() == ctxs.size() + 1;  // (a workgroup hosts at least one context: then each hosts exactly one, in order)
+  for (size_t w = 0; img->one_each && w < g.wg_begin.size(); ++w) img->one_each = g.wg_begin[w] == (int32_t)w;
   std::vector<int32_t> hosting(g.wg_begin);
-  hosting.insert(hosting.end(), g.ctx_tb.begin(), g.ctx_tb.end());
-  hosting.insert(hosting.end(), g.ctx_slice.begin(), g.ctx_slice.end());
-  img->hosting_wg_words = g.wg_begin.size();
-  img->hosting_ctx_words = g.ctx_tb.size();
   img->bytes.clear();
   img->off_tbs = append_table(img->bytes, htb);
   img->off_ops = append_table(img->bytes, hop);
   img->off_extras = append_table(img->bytes, extras, kExtraDepWords);
   img->off_conns = append_table(img->bytes, hcn);
   img->off_hosting = append_table(img->bytes, hosting);
+  img->off_ctxs = append_table(img->bytes, ctxs);
   return MSCCLX_OK;
 }
 
@@ -330,8 +367,8 @@ static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img,
   }
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan.tbs.size(); kp.nconns = (int)plan.conns.size();
   kp.wg_begin = (const int32_t*)(tables + img.off_hosting);
-  kp.ctx_tb = kp.wg_begin + img.hosting_wg_words;
-  kp.ctx_slice = kp.ctx_tb + img.hosting_ctx_words;
+  kp.ctxs = (const DevCtx*)(tables + img.off_ctxs);
+  kp.one_each = img.one_each ? 1u : 0u;
   return kp;
 }
 

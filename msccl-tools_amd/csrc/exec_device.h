@@ -366,7 +366,6 @@ __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t
 // f = launch number (10 bits) | message number + 1 (22 bits): never 0, so a cleared slot matches
 // nothing, and what an earlier message or launch left in a line cannot be taken for this message.
 // ------------------------------------------------------------------------------------------------
-constexpr int kLLUnitBytes = 32;
 __device__ __forceinline__ uint32_t ll_flag(uint32_t epoch, u64 seq) { return ((epoch & 0x3ffu) << 22) | (uint32_t)((seq + 1) & 0x3fffffu); }
 __device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { return l0.y == f && l0.w == f && l1.y == f && l1.w == f; }
 
@@ -489,28 +488,6 @@ enum {
   kMany = 64,    // dst = ((dst (+) a[0]) (+) a[1]) ...: `rows` sources, `out` bytes apart
 };
 enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
-
-// One hosted context = (threadblock, slice), run by one lane of wave 0.  What never changes while it
-// runs sits in LDS (one entry per lane, touched by that lane only), so that it occupies no registers
-// while the workgroup moves data; what changes from step to step is the lane's Context.
-struct Hosted {
-  int nops, op_begin;
-  unsigned npasses;
-  // Slots: offsets from the start of the FIFO region, in 16-byte steps on the vector path and in bytes otherwise; counters: 64-bit word index
-  // inside this launch's counter area.  32 bits each, so that the lot is read from LDS in one go.
-  uint32_t in_slots, out_slots;    // first slot of the incoming / outgoing connection, in this slice
-  uint32_t in_slot_bytes, out_slot_bytes;
-  uint32_t in_wrap, out_wrap;      // depth * slot bytes: where the ring of slots starts over
-  uint32_t flags;                  // flag of threadblock t of this slice is flags + t * kSyncStrideWords
-  uint32_t my_flag;
-  uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
-  uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
-  int tb, slice;                   // for the watchdog's report only
-};
-
-__device__ __forceinline__ u64* slice_area(u64* base, const KernelParams& p, int slice) {
-  return base + kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words;
-}
 
 // The changing part.  Everything that depends on the pass or on how many messages went by is kept
 // as a running value, advanced when a step finishes: the lane's instructions between two moves are
@@ -656,46 +633,23 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
   else describe_step<UB == 16, LL>(c, h, p, epoch, next);
 }
 
-// Set up the context (threadblock tbi, slice) : its constants in `h`, its state in `c`, standing at
-// its first step.  `writer` also clears, for the next launch, the counters this context alone writes.
+// Set up hosted context number `ctx`: its constants in `h` (the record worked out when the buffers were
+// bound), its state in `c`, standing at its first step.  `writer` also clears, for the next launch,
+// the counters this context alone writes.
 template <bool VEC, int EB, bool LL>
-__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int tbi, int slice, bool writer) {
-  constexpr uint64_t UB = VEC ? 16 : EB;
-  constexpr uint64_t FB = LL ? kLLUnitBytes : UB;
-  h.tb = tbi;
-  h.slice = slice;
-  const DevTb tb = p.tbs[tbi];
-  h.nops = tb.nops; h.op_begin = tb.op_begin;
-  const uint64_t u0 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice), u1 = slice_begin(p.chunk_units, p.slice_grain, p.slices, slice + 1);
-  h.npasses = (unsigned)((u1 - u0 + p.piece_units - 1) / p.piece_units);
-  const uint64_t slice_fifo = (uint64_t)slice * p.slice_fifo_units * FB;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
-  const uint32_t area = (uint32_t)(kSyncHeaderWords + (uint64_t)slice * p.sync_slice_words);
-  const uint32_t heads = area + (uint32_t)p.ntbs * kSyncStrideWords, tails = heads + (uint32_t)p.nconns * kSyncStrideWords;
-  h.flags = area;
-  h.my_flag = area + (uint32_t)tbi * kSyncStrideWords;
-  h.in_slots = h.out_slots = 0; h.in_slot_bytes = h.out_slot_bytes = 0; h.in_wrap = h.out_wrap = 0;
-  h.head_in = h.tail_out = h.head_out = h.tail_in = 0;
-  if (tb.recv_conn >= 0) {
-    const DevConn cn = p.conns[tb.recv_conn];
-    h.in_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.in_slot_bytes = (uint32_t)(cn.slot_units * FB); h.in_wrap = h.in_slot_bytes * (uint32_t)p.depth;
-    h.head_in = heads + (uint32_t)tb.recv_conn * kSyncStrideWords; h.tail_out = tails + (uint32_t)tb.recv_conn * kSyncStrideWords;
-  }
-  if (tb.send_conn >= 0) {
-    const DevConn cn = p.conns[tb.send_conn];
-    h.out_slots = (uint32_t)((slice_fifo + cn.fifo_off * FB) / (VEC ? 16 : 1)); h.out_slot_bytes = (uint32_t)(cn.slot_units * FB); h.out_wrap = h.out_slot_bytes * (uint32_t)p.depth;
-    h.head_out = heads + (uint32_t)tb.send_conn * kSyncStrideWords; h.tail_in = tails + (uint32_t)tb.send_conn * kSyncStrideWords;
-  }
+__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int ctx, bool writer) {
+  const DevCtx rec = p.ctxs[ctx];
+  h = rec.h;
   c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
-  c.left = (uint32_t)(u1 - u0);
-  c.off = u0 * UB;
-  c.active = tb.nops > 0 && h.npasses > 0;
-  if (writer) {
-    u64* nxt = slice_area(p.sync_nxt, p, slice);
-    nxt[(uint64_t)tbi * kSyncStrideWords] = 0;
-    if (tb.send_conn >= 0) nxt[((uint64_t)p.ntbs + tb.send_conn) * kSyncStrideWords] = 0;
-    if (tb.recv_conn >= 0) nxt[((uint64_t)p.ntbs + p.nconns + tb.recv_conn) * kSyncStrideWords] = 0;
+  c.left = rec.left;
+  c.off = rec.off;
+  c.active = h.nops > 0 && h.npasses > 0;
+  if (writer) {  // (word 0 of an area is the abort word: no head or tail has index 0, which therefore says "no such connection")
+    p.sync_nxt[h.my_flag] = 0;
+    if (h.head_out) p.sync_nxt[h.head_out] = 0;
+    if (h.tail_out) p.sync_nxt[h.tail_out] = 0;
   }
-  if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[tb.op_begin]);
+  if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[h.op_begin]);
 }
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
@@ -921,10 +875,14 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
   Hosted h;
+  uint32_t left;  // units of the slice still to do (this pass included)
+  u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<true, R::kElemBytes, true>(h, first, p, epoch, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+    init_context<true, R::kElemBytes, true>(h, first, p, epoch, ctx, writer);
     if (!first.active) return;
+    left = uniform(first.left);
+    off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
   const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
@@ -938,8 +896,6 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
   const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
   uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
-  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice));
-  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice) * 16;
   DevOp op = fetch_step(ops);
   MSCCLX_CHAIN_CLOCK(prof_begin);
   u64 prof_mark = 0;  // profiling builds: when the previous step's stores were issued
@@ -1076,10 +1032,14 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
   Hosted h;
+  uint32_t left;  // units of the slice still to do (this pass included)
+  u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<true, R::kElemBytes, false>(h, first, p, 0, p.ctx_tb[ctx], p.ctx_slice[ctx], writer);
+    init_context<true, R::kElemBytes, false>(h, first, p, 0, ctx, writer);
     if (!first.active) return;
+    left = uniform(first.left);
+    off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
   const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
@@ -1095,8 +1055,6 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
   const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
   uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
-  uint32_t left = (uint32_t)(slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice + 1) - slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice));
-  u64 off = slice_begin(p.chunk_units, p.slice_grain, p.slices, watch.slice) * 16;
   DevOp op = fetch_step(ops);
   // (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for the step's counters, 1 moving its rows,
   // 2 waiting for the stores' acknowledgement, 3 on the bookkeeping between steps, 4 in all)
@@ -1220,7 +1178,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
   u64* const abort_word = p.sync_cur;
   const int lane = threadIdx.x;
   const bool poller = threadIdx.x < 64;
-  const int ctx_begin = p.wg_begin[blockIdx.x], hosted = p.wg_begin[blockIdx.x + 1] - ctx_begin;
+  const int ctx_begin = p.one_each ? (int)blockIdx.x : p.wg_begin[blockIdx.x], hosted = p.one_each ? 1 : p.wg_begin[blockIdx.x + 1] - ctx_begin;
   // LL, one hosted context: nothing else could run while it waits for a message, so the lane does not
   // watch for it; the moving threads go straight to the lines and retry them until they are there.
   const bool direct = LL && hosted == 1;
@@ -1254,7 +1212,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin);
 #endif
   } else {
-  if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, p.ctx_tb[ctx_begin + lane], p.ctx_slice[ctx_begin + lane], true);
+  if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, ctx_begin + lane, true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
   int cursor = 0;
   unsigned busy_rounds = 0;

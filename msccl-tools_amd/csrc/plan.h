@@ -90,6 +90,35 @@ struct DevConn {
   uint32_t pad;
 };
 
+// One hosted context = (threadblock, slice), run by one lane of wave 0.  What never changes while it
+// runs sits in LDS (one entry per lane, touched by that lane only), so that it occupies no registers
+// while the workgroup moves data; what changes from step to step is the lane's Context.
+struct Hosted {
+  int nops, op_begin;
+  unsigned npasses;
+  // Slots: offsets from the start of the FIFO region, in 16-byte steps on the vector path and in bytes otherwise; counters: 64-bit word index
+  // inside this launch's counter area.  32 bits each, so that the lot is read from LDS in one go.
+  uint32_t in_slots, out_slots;    // first slot of the incoming / outgoing connection, in this slice
+  uint32_t in_slot_bytes, out_slot_bytes;
+  uint32_t in_wrap, out_wrap;      // depth * slot bytes: where the ring of slots starts over
+  uint32_t flags;                  // flag of threadblock t of this slice is flags + t * kSyncStrideWords
+  uint32_t my_flag;
+  uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
+  uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
+  int tb, slice;                   // for the watchdog's report only
+};
+
+// A context's record as the device reads it: everything about (threadblock, slice) that the geometry and
+// the tables fix, worked out once when buffers are bound, so that a workgroup starts a context with
+// one round of loads instead of a walk hosting table -> threadblock -> connections and a handful of
+// 64-bit divisions for the slice's bounds.
+struct DevCtx {
+  Hosted h;
+  uint32_t left;   // units of the slice (what the first pass has in front of it)
+  uint64_t off;    // byte offset of the slice inside every chunk
+};
+static_assert(sizeof(DevCtx) == 80, "five 16-byte loads fetch a context");
+
 struct Geometry {
   uint64_t chunk_units = 0;   // units (16-byte vectors or elements) per chunk
   uint32_t unit_bytes = 0;
@@ -132,8 +161,8 @@ struct KernelParams {
   uint32_t finish_group;        // workgroups per group of the end-of-launch count
   int32_t slices, depth, ntbs, nconns;
   const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
-  const int32_t* ctx_tb;        // hosted contexts, grouped by workgroup: threadblock row ...
-  const int32_t* ctx_slice;     // ... and slice
+  const DevCtx* ctxs;           // hosted contexts, grouped by workgroup
+  uint32_t one_each;            // 1: workgroup w hosts context w and no other (wg_begin need not be read)
 };
 
 #ifdef __HIPCC__
@@ -152,6 +181,7 @@ MSCCLX_HOST_DEVICE inline uint64_t slice_begin(uint64_t chunk_units, uint32_t gr
 constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
 constexpr int kProfTrace = 248;       // MSCCLX_PROFILE builds: moves logged per workgroup ...
 constexpr int kProfWords = 8 + kProfTrace;  // ... after its 8 words of totals
+constexpr int kLLUnitBytes = 32;       // a flag-in-data line pair: 16 bytes of payload in 32
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
 // The control block in front of the two counter areas: word 0 = launches finished so far, word 1 =
