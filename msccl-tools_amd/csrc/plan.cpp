@@ -593,13 +593,15 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // chunks: 6 to 40 % off twenty-odd of them (PCIe-hierarchical all-reduce at 16 KiB chunks 56 -> 33 us,
       // pipelined all-pairs 33 -> 23 us), within 2 % for the rest.  Bigger chunks lose as often as they win, and
       // a ring whose every threadblock is busy all the time (64 ranks) loses beyond one context per SIMD.
-      if (g.vector_path && chunk_bytes <= 64 * 1024 && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups) {
+      // Chunks of up to 128 KiB too where ALL contexts are at most one per SIMD (8-rank ring on 1 MiB: 33.3 -> 31.5 us).
+      if (g.vector_path && chunk_bytes <= 128 * 1024 && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups) {
+        const double busy_share = chunk_bytes <= 64 * 1024 ? ratio : 1.0;
         int64_t fine = 1;
         while ((uint64_t)fine * 1024 < chunk_bytes) fine *= 2;  // pieces of at most 1 KiB
         for (int64_t s : {fine, fine / 2}) {
           if (s <= slices || (uint64_t)s > g.chunk_units) continue;
           const int64_t contexts = s * ntbs;
-          if (contexts > capacity_by_threads[thread_index(64)] || (double)contexts > ratio * 4.0 * (double)num_cus) continue;
+          if (contexts > capacity_by_threads[thread_index(64)] || (double)contexts > busy_share * 4.0 * (double)num_cus) continue;
           slices = s;
           break;
         }

@@ -208,7 +208,7 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
     MI355X: (workgroups, threads, slices, piece bytes, passes, most contexts on a workgroup)."""
     from msccl.executor.workloads import WORKLOADS
     want = {
-        "c1": (512, 64, 64, 2048, 1, 1),        # latency bound: two workgroups of one wave per compute unit, 2 KiB pieces
+        "c1": (1024, 64, 128, 1024, 1, 1),      # latency bound: one workgroup of one wave per SIMD, one 16-byte unit per lane
         "c2": (512, 512, 64, 131072, 1, 4),     # a ring is always busy: 4 contexts per workgroup, one pass
         "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
