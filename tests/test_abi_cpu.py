@@ -247,6 +247,29 @@ def test_geometry_between_the_benchmark_sizes(mscclx_lib):
         assert (i.threads, i.slices, i.piece_bytes) == expect, (key, nbytes, (i.threads, i.slices, i.piece_bytes))
 
 
+def test_small_chunks_are_cut_one_unit_per_lane(mscclx_lib):
+    """Chunks of up to 64 KiB: pieces of 1 KiB (one 16-byte unit per lane of a one-wave workgroup), else 2 KiB,
+    where every context keeps a workgroup of its own and the busy ones are at most one per SIMD;
+    (workgroups, threads, slices, piece bytes, most contexts on a workgroup) on a 256-CU part."""
+    want = {
+        ("allreduce_a100_pcie_hierarchical_8r", 16 << 10): (2048, 64, 16, 1024, 1),   # 128 threadblocks that wait two thirds of the time
+        ("pipeline_a100_allpairs_8r", 16 << 10): (2176, 64, 16, 1024, 1),
+        ("allreduce_1step_4r", 64 << 10): (1024, 64, 64, 1024, 1),
+        ("allreduce_allpairs_8r_2inst", 16 << 10): (1024, 64, 8, 2048, 1),             # 1 KiB pieces would be 2048 busy contexts: 2 KiB
+        ("c5_allreduce_ring_64r_1ch_1inst", 16 << 10): (1024, 64, 16, 1024, 1),        # every threadblock busy: one context per SIMD ...
+        ("c5_allreduce_ring_64r_1ch_1inst", 64 << 10): (512, 64, 8, 8192, 1),          # ... and no more
+        ("c4_hierarchical_allreduce_8x4_2inst_auto", 4 << 10): (3840, 64, 2, 2048, 1),  # 1920 threadblocks: four slices would not get a workgroup each
+        ("c1_allreduce_ring_8r_1ch_1inst", 128 << 10): (1024, 64, 128, 1024, 1),       # up to 128 KiB where ALL contexts are one per SIMD
+        ("allgather_recursive_doubling_8r", 128 << 10): (768, 64, 32, 4096, 1),        # 3072 contexts would be three per SIMD: the latency model's 32
+    }
+    for (name, chunk_bytes), expect in want.items():
+        i = Plan(parse_algo_xml(golden_util.load(name))).configure(chunk_bytes, "float32", max_workgroups=4096)
+        assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.max_hosted) == expect, (name, chunk_bytes, (i.workgroups, i.threads, i.slices, i.piece_bytes, i.max_hosted))
+    # a knob that fixes the workgroups keeps the latency model's slices
+    i = Plan(parse_algo_xml(golden_util.load("allreduce_a100_pcie_hierarchical_8r"))).configure(16 << 10, "float32", max_workgroups=4096, threads=128)
+    assert i.slices == 4
+
+
 def test_run_static_refuses_an_oversized_plan_before_touching_the_gpu(mscclx_lib):
     """The size check of mscclx_plan_run_static is host arithmetic: a plan whose tables, counters and
     FIFO slots exceed MSCCLX_STATIC_SCRATCH_BYTES is refused with CAPACITY before any HIP call."""
