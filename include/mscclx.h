@@ -121,7 +121,7 @@ typedef struct {
   int32_t fifo_depth;
   int32_t passes;      /* passes of the step list the longest slice makes          */
   int32_t connections;
-  int32_t vector_path; /* 1: 16-byte vector path, 0: element path                  */
+  int32_t vector_path; /* 1: 16-byte units (chunk_bytes a multiple of 4), 0: element by element */
   int32_t zero_copy_messages; /* messages per pass read in place instead of staged  */
   int32_t staged_messages;
   int32_t max_hosted;  /* most contexts any workgroup hosts                         */
@@ -162,7 +162,9 @@ int mscclx_plan_min_fifo_depth(const mscclx_plan* plan);
 uint64_t mscclx_plan_algorithmic_units(const mscclx_plan* plan);
 
 /* Fixes the geometry for chunks of `chunk_bytes` bytes of `dtype` and reports it, including the
- * workspace the caller must provide.  Queries the current device unless cfg->max_workgroups > 0. */
+ * workspace the caller must provide.  Queries the current device unless cfg->max_workgroups > 0.
+ * Any positive multiple of the element size is accepted; multiples of 4 bytes move in 16-byte units
+ * (fastest when chunks start on cache lines: multiples of 256), the rest element by element. */
 int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, int32_t redop,
                           const mscclx_config* cfg, mscclx_info* info);
 

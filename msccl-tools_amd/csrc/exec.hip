@@ -320,6 +320,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
         if (!slots_of(tb.send_conn, &h.out_slots, &h.out_slot_bytes, &h.out_wrap)) return fail(MSCCLX_ERR_CAPACITY, "FIFO region beyond 32-bit slot offsets");
         h.head_out = (uint32_t)(heads + (uint64_t)tb.send_conn * kSyncStrideWords); h.tail_in = (uint32_t)(tails + (uint64_t)tb.send_conn * kSyncStrideWords);
       }
+      h.clip = slice + 1 == g.slices ? (uint32_t)(g.chunk_units * ub - plan->chunk_bytes) : 0u;  // (0 unless the chunk ends inside its last unit)
       rec.left = (uint32_t)(u1 - u0);
       rec.off = u0 * ub;
       ctxs[k] = rec;
@@ -354,6 +355,7 @@ static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img,
   kp.host_status = status;
   kp.prof = prof;
   kp.chunk_units = g.chunk_units;
+  kp.chunk_bytes = plan.chunk_bytes;
   kp.slice_fifo_units = g.slice_fifo_units;
   kp.sync_slice_words = g.sync_slice_words;
   kp.timeout_ticks = (uint64_t)plan.timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
@@ -444,7 +446,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   if (redop < 0 || redop >= MSCCLX_NUM_REDOPS) return fail(MSCCLX_ERR_INVALID_ARG, "unknown reduction");
   const int elem = dtype_size(dtype);
   if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
-  const bool vec = chunk_bytes % 16 == 0;
+  const bool vec = chunk_takes_vector_path(chunk_bytes);
   int num_cus = 256;
   int capacity[kThreadChoices];
   if (cfg.max_workgroups > 0) {

@@ -206,13 +206,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 #endif
 constexpr int kUnroll = MSCCLX_UNROLL;
 
-// out1[, out2] = a [(+) b] over n units of W bytes.
+// out1[, out2] = a [(+) b] over n units of W bytes, the last of which lacks `clip` bytes (the end of a chunk that is
+// no multiple of 16 bytes: the descriptors end there, so the missing dwords read as zero and are not written).
 template <class R, int W, bool HAS_B, bool HAS_O2, bool NT1>
-__device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n) {
+__device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n, uint32_t clip) {
   typedef Access<W> A;
   typedef typename A::word word;
   constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const uint32_t bytes = n * W;
+  const uint32_t bytes = n * W - clip;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
   const uint32_t T = blockDim.x;
@@ -250,12 +251,12 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
   }
 }
 
-// rows x n units.  Consecutive rows of an operand are `stride_*` units apart: a chunk for rank
-// buffers, n for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
-// buffer, o2 (the forwarded copy) always a FIFO slot.
+// rows x n units.  Consecutive rows of an operand are `stride_*` BYTES apart: a chunk for rank
+// buffers, n units for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
+// buffer, o2 (the forwarded copy) always a FIFO slot.  clip: see move_units.
 template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool NT1 = false>
 __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
-                                          const unsigned char* b, uint64_t stride_b, int rows, uint32_t n) {
+                                          const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t clip) {
   constexpr int W = VEC ? 16 : R::kElemBytes;
   if (!HAS_B && !HAS_O2 && __builtin_expect(rows > 1 && n <= blockDim.x, 0)) {  // (plain copies only: the scatter and gather steps of all-pairs and all-to-all programs)
     // Several short rows (a multi-chunk step of a latency-bound program): one unit per thread and
@@ -267,16 +268,16 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
     constexpr int RB = 4;
     const uint32_t i = threadIdx.x;
     if (i >= n) return;
-    const uint32_t bytes = n * W;
+    const uint32_t bytes = n * W - clip;
     for (int r0 = 0; r0 < rows; r0 += RB) {
       word x[RB], y[RB];
 #pragma unroll
       for (int k = 0; k < RB; ++k)
-        if (r0 + k < rows) x[k] = A::template ld<XL>(make_rsrc(a + (uint64_t)(r0 + k) * stride_a * W, bytes), (int)(i * W));
+        if (r0 + k < rows) x[k] = A::template ld<XL>(make_rsrc(a + (uint64_t)(r0 + k) * stride_a, bytes), (int)(i * W));
       if (HAS_B) {
 #pragma unroll
         for (int k = 0; k < RB; ++k)
-          if (r0 + k < rows) y[k] = A::template ld<XL>(make_rsrc(b + (uint64_t)(r0 + k) * stride_b * W, bytes), (int)(i * W));
+          if (r0 + k < rows) y[k] = A::template ld<XL>(make_rsrc(b + (uint64_t)(r0 + k) * stride_b, bytes), (int)(i * W));
 #pragma unroll
         for (int k = 0; k < RB; ++k)
           if (r0 + k < rows) x[k] = R::combine(y[k], x[k]);
@@ -284,26 +285,26 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
 #pragma unroll
       for (int k = 0; k < RB; ++k)
         if (r0 + k < rows) {
-          A::template st<X1>(make_rsrc(o1 + (uint64_t)(r0 + k) * stride_o1 * W, bytes), (int)(i * W), x[k]);
+          A::template st<X1>(make_rsrc(o1 + (uint64_t)(r0 + k) * stride_o1, bytes), (int)(i * W), x[k]);
           if (HAS_O2) A::template st<XS>(make_rsrc(o2 + (uint64_t)(r0 + k) * n * W, bytes), (int)(i * W), x[k]);
         }
     }
     return;
   }
   for (int r = 0; r < rows; ++r)
-    move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1 * W, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
-                                    a + (uint64_t)r * stride_a * W, HAS_B ? b + (uint64_t)r * stride_b * W : nullptr, n);
+    move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
+                                    a + (uint64_t)r * stride_a, HAS_B ? b + (uint64_t)r * stride_b : nullptr, n, clip);
 }
 
 // dst = ((dst (+) a0) (+) a1) ... (+) a[m-1] over n units of W bytes; source k starts `stride` bytes
 // after source k-1.  All sources of a unit are in flight together and folded in order, so the result
 // is bit for bit that of m reduce steps -- which would read and write dst m times.
 template <class R, int W, bool NT1>
-__device__ __forceinline__ void move_reduce_many(unsigned char* dst, const unsigned char* a, uint32_t stride, int m, uint32_t n) {
+__device__ __forceinline__ void move_reduce_many(unsigned char* dst, const unsigned char* a, uint32_t stride, int m, uint32_t n, uint32_t clip) {
   typedef Access<W> A;
   typedef typename A::word word;
   constexpr int XL = MSCCLX_AUX_LD, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const uint32_t bytes = n * W;
+  const uint32_t bytes = n * W - clip;
   const __amdgpu_buffer_rsrc_t rd = make_rsrc(dst, bytes);
   // one descriptor for all sources (the host keeps their span below 2 GiB); source k is reached
   // through the scalar offset of the load, so that the sources cost one scalar register each
@@ -391,13 +392,15 @@ __device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int 
 // IN_LL (its lines are retried until they carry `fin`), a rank buffer otherwise; b is a rank buffer.
 template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1>
 __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* llo, const unsigned char* a, const unsigned char* b, uint32_t n,
-                                              uint32_t fin, uint32_t fout, const LLWatch& watch) {
+                                              uint32_t clip, uint32_t fin, uint32_t fout, const LLWatch& watch) {
   typedef Access<16> A;
   // XV: the retried loads must really be issued again each time round the loop (bit 31 = volatile, for the compiler only)
   constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, XV = (int)(0x80000000u | MSCCLX_AUX), X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, n * (IN_LL ? kLLUnitBytes : 16));
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, n * (HAS_B ? 16 : (IN_LL ? kLLUnitBytes : 16)));
-  const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? n * 16 : 0);
+  // (rank buffers end `clip` bytes inside their last unit; lines are always whole: their flags must arrive)
+  const uint32_t local_bytes = n * 16 - clip;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, IN_LL ? n * kLLUnitBytes : local_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, HAS_B ? local_bytes : (IN_LL ? n * kLLUnitBytes : local_bytes));
+  const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? local_bytes : 0);
   const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * kLLUnitBytes : 0);
   const uint32_t T = blockDim.x;
   constexpr int UA = 2;  // small pieces: few lines per thread, few registers
@@ -456,16 +459,16 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
   }
 }
 
-// rows x n units; rank-buffer rows are `stride_*` units apart, slot rows are packed.
+// rows x n units; rank-buffer rows are `stride_*` bytes apart, slot rows are packed.
 template <class R, bool IN_LL, bool HAS_B, bool HAS_O1, bool OUT_LL, bool NT1 = false>
 __device__ __forceinline__ void move_rows_ll(unsigned char* o1, uint64_t stride_o1, unsigned char* llo, const unsigned char* a, uint64_t stride_a,
-                                             const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t fin, uint32_t fout,
+                                             const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t clip, uint32_t fin, uint32_t fout,
                                              const LLWatch& watch) {
   for (int r = 0; r < rows; ++r)
-    move_units_ll<R, IN_LL, HAS_B, HAS_O1, OUT_LL, NT1>(HAS_O1 ? o1 + (uint64_t)r * stride_o1 * 16 : nullptr,
+    move_units_ll<R, IN_LL, HAS_B, HAS_O1, OUT_LL, NT1>(HAS_O1 ? o1 + (uint64_t)r * stride_o1 : nullptr,
                                                        OUT_LL ? llo + (uint64_t)r * n * kLLUnitBytes : nullptr,
-                                                       a + (uint64_t)r * (IN_LL ? (uint64_t)n * kLLUnitBytes : stride_a * 16),
-                                                       HAS_B ? b + (uint64_t)r * stride_b * 16 : nullptr, n, fin, fout, watch);
+                                                       a + (uint64_t)r * (IN_LL ? (uint64_t)n * kLLUnitBytes : stride_a),
+                                                       HAS_B ? b + (uint64_t)r * stride_b : nullptr, n, clip, fin, fout, watch);
 }
 
 // What the workgroup does for one step of one context: operands as byte addresses, filled in by the
@@ -486,6 +489,7 @@ enum {
   kAPacked = 16, // a is a slot
   kToSlot = 32,  // the first (only) destination is `out` instead of dst
   kMany = 64,    // dst = ((dst (+) a[0]) (+) a[1]) ...: `rows` sources, `out` bytes apart
+  kClipShift = 8, kClipMask = 3 << 8,  // bits 8-9: dwords that the last unit of a rank-buffer row lacks (see move_units)
 };
 enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
 
@@ -535,7 +539,7 @@ __device__ __forceinline__ bool extras_ready(const Context& c, const Hosted& h, 
 __device__ __forceinline__ void mark_many_sources(Context& c, const DevOp& op) {
   if ((op.word & 15u) == MSCCLX_OP_REDUCE && op.in_addr) {
     c.m.out = op.in_addr;
-    c.m.kind = kMany | ((op.word & kOpNtStore) ? (int)kNt1 : 0);
+    c.m.kind = kMany | ((op.word & kOpNtStore) ? (int)kNt1 : 0) | (c.m.kind & kClipMask);
   }
 }
 
@@ -592,7 +596,8 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     case MSCCLX_OP_REDUCE: m.a = op.src_addr + c.off; kind = kHasB; break;
     default: break;
   }
-  m.kind = kind;
+  // the pass that reaches the end of the slice: its rows may end inside their last unit
+  m.kind = kind | (c.left <= p.piece_units ? (int)(h.clip >> 2) << kClipShift : 0);
 }
 
 // The description of the step after the one `c` stands at.  It is fetched before the counters of
@@ -657,39 +662,41 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
 template <class R, bool VEC, bool LL, bool FOLD = false>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
-  const u64 cs = p.chunk_units;
+  constexpr int W = VEC ? 16 : R::kElemBytes;
+  const u64 cs = p.chunk_bytes;                   // rows of a rank buffer are a chunk apart ...
+  const u64 packed = (u64)m.n * W;                // ... rows in a slot are packed
+  const uint32_t clip = (((uint32_t)m.kind & kClipMask) >> kClipShift) * 4u;
   unsigned char* const dst = (unsigned char*)m.dst;
   unsigned char* const out = (unsigned char*)m.out;
   const unsigned char* const a = (const unsigned char*)m.a;
   if (FOLD && __builtin_expect((m.kind & kMany) != 0, 0)) {  // (only the bind of a FOLD kernel makes such steps)
-    constexpr int W = VEC ? 16 : R::kElemBytes;
-    if (m.kind & kNt1) move_reduce_many<R, W, true>(dst, a, (uint32_t)m.out, m.rows, m.n);
-    else move_reduce_many<R, W, false>(dst, a, (uint32_t)m.out, m.rows, m.n);
+    if (m.kind & kNt1) move_reduce_many<R, W, true>(dst, a, (uint32_t)m.out, m.rows, m.n, clip);
+    else move_reduce_many<R, W, false>(dst, a, (uint32_t)m.out, m.rows, m.n, clip);
     return;
   }
   if (LL && (m.kind & kLLKind)) {
     const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
     const LLWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, tb, step, slice, (u64)pass};
     switch (m.kind & 7) {
-      case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, m.n, nullptr, 0, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
-      case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, m.n, dst, cs, m.rows, m.n, fin, fout, watch); break;
+      case kLLSend: move_rows_ll<R, false, false, false, true>(nullptr, 0, out, a, cs, nullptr, 0, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRecv: move_rows_ll<R, true, false, true, false>(dst, cs, nullptr, a, 0, nullptr, 0, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRecvNt: move_rows_ll<R, true, false, true, false, true>(dst, cs, nullptr, a, 0, nullptr, 0, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRcs: move_rows_ll<R, true, false, true, true>(dst, cs, out, a, 0, nullptr, 0, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRrc: move_rows_ll<R, true, true, true, false>(dst, cs, nullptr, a, 0, dst, cs, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRrs: move_rows_ll<R, true, true, false, true>(nullptr, 0, out, a, 0, dst, cs, m.rows, m.n, clip, fin, fout, watch); break;
+      case kLLRrcs: move_rows_ll<R, true, true, true, true>(dst, cs, out, a, 0, dst, cs, m.rows, m.n, clip, fin, fout, watch); break;
       default: break;
     }
   } else {
-    const u64 stride_a = (m.kind & kAPacked) ? (u64)m.n : cs;
+    const u64 stride_a = (m.kind & kAPacked) ? packed : cs;
     unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
-    const u64 stride_o1 = (m.kind & kToSlot) ? (u64)m.n : cs;
+    const u64 stride_o1 = (m.kind & kToSlot) ? packed : cs;
     switch (m.kind & 7) {
-      case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n); break;
-      case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n); break;
-      case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n); break;
+      case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n, clip); break;
+      case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n, clip); break;
       default: break;
     }
   }
@@ -885,7 +892,8 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
     off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
-  const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  const u64 row_stride = p.chunk_bytes;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  const uint32_t end_clip = uniform(h.clip);  // bytes that the last unit of the slice's last pass lacks (see move_units)
   unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
   unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
   const u64* const flags = p.sync_cur + uniform(h.flags);
@@ -940,10 +948,11 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
     unsigned char* out_row = out_ring + sslot;
     u64 src_row = op.src_addr + off, dst_row = op.dst_addr + off;
     const uint32_t row_line_bytes = n * kLLUnitBytes;
+    const uint32_t local_bytes = n * 16 - (left <= piece ? end_clip : 0u);  // rank-buffer rows may end inside their last unit; lines are whole
     if (t != MSCCLX_OP_NOP) {
       for (uint32_t row = 0; row < cnt; ++row) {
         const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, row_line_bytes), rout = make_rsrc(out_row, row_line_bytes);
-        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, n * 16), rdst = make_rsrc((const void*)dst_row, n * 16);
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, local_bytes), rdst = make_rsrc((const void*)dst_row, local_bytes);
         if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
           if (!chain_round<R, 1>(rin, rout, rsrc, rdst, lane, n, rcv, snd, from_src, has_b, to_local, nt, fin, fout, gate, gate_target, watch, (int)step, pass,
                                  prof_acc, prof_mark, prof_floor)) return;
@@ -1042,7 +1051,8 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
     off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
-  const u64 row_stride = p.chunk_units * 16;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  const u64 row_stride = p.chunk_bytes;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
+  const uint32_t end_clip = uniform(h.clip);  // bytes that the last unit of the slice's last pass lacks (see move_units)
   unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
   unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
   const u64* const flags = p.sync_cur + uniform(h.flags);
@@ -1103,7 +1113,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       u64 a_row = rcv ? (in_place ? op.in_addr + off : (u64)(in_ring + rslot)) : op.src_addr + off;
       const u64 a_stride = (rcv && !in_place) ? (u64)n * 16 : row_stride;
       u64 local_row = op.dst_addr + off, slot_row = (u64)(out_ring + sslot);
-      const uint32_t row_bytes = n * 16;
+      const uint32_t row_bytes = n * 16 - (left <= piece ? end_clip : 0u);  // (slot rows are n units apart, and end where their rank-buffer rows do)
       for (uint32_t row = 0; row < cnt; ++row) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc((const void*)a_row, row_bytes), rlocal = make_rsrc((const void*)local_row, row_bytes);
         const __amdgpu_buffer_rsrc_t rslot_out = make_rsrc((const void*)slot_row, row_bytes);
@@ -1112,7 +1122,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
         else if (n <= 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else  // (eight loads in flight per lane and operand, as the workgroup-wide mover has)
           for (uint32_t base = 0; base < n; base += 512) chain_copy_round<R, 8>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
-        a_row += a_stride; local_row += row_stride; slot_row += row_bytes;
+        a_row += a_stride; local_row += row_stride; slot_row += (u64)n * 16;
       }
       MSCCLX_CHAIN_CLOCK(prof_issued);
       MSCCLX_CHAIN_ADD(1, prof_ready, prof_issued);

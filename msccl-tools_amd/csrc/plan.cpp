@@ -470,11 +470,11 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (cfg.slices < 0 || cfg.piece_bytes < 0 || cfg.fifo_depth < 0 || cfg.workgroups < 0 || cfg.threads < 0)
     return fail(MSCCLX_ERR_INVALID_ARG, "geometry knobs must be >= 0");
   Geometry g;
-  g.vector_path = (chunk_bytes % 16 == 0) ? 1 : 0;
+  g.vector_path = chunk_takes_vector_path(chunk_bytes) ? 1 : 0;
   g.unit_bytes = g.vector_path ? 16 : elem;
-  g.chunk_units = chunk_bytes / g.unit_bytes;
+  g.chunk_units = (chunk_bytes + g.unit_bytes - 1) / g.unit_bytes;  // (the vector path's last unit may be partial)
   if (cfg.protocol < 0 || cfg.protocol > MSCCLX_PROTO_LL) return fail(MSCCLX_ERR_INVALID_ARG, "unknown protocol");
-  if (cfg.protocol == MSCCLX_PROTO_LL && !g.vector_path) return fail(MSCCLX_ERR_UNSUPPORTED, "the LL protocol needs chunks that are a multiple of 16 bytes");
+  if (cfg.protocol == MSCCLX_PROTO_LL && !g.vector_path) return fail(MSCCLX_ERR_UNSUPPORTED, "the LL protocol needs chunks that are a multiple of 4 bytes");
   g.staging = cfg.staging ? 1 : 0;
   const int64_t ntbs = (int64_t)plan.tbs.size();
   if (ntbs == 0) return fail(MSCCLX_ERR_BAD_IR, "the algorithm has no threadblocks");
@@ -539,7 +539,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       for (int64_t c : candidates) {
         // the workgroups this choice would run on: threads follow the piece, workgroups the threads
         const uint64_t slice_bytes = chunk_bytes / (uint64_t)c;
-        const uint64_t piece_bytes = slice_bytes > 128 * 1024 ? 64 * 1024 : slice_bytes;
+        const uint64_t piece_bytes = slice_bytes > 128 * 1024 + 2048 ? 64 * 1024 : slice_bytes;
         int threads = cfg.threads && thread_index(cfg.threads) >= 0 ? cfg.threads : threads_for_piece(piece_bytes);
         while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
         int64_t wgs = cfg.workgroups ? cfg.workgroups : (int64_t)num_cus * 16 / (threads / 64);
@@ -645,10 +645,12 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     longest_slice = std::max(longest_slice, slice_begin(g.chunk_units, g.slice_grain, (int32_t)slices, (int32_t)j + 1) -
                                                 slice_begin(g.chunk_units, g.slice_grain, (int32_t)slices, (int32_t)j));
   uint64_t piece_units = cfg.piece_bytes ? std::max<uint64_t>(1, (uint64_t)cfg.piece_bytes / g.unit_bytes) : longest_slice;
-  if (!cfg.piece_bytes && longest_slice * g.unit_bytes > 128 * 1024) {
-    // equal passes of at most 64 KiB (a short last pass costs as many hand-offs as a full one), on 256-byte boundaries
+  // (a slice a few units over -- a chunk that is no power of two -- is not worth a pass of its own: 2 KiB of slack)
+  const uint64_t slack = 2048 / g.unit_bytes;
+  if (!cfg.piece_bytes && longest_slice * g.unit_bytes > 128 * 1024 + 2048) {
+    // equal passes of about 64 KiB (a short last pass costs as many hand-offs as a full one), on 256-byte boundaries
     const uint64_t target = (uint64_t)(64 * 1024) / g.unit_bytes;
-    const uint64_t passes = (longest_slice + target - 1) / target;
+    const uint64_t passes = (longest_slice - slack + target - 1) / target;
     piece_units = (longest_slice + passes - 1) / passes;
     piece_units = (piece_units + g.slice_grain - 1) / g.slice_grain * g.slice_grain;
   }

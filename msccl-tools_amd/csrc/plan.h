@@ -105,6 +105,7 @@ struct Hosted {
   uint32_t my_flag;
   uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
   uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
+  uint32_t clip;                   // bytes that the slice's last unit lacks (the chunk's last slice, when a chunk is no multiple of 16 bytes)
   int tb, slice;                   // for the watchdog's report only
 };
 
@@ -117,7 +118,7 @@ struct DevCtx {
   uint32_t left;   // units of the slice (what the first pass has in front of it)
   uint64_t off;    // byte offset of the slice inside every chunk
 };
-static_assert(sizeof(DevCtx) == 80, "five 16-byte loads fetch a context");
+static_assert(sizeof(DevCtx) == 88, "a context is fetched with six loads");
 
 struct Geometry {
   uint64_t chunk_units = 0;   // units (16-byte vectors or elements) per chunk
@@ -151,7 +152,8 @@ struct KernelParams {
   unsigned char* fifo;
   mscclx_status* host_status;   // pinned host memory
   unsigned long long* prof;     // per-workgroup tick counters of MSCCLX_PROFILE builds, else null
-  uint64_t chunk_units;
+  uint64_t chunk_units;         // units per chunk; the last one may be partial on the vector path
+  uint64_t chunk_bytes;         // rows of a rank buffer are this far apart
   uint64_t slice_fifo_units;
   uint64_t sync_slice_words;
   uint64_t sync_words;
@@ -170,6 +172,11 @@ struct KernelParams {
 #else
 #define MSCCLX_HOST_DEVICE
 #endif
+// The vector path moves 16-byte units.  A chunk need only be a multiple of 4 bytes for it: rows then start on
+// 4-byte boundaries (multi-dword accesses need no more), and the last unit of a chunk may be partial --
+// its buffer descriptor ends where the chunk ends, and dwords beyond a descriptor's end read as zero and
+// are not written (the range check of a raw buffer is per dword).  Anything else goes element by element.
+MSCCLX_HOST_DEVICE inline bool chunk_takes_vector_path(uint64_t chunk_bytes) { return chunk_bytes % 4 == 0; }
 // First unit of slice j of a chunk (j = slices: one past the chunk's last unit).  The chunk is dealt
 // out in groups of `grain` units (256 bytes where a chunk has at least one such group per slice, so
 // that no slice starts in the middle of a cache line; else 1); the last slice takes the remainder.

@@ -210,10 +210,44 @@ def test_ll_geometry_and_relaunch(knobs):
 @pytest.mark.parametrize("chunk_elems,dtype", [(1, "float32"), (3, "float32"), (4, "float32"), (1001, "float16"),
                                                (7, "uint8"), (16, "uint8"), (100003, "int32")])
 def test_ragged_chunk_sizes(chunk_elems, dtype):
-    """Chunks that are not a multiple of 16 bytes take the element path; tiny chunks leave most
-    slices empty-handed, so the geometry must shrink."""
+    """Chunks that are not a multiple of 4 bytes take the element path, multiples of 4 the vector path with
+    a partial last unit; tiny chunks leave most slices empty-handed, so the geometry must shrink."""
     got, want, _, info = run_both(ir_samples.ring_allreduce_xml(4), chunk_elems, dtype)
     assert_same(got, want)
+
+
+# chunk sizes in bytes that are a multiple of 4 but not of 16: the vector path with a partial last unit
+PARTIAL_UNIT_CASES = [(1001, "float32"), (1002, "float32"), (1003, "float32"), (5002, "bfloat16"), (1004, "uint8"), (1001, "float64"),
+                      (3, "int32"), (40001, "float32"), (524289, "int32")]
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("chunk_elems,dtype", PARTIAL_UNIT_CASES)
+def test_chunks_that_end_inside_a_unit(chunk_elems, dtype, mode):
+    """A chunk of 4k bytes that is no multiple of 16 moves in 16-byte units all the same: rows start on
+    4-byte boundaries and the last unit of every row is cut where the chunk ends.  Every byte of every
+    buffer is compared, so a store that ran past a chunk's end would show in the chunk behind it.
+    Ring (rrs/rrcs/rcs), all-pairs (folded nops, reduce chains as one step), multi-chunk steps."""
+    from msccl.executor import DTYPE_SIZES
+    assert (chunk_elems * DTYPE_SIZES[dtype]) % 4 == 0 and (chunk_elems * DTYPE_SIZES[dtype]) % 16 != 0
+    for xml in (ir_samples.ring_allreduce_xml(8, 2), ir_samples.allpairs_allreduce_xml(5), ir_samples.RRC_CPY_NOP_XML):
+        got, want, _, info = run_both(xml, chunk_elems, dtype, seed=chunk_elems % 97, **MODES[mode])
+        assert info.vector_path == 1
+        assert_same(got, want)
+
+
+@pytest.mark.parametrize("knobs", [dict(slices=1, piece_bytes=4096), dict(slices=3, piece_bytes=16 * 7, threads=128), dict(slices=2, workgroups=1, threads=64),
+                                   dict(slices=5, threads=512), dict(slices=16, threads=64), dict(slices=4, workgroups=3, threads=256)])
+@pytest.mark.parametrize("protocol", PROTOCOLS)
+def test_partial_units_under_explicit_geometries(knobs, protocol):
+    """The partial unit sits in the last pass of the last slice, whatever the passes, slices and hosting are;
+    on one-wave workgroups with one context each the chain loops move it."""
+    for xml, dtype in ((ir_samples.ring_allreduce_xml(8, 2), "float32"), (ir_samples.allpairs_allreduce_xml(5), "bfloat16"),
+                       (ir_samples.ring_allgather_xml(8, 2), "int32")):
+        elems = 10001 if dtype != "bfloat16" else 20002
+        got, want, _, info = run_both(xml, elems, dtype, seed=7, protocol=protocol, **knobs)
+        assert info.vector_path == 1 and info.slices == knobs["slices"]
+        assert_same(got, want)
 
 
 @pytest.mark.parametrize("knobs", [dict(), dict(slices=1, piece_bytes=4096), dict(threads=256, slices=2), dict(threads=64, slices=3)])
