@@ -171,7 +171,9 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
 /* Attaches device memory: in/out/scratch[r] are rank r's buffers of i/o/s_chunks * chunk_bytes
  * bytes (may be NULL where the extent is 0; in == out aliasing is the caller's choice, as with an
  * in-place NCCL call; buffers that overlap in memory need a plan configured with staging=1, else
- * MSCCLX_ERR_ALIASED).  Uploads the plan tables to the current device and clears the workspace.
+ * MSCCLX_ERR_ALIASED).  A buffer must start on a boundary of its element type, and on a 4-byte
+ * boundary where chunk_bytes is a multiple of 4 -- a view into a larger tensor is fine.
+ * Uploads the plan tables to the current device and clears the workspace.
  * Binding again after a launch has been waited for (new buffers, same geometry) re-uses the
  * device-side allocations: one upload of the tables, no allocation. */
 int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void* const* scratch,

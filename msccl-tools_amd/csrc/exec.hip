@@ -107,7 +107,8 @@ static int collect_buffers(const mscclx_plan& plan, void* const* in, void* const
       void* ptr = tables[b] ? tables[b][r] : nullptr;
       if (plan.rank_chunks[(size_t)r * 3 + b] > 0) {
         if (!ptr) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer " + "ios"[b] + " is used by the algorithm but NULL was given");
-        if (g.vector_path && (uintptr_t)ptr % 16) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffers must be 16-byte aligned");
+        // (rows of a buffer start on 4-byte boundaries anyway when chunks are no multiple of 16 bytes; the kernel lays its units out from the destination's lines)
+        if (g.vector_path && (uintptr_t)ptr % 4) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffers must be 4-byte aligned (chunks that are a multiple of 4 bytes move in 16-byte units)");
         if ((uintptr_t)ptr % dtype_size(plan.dtype)) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer not aligned to its element type");
       }
       bufs[(size_t)r * 3 + b] = ptr;

@@ -236,6 +236,36 @@ def test_chunks_that_end_inside_a_unit(chunk_elems, dtype, mode):
         assert_same(got, want)
 
 
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("first_elem,chunk_elems", [(1, 1000), (3, 1001), (2, 40004), (1, 131075)])
+def test_buffers_that_start_off_a_16_byte_boundary(first_elem, chunk_elems, mode):
+    """Rank buffers need only start on a 4-byte boundary -- a view into a larger tensor, say: the units are
+    laid out from the destination's cache lines, wherever the row starts.  The words around every
+    view must come through untouched."""
+    from msccl.executor import Executor
+    for xml in (ir_samples.ring_allreduce_xml(8, 2), ir_samples.allpairs_allreduce_xml(5)):
+        algo = oi.parse_xml(xml)
+        n, elems = algo.ngpus, algo.gpus[0].i_chunks * chunk_elems
+        x = make_inputs(n, elems, "float32", seed=first_elem + chunk_elems)
+        want = oc.place_inputs(algo, x, chunk_elems, "float32")
+        oi.Interpreter(algo).run(want, chunk_elems, "float32")
+        guard = np.float32(-12345.5)
+        whole = [torch.full((elems + 8,), float(guard), dtype=torch.float32, device="cuda:0") for _ in range(n)]
+        views = [w[first_elem:first_elem + elems] for w in whole]
+        for r in range(n):
+            views[r].copy_(torch.from_numpy(x[r]))
+        assert all(v.data_ptr() % 16 == 4 * first_elem for v in views)
+        ex = Executor(xml)
+        print(f"case: {algo.name} first_elem={first_elem} chunk_elems={chunk_elems} mode={mode}", flush=True)
+        ex.setup(chunk_elems * 4, "float32", **MODES[mode])
+        ex.run(views, [None] * n)
+        torch.cuda.synchronize()
+        for r in range(n):
+            got = whole[r].cpu().numpy()
+            assert np.array_equal(got[first_elem:first_elem + elems].view(np.uint32), want[r]["i"].view(np.uint32)), (algo.name, r)
+            assert (got[:first_elem] == guard).all() and (got[first_elem + elems:] == guard).all(), (algo.name, r, "guard words")
+
+
 @pytest.mark.parametrize("knobs", [dict(slices=1, piece_bytes=4096), dict(slices=3, piece_bytes=16 * 7, threads=128), dict(slices=2, workgroups=1, threads=64),
                                    dict(slices=5, threads=512), dict(slices=16, threads=64), dict(slices=4, workgroups=3, threads=256)])
 @pytest.mark.parametrize("protocol", PROTOCOLS)
