@@ -121,7 +121,7 @@ typedef struct {
   int32_t fifo_depth;
   int32_t passes;      /* passes of the step list the longest slice makes          */
   int32_t connections;
-  int32_t vector_path; /* 1: 16-byte units (chunk_bytes a multiple of 4), 0: element by element */
+  int32_t vector_path; /* always 1: every chunk size moves in 16-byte units            */
   int32_t zero_copy_messages; /* messages per pass read in place instead of staged  */
   int32_t staged_messages;
   int32_t max_hosted;  /* most contexts any workgroup hosts                         */
@@ -163,16 +163,16 @@ uint64_t mscclx_plan_algorithmic_units(const mscclx_plan* plan);
 
 /* Fixes the geometry for chunks of `chunk_bytes` bytes of `dtype` and reports it, including the
  * workspace the caller must provide.  Queries the current device unless cfg->max_workgroups > 0.
- * Any positive multiple of the element size is accepted; multiples of 4 bytes move in 16-byte units
- * (fastest when chunks start on cache lines: multiples of 256), the rest element by element. */
+ * Any positive multiple of the element size is accepted (fastest when chunks start on cache
+ * lines: multiples of 128 bytes). */
 int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, int32_t redop,
                           const mscclx_config* cfg, mscclx_info* info);
 
 /* Attaches device memory: in/out/scratch[r] are rank r's buffers of i/o/s_chunks * chunk_bytes
  * bytes (may be NULL where the extent is 0; in == out aliasing is the caller's choice, as with an
  * in-place NCCL call; buffers that overlap in memory need a plan configured with staging=1, else
- * MSCCLX_ERR_ALIASED).  A buffer must start on a boundary of its element type, and on a 4-byte
- * boundary where chunk_bytes is a multiple of 4 -- a view into a larger tensor is fine.
+ * MSCCLX_ERR_ALIASED).  A buffer must start on a boundary of its element type; a view into a
+ * larger tensor is fine.
  * Uploads the plan tables to the current device and clears the workspace.
  * Binding again after a launch has been waited for (new buffers, same geometry) re-uses the
  * device-side allocations: one upload of the tables, no allocation. */

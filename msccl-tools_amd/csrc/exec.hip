@@ -27,18 +27,18 @@ namespace mscclx {
 typedef void (*kernel_fn)(const KernelParams);
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
-kernel_fn pick_kernel_group_0(int dtype, int op, bool vec, bool ll, bool fold);
-kernel_fn pick_kernel_group_1(int dtype, int op, bool vec, bool ll, bool fold);
-kernel_fn pick_kernel_group_2(int dtype, int op, bool vec, bool ll, bool fold);
-kernel_fn pick_kernel_group_3(int dtype, int op, bool vec, bool ll, bool fold);
-kernel_fn pick_kernel_group_4(int dtype, int op, bool vec, bool ll, bool fold);
-static kernel_fn pick_kernel(int dtype, int op, bool vec, bool ll, bool fold) {
+kernel_fn pick_kernel_group_0(int dtype, int op, bool ll, bool fold);
+kernel_fn pick_kernel_group_1(int dtype, int op, bool ll, bool fold);
+kernel_fn pick_kernel_group_2(int dtype, int op, bool ll, bool fold);
+kernel_fn pick_kernel_group_3(int dtype, int op, bool ll, bool fold);
+kernel_fn pick_kernel_group_4(int dtype, int op, bool ll, bool fold);
+static kernel_fn pick_kernel(int dtype, int op, bool ll, bool fold) {
   switch (dtype / 2) {
-    case 0: return pick_kernel_group_0(dtype, op, vec, ll, fold);
-    case 1: return pick_kernel_group_1(dtype, op, vec, ll, fold);
-    case 2: return pick_kernel_group_2(dtype, op, vec, ll, fold);
-    case 3: return pick_kernel_group_3(dtype, op, vec, ll, fold);
-    case 4: return pick_kernel_group_4(dtype, op, vec, ll, fold);
+    case 0: return pick_kernel_group_0(dtype, op, ll, fold);
+    case 1: return pick_kernel_group_1(dtype, op, ll, fold);
+    case 2: return pick_kernel_group_2(dtype, op, ll, fold);
+    case 3: return pick_kernel_group_3(dtype, op, ll, fold);
+    case 4: return pick_kernel_group_4(dtype, op, ll, fold);
     default: return nullptr;
   }
 }
@@ -107,8 +107,6 @@ static int collect_buffers(const mscclx_plan& plan, void* const* in, void* const
       void* ptr = tables[b] ? tables[b][r] : nullptr;
       if (plan.rank_chunks[(size_t)r * 3 + b] > 0) {
         if (!ptr) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer " + "ios"[b] + " is used by the algorithm but NULL was given");
-        // (rows of a buffer start on 4-byte boundaries anyway when chunks are no multiple of 16 bytes; the kernel lays its units out from the destination's lines)
-        if (g.vector_path && (uintptr_t)ptr % 4) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffers must be 4-byte aligned (chunks that are a multiple of 4 bytes move in 16-byte units)");
         if ((uintptr_t)ptr % dtype_size(plan.dtype)) return fail(MSCCLX_ERR_INVALID_ARG, "rank " + std::to_string(r) + ": buffer not aligned to its element type");
       }
       bufs[(size_t)r * 3 + b] = ptr;
@@ -143,8 +141,8 @@ static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<
 static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bufs, DeviceImage* img) {
   const mscclx_plan* plan = &plan_ref;
   const Geometry& g = plan->geo;
-  const bool fold = g.vector_path && !g.ll && has_foldable_nops(*plan);
-  img->kernel = pick_kernel(plan->dtype, plan->redop, g.vector_path != 0, g.ll != 0, fold);
+  const bool fold = !g.ll && has_foldable_nops(*plan);
+  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold);
   if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   DeviceImage* d = img;
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
@@ -291,7 +289,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
   // One record per hosted context, in hosting order: where its counters and slots are, its slice's bounds.
   std::vector<DevCtx> ctxs(g.ctx_tb.size());
   {
-    const uint64_t ub = g.unit_bytes, fb = g.ll ? (uint64_t)kLLUnitBytes : ub, slot_step = g.vector_path ? 16 : 1;
+    const uint64_t ub = g.unit_bytes, fb = g.ll ? (uint64_t)kLLUnitBytes : ub, slot_step = 16;
     for (size_t k = 0; k < ctxs.size(); ++k) {
       const int32_t tbi = g.ctx_tb[k], slice = g.ctx_slice[k];
       const DevTb& tb = htb[(size_t)tbi];
@@ -447,19 +445,18 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   if (redop < 0 || redop >= MSCCLX_NUM_REDOPS) return fail(MSCCLX_ERR_INVALID_ARG, "unknown reduction");
   const int elem = dtype_size(dtype);
   if (chunk_bytes == 0 || chunk_bytes % elem) return fail(MSCCLX_ERR_INVALID_ARG, "chunk_bytes must be a positive multiple of the element size");
-  const bool vec = chunk_takes_vector_path(chunk_bytes);
   int num_cus = 256;
   int capacity[kThreadChoices];
   if (cfg.max_workgroups > 0) {
     for (int i = 0; i < kThreadChoices; ++i) capacity[i] = cfg.max_workgroups;
   } else {
-    const bool ll = cfg.protocol == MSCCLX_PROTO_LL && vec;  // (LL without the vector path is refused below)
-    const bool fold = vec && !ll && has_foldable_nops(*plan);
-    int rc = query_capacity(pick_kernel(dtype, redop, vec, ll, fold), &num_cus, capacity);
+    const bool ll = cfg.protocol == MSCCLX_PROTO_LL;
+    const bool fold = !ll && has_foldable_nops(*plan);
+    int rc = query_capacity(pick_kernel(dtype, redop, ll, fold), &num_cus, capacity);
     if (rc) return rc;
-    if (cfg.protocol == MSCCLX_PROTO_AUTO && vec && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
+    if (cfg.protocol == MSCCLX_PROTO_AUTO && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
       int other[kThreadChoices];
-      rc = query_capacity(pick_kernel(dtype, redop, true, true, false), &num_cus, other);
+      rc = query_capacity(pick_kernel(dtype, redop, true, false), &num_cus, other);
       if (rc) return rc;
       for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
     }

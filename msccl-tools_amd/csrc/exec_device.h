@@ -206,10 +206,43 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 #endif
 constexpr int kUnroll = MSCCLX_UNROLL;
 
+// The last 1 to 3 bytes of a row that is no whole number of dwords (chunks of 8- or 16-bit elements that are no
+// multiple of 4 bytes), moved element by element by the first lanes: out1[, out2] = a [(+) b].  In two halves, so
+// that the loads travel with the row's other loads and the stores with its other stores -- a round trip of its own
+// per row would show in every step of a latency-bound program.
+template <class R, bool HAS_B>
+struct SubDword {
+  static constexpr int E = R::kElemBytes < 4 ? R::kElemBytes : 1;  // (wider elements have no such rows; nothing below runs for them)
+  typedef Access<E> A;
+  typedef typename A::word word;
+  word x, y;
+  __device__ __forceinline__ void load(const unsigned char* a, const unsigned char* b, uint32_t bytes) {
+    if constexpr (R::kElemBytes < 4) {
+      const uint32_t i = threadIdx.x * E;
+      if (i < bytes) {
+        x = A::template ld<MSCCLX_AUX_LD>(make_rsrc(a, bytes), (int)i);
+        if (HAS_B) y = A::template ld<MSCCLX_AUX_LD>(make_rsrc(b, bytes), (int)i);
+      }
+    }
+  }
+  template <bool HAS_O2, bool NT1>
+  __device__ __forceinline__ void store(unsigned char* o1, unsigned char* o2, uint32_t bytes) {
+    if constexpr (R::kElemBytes < 4) {
+      const uint32_t i = threadIdx.x * E;
+      if (i < bytes) {
+        if (HAS_B) x = R::combine(y, x);
+        A::template st<NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST>(make_rsrc(o1, bytes), (int)i, x);
+        if (HAS_O2) A::template st<MSCCLX_AUX_ST>(make_rsrc(o2, bytes), (int)i, x);
+      }
+    }
+  }
+};
+
 // o1 = a [(+) b] over `bytes` bytes in units of W, UA units in flight per thread and operand: the loop of
 // move_units, for the part of a row that starts on a line of its destination.
-template <class R, int W, bool HAS_B, bool NT1, int UA>
+template <class R, bool HAS_B, bool NT1, int UA>
 __device__ __forceinline__ void move_units_body(unsigned char* o1, const unsigned char* a, const unsigned char* b, uint32_t bytes) {
+  constexpr int W = 16;
   typedef Access<W> A;
   typedef typename A::word word;
   constexpr int XL = MSCCLX_AUX_LD, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
@@ -230,14 +263,19 @@ __device__ __forceinline__ void move_units_body(unsigned char* o1, const unsigne
   }
 }
 
-// out1[, out2] = a [(+) b] over n units of W bytes, the last of which lacks `clip` bytes (the end of a chunk that is
-// no multiple of 16 bytes: the descriptors end there, so the missing dwords read as zero and are not written).
-template <class R, int W, bool HAS_B, bool HAS_O2, bool NT1>
+// out1[, out2] = a [(+) b] over n units of 16 bytes, the last of which lacks `clip` bytes (the end of a chunk that is
+// no multiple of 16 bytes: the descriptors end there, so the missing dwords read as zero and are not written --
+// the range check is per dword, so descriptors end on whole dwords and what is left of the row, 1 to 3 bytes when a
+// chunk is no multiple of 4, goes element by element).
+template <class R, bool HAS_B, bool HAS_O2, bool NT1>
 __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2, const unsigned char* a, const unsigned char* b, uint32_t n, uint32_t clip) {
+  constexpr int W = 16;
   typedef Access<W> A;
   typedef typename A::word word;
   constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-  const uint32_t bytes = n * W - clip;
+  const uint32_t total = n * W - clip;                       // the row's bytes
+  const uint32_t bytes = total & ~3u;                        // what whole dwords cover, counted from the row's start
+  const uint32_t odd = total - bytes;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, bytes), r1 = make_rsrc(o1, bytes);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, bytes), r2 = make_rsrc(HAS_O2 ? o2 : o1, bytes);
   const uint32_t T = blockDim.x;
@@ -246,17 +284,20 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
     // needs in flight would only be instructions in the way here (measured: 4 % of a 64-rank ring
     // all-reduce on 512-byte pieces).
     const uint32_t i = threadIdx.x;
+    SubDword<R, HAS_B> tail;
+    if (odd) tail.load(a + bytes, HAS_B ? b + bytes : nullptr, odd);
     if (i < n) {
       word x = A::template ld<XL>(ra, (int)(i * W));
       if (HAS_B) x = R::combine(A::template ld<XL>(rb, (int)(i * W)), x);
       A::template st<X1>(r1, (int)(i * W), x);
       if (HAS_O2) A::template st<XS>(r2, (int)(i * W), x);
     }
+    if (odd) tail.template store<HAS_O2, NT1>(o1 + bytes, HAS_O2 ? o2 + bytes : nullptr, odd);
     return;
   }
   // kUnroll loads are in flight per thread either way: all of a, or half of a and half of b
   constexpr int UA = HAS_B ? (kUnroll / 2 > 0 ? kUnroll / 2 : 1) : kUnroll;
-  if (W == 16 && !HAS_O2) {
+  if (!HAS_O2) {
     // A destination that does not start on a 128-byte line (chunks that are no multiple of 128 bytes) costs a
     // sixth of the memory system's rate when every wave's kilobyte of stores straddles nine lines instead of
     // covering eight; where the source starts does not matter (measured with a plain streaming kernel:
@@ -265,18 +306,28 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
     // at that boundary, and the head in front of it -- at most 8 units, the last one cut by descriptors that
     // end where the body begins -- by the first lanes, loaded here and stored after the body.
     const uint32_t head = (128u - ((uint32_t)(uintptr_t)o1 & 127u)) & 127u;
-    if (head != 0 && head < bytes) {
-      const __amdgpu_buffer_rsrc_t hra = make_rsrc(a, head), hr1 = make_rsrc(o1, head), hrb = make_rsrc(HAS_B ? b : a, head);
+    if (head != 0 && head < total) {
+      // (head and body each count their dwords from their own start: a row that starts on an odd 2-byte
+      // boundary has a head of 4k + 2 bytes, and the body's dwords then sit on the destination's)
+      const uint32_t hv = head & ~3u, hodd = head - hv, body = (total - head) & ~3u, bodd = total - head - body;
+      const __amdgpu_buffer_rsrc_t hra = make_rsrc(a, hv), hr1 = make_rsrc(o1, hv), hrb = make_rsrc(HAS_B ? b : a, hv);
       const uint32_t h = threadIdx.x * W;
-      word hx = A::template ld<XL>(hra, (int)(h < head ? h : 0x7ffffff0u));
+      word hx = A::template ld<XL>(hra, (int)(h < hv ? h : 0x7ffffff0u));
       word hy = hx;
-      if (HAS_B) hy = A::template ld<XL>(hrb, (int)(h < head ? h : 0x7ffffff0u));
-      move_units_body<R, W, HAS_B, NT1, UA>(o1 + head, a + head, HAS_B ? b + head : nullptr, bytes - head);
+      if (HAS_B) hy = A::template ld<XL>(hrb, (int)(h < hv ? h : 0x7ffffff0u));
+      SubDword<R, HAS_B> head_tail, body_tail;
+      if (hodd) head_tail.load(a + hv, HAS_B ? b + hv : nullptr, hodd);
+      if (bodd) body_tail.load(a + head + body, HAS_B ? b + head + body : nullptr, bodd);
+      move_units_body<R, HAS_B, NT1, UA>(o1 + head, a + head, HAS_B ? b + head : nullptr, body);
       if (HAS_B) hx = R::combine(hy, hx);
-      if (h < head) A::template st<X1>(hr1, (int)h, hx);
+      if (h < hv) A::template st<X1>(hr1, (int)h, hx);
+      if (hodd) head_tail.template store<false, NT1>(o1 + hv, nullptr, hodd);
+      if (bodd) body_tail.template store<false, NT1>(o1 + head + body, nullptr, bodd);
       return;
     }
   }
+  SubDword<R, HAS_B> tail;
+  if (odd) tail.load(a + bytes, HAS_B ? b + bytes : nullptr, odd);
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
     word x[UA], y[UA];
 #pragma unroll
@@ -294,16 +345,17 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
       for (int u = 0; u < UA; ++u) A::template st<XS>(r2, (int)((i + u * T) * W), x[u]);
     }
   }
+  if (odd) tail.template store<HAS_O2, NT1>(o1 + bytes, HAS_O2 ? o2 + bytes : nullptr, odd);
 }
 
 // rows x n units.  Consecutive rows of an operand are `stride_*` BYTES apart: a chunk for rank
 // buffers, n units for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
 // buffer, o2 (the forwarded copy) always a FIFO slot.  clip: see move_units.
-template <class R, bool VEC, bool HAS_B, bool HAS_O2, bool NT1 = false>
+template <class R, bool HAS_B, bool HAS_O2, bool NT1 = false>
 __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
                                           const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t clip) {
-  constexpr int W = VEC ? 16 : R::kElemBytes;
-  if (!HAS_B && !HAS_O2 && __builtin_expect(rows > 1 && n <= blockDim.x, 0)) {  // (plain copies only: the scatter and gather steps of all-pairs and all-to-all programs)
+  constexpr int W = 16;
+  if (!HAS_B && !HAS_O2 && __builtin_expect(rows > 1 && n <= blockDim.x && ((n * W - clip) & 3u) == 0, 0)) {  // (plain copies only: the scatter and gather steps of all-pairs and all-to-all programs)
     // Several short rows (a multi-chunk step of a latency-bound program): one unit per thread and
     // row.  Four rows are loaded before the first is stored -- row by row, every row would wait
     // for its own round trip to memory.
@@ -337,7 +389,7 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
     return;
   }
   for (int r = 0; r < rows; ++r)
-    move_units<R, W, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
+    move_units<R, HAS_B, HAS_O2, NT1>(o1 + (uint64_t)r * stride_o1, HAS_O2 ? o2 + (uint64_t)r * n * W : nullptr,
                                     a + (uint64_t)r * stride_a, HAS_B ? b + (uint64_t)r * stride_b : nullptr, n, clip);
 }
 
@@ -534,7 +586,7 @@ enum {
   kAPacked = 16, // a is a slot
   kToSlot = 32,  // the first (only) destination is `out` instead of dst
   kMany = 64,    // dst = ((dst (+) a[0]) (+) a[1]) ...: `rows` sources, `out` bytes apart
-  kClipShift = 8, kClipMask = 3 << 8,  // bits 8-9: dwords that the last unit of a rank-buffer row lacks (see move_units)
+  kClipShift = 8, kClipMask = 15 << 8,  // bits 8-11: bytes that the last unit of a rank-buffer row lacks (see move_units)
 };
 enum { kLLSend = 0, kLLRecv, kLLRecvNt, kLLRcs, kLLRrc, kLLRrs, kLLRrcs };
 
@@ -592,7 +644,7 @@ __device__ __forceinline__ void mark_many_sources(Context& c, const DevOp& op) {
 // where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
 // last 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order,
 // so this is a hint that the message is about to be complete; the threads that read it check every line.
-template <bool VEC, bool LL>
+template <bool LL>
 __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const KernelParams& p, uint32_t epoch, const DevOp& op) {
   const int t = (int)(op.word & 15u);
   const int cnt = (int)(op.word >> kOpCntShift);
@@ -609,14 +661,14 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
 
   const uint32_t n = c.left < p.piece_units ? c.left : p.piece_units;
   // out: the slot to fill, or 0 when the receiver will read this step's payload in place
-  const u64 out = (snd && out_staged) ? (u64)p.fifo + (u64)h.out_slots * (VEC ? 16 : 1) + c.sslot : 0;
+  const u64 out = (snd && out_staged) ? (u64)p.fifo + (u64)h.out_slots * 16 + c.sslot : 0;
   // in: the incoming payload -- packed in a slot, or still where the sender has it (then its rows are
   // a chunk apart, like any rank buffer)
   u64 in = 0;
   int in_packed = kAPacked;
   if (rcv) {
     if (in_place) { in = op.in_addr + c.off; in_packed = 0; }
-    else in = (u64)p.fifo + (u64)h.in_slots * (VEC ? 16 : 1) + c.rslot;
+    else in = (u64)p.fifo + (u64)h.in_slots * 16 + c.rslot;
     if (LL) {
       c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
       c.t1 = ll_flag(epoch, c.rseq);
@@ -642,7 +694,7 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     default: break;
   }
   // the pass that reaches the end of the slice: its rows may end inside their last unit
-  m.kind = kind | (c.left <= p.piece_units ? (int)(h.clip >> 2) << kClipShift : 0);
+  m.kind = kind | (c.left <= p.piece_units ? (int)h.clip << kClipShift : 0);
 }
 
 // The description of the step after the one `c` stands at.  It is fetched before the counters of
@@ -656,7 +708,7 @@ __device__ __forceinline__ DevOp fetch_next_op(const Context& c, const Hosted& h
 // Announce the completed step and move the context to its next one, described by `next`.
 // `writer`: this thread stores the counters (the context's lane; one thread of a wave that runs a
 // context with all its lanes).
-template <int UB, bool LL>
+template <bool LL>
 __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next, bool writer = true) {
   const Hosted h = entry;  // one batch of LDS reads, one wait -- not one wait per field as they are needed
   if (is_send(c.type)) {
@@ -677,16 +729,16 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
     c.step = 0;
     ++c.pass;
     c.left -= c.left < p.piece_units ? c.left : p.piece_units;
-    c.off += (u64)p.piece_units * UB;
+    c.off += (u64)p.piece_units * 16;
   }
   if (c.pass >= h.npasses) c.active = false;
-  else describe_step<UB == 16, LL>(c, h, p, epoch, next);
+  else describe_step<LL>(c, h, p, epoch, next);
 }
 
 // Set up hosted context number `ctx`: its constants in `h` (the record worked out when the buffers were
 // bound), its state in `c`, standing at its first step.  `writer` also clears, for the next launch,
 // the counters this context alone writes.
-template <bool VEC, int EB, bool LL>
+template <bool LL>
 __device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int ctx, bool writer) {
   const DevCtx rec = p.ctxs[ctx];
   h = rec.h;
@@ -699,24 +751,31 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
     if (h.head_out) p.sync_nxt[h.head_out] = 0;
     if (h.tail_out) p.sync_nxt[h.tail_out] = 0;
   }
-  if (c.active) describe_step<VEC, LL>(c, h, p, epoch, p.ops[h.op_begin]);
+  if (c.active) describe_step<LL>(c, h, p, epoch, p.ops[h.op_begin]);
 }
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
 // incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool VEC, bool LL, bool FOLD = false>
+template <class R, bool LL, bool FOLD = false>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
-  constexpr int W = VEC ? 16 : R::kElemBytes;
+  constexpr int W = 16;
   const u64 cs = p.chunk_bytes;                   // rows of a rank buffer are a chunk apart ...
   const u64 packed = (u64)m.n * W;                // ... rows in a slot are packed
-  const uint32_t clip = (((uint32_t)m.kind & kClipMask) >> kClipShift) * 4u;
+  const uint32_t clip = ((uint32_t)m.kind & kClipMask) >> kClipShift;
   unsigned char* const dst = (unsigned char*)m.dst;
   unsigned char* const out = (unsigned char*)m.out;
   const unsigned char* const a = (const unsigned char*)m.a;
   if (FOLD && __builtin_expect((m.kind & kMany) != 0, 0)) {  // (only the bind of a FOLD kernel makes such steps)
-    if (m.kind & kNt1) move_reduce_many<R, W, true>(dst, a, (uint32_t)m.out, m.rows, m.n, clip);
-    else move_reduce_many<R, W, false>(dst, a, (uint32_t)m.out, m.rows, m.n, clip);
+    // (whole dwords in 16-byte units; what is left of a row that is no whole number of dwords, element by element)
+    const uint32_t total = m.n * W - clip, odd = total & 3u;
+    if (m.kind & kNt1) move_reduce_many<R, W, true>(dst, a, (uint32_t)m.out, m.rows, m.n, clip + odd);
+    else move_reduce_many<R, W, false>(dst, a, (uint32_t)m.out, m.rows, m.n, clip + odd);
+    if (odd) {
+      constexpr int E = R::kElemBytes;
+      if (m.kind & kNt1) move_reduce_many<R, E, true>(dst + (total - odd), a + (total - odd), (uint32_t)m.out, m.rows, odd / E, 0);
+      else move_reduce_many<R, E, false>(dst + (total - odd), a + (total - odd), (uint32_t)m.out, m.rows, odd / E, 0);
+    }
     return;
   }
   if (LL && (m.kind & kLLKind)) {
@@ -737,11 +796,11 @@ __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, ui
     unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
     const u64 stride_o1 = (m.kind & kToSlot) ? packed : cs;
     switch (m.kind & 7) {
-      case 0: move_rows<R, VEC, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
-      case kNt1: move_rows<R, VEC, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
-      case kHasO2: move_rows<R, VEC, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
-      case kHasB: move_rows<R, VEC, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n, clip); break;
-      case kHasB | kHasO2: move_rows<R, VEC, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n, clip); break;
+      case 0: move_rows<R, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kNt1: move_rows<R, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kHasO2: move_rows<R, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kHasB: move_rows<R, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n, clip); break;
+      case kHasB | kHasO2: move_rows<R, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n, clip); break;
       default: break;
     }
   }
@@ -931,7 +990,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<true, R::kElemBytes, true>(h, first, p, epoch, ctx, writer);
+    init_context<true>(h, first, p, epoch, ctx, writer);
     if (!first.active) return;
     left = uniform(first.left);
     off = uniform((uint64_t)first.off);
@@ -1090,7 +1149,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<true, R::kElemBytes, false>(h, first, p, 0, ctx, writer);
+    init_context<false>(h, first, p, 0, ctx, writer);
     if (!first.active) return;
     left = uniform(first.left);
     off = uniform((uint64_t)first.off);
@@ -1158,15 +1217,31 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       u64 a_row = rcv ? (in_place ? op.in_addr + off : (u64)(in_ring + rslot)) : op.src_addr + off;
       const u64 a_stride = (rcv && !in_place) ? (u64)n * 16 : row_stride;
       u64 local_row = op.dst_addr + off, slot_row = (u64)(out_ring + sslot);
-      const uint32_t row_bytes = n * 16 - (left <= piece ? end_clip : 0u);  // (slot rows are n units apart, and end where their rank-buffer rows do)
+      const uint32_t row_total = n * 16 - (left <= piece ? end_clip : 0u);  // (slot rows are n units apart, and end where their rank-buffer rows do)
+      const uint32_t row_bytes = row_total & ~3u, odd = row_total - row_bytes;  // whole dwords; then 1 to 3 bytes, element by element (see move_units)
       for (uint32_t row = 0; row < cnt; ++row) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc((const void*)a_row, row_bytes), rlocal = make_rsrc((const void*)local_row, row_bytes);
         const __amdgpu_buffer_rsrc_t rslot_out = make_rsrc((const void*)slot_row, row_bytes);
+        typedef Access<(R::kElemBytes < 4 ? R::kElemBytes : 1)> AE;
+        typename AE::word tail_x{}, tail_y{};
+        if constexpr (R::kElemBytes < 4) {
+          if (odd && lane * R::kElemBytes < odd) {
+            tail_x = AE::template ld<MSCCLX_AUX_LD>(make_rsrc((const void*)(a_row + row_bytes), odd), (int)(lane * R::kElemBytes));
+            if (has_b) tail_y = AE::template ld<MSCCLX_AUX_LD>(make_rsrc((const void*)(local_row + row_bytes), odd), (int)(lane * R::kElemBytes));
+          }
+        }
         if (n <= 64) chain_copy_round<R, 1>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else if (n <= 128) chain_copy_round<R, 2>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else if (n <= 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else  // (eight loads in flight per lane and operand, as the workgroup-wide mover has)
           for (uint32_t base = 0; base < n; base += 512) chain_copy_round<R, 8>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
+        if constexpr (R::kElemBytes < 4) {
+          if (odd && lane * R::kElemBytes < odd) {
+            if (has_b) tail_x = R::combine(tail_y, tail_x);
+            if (to_local) AE::template st<MSCCLX_AUX_ST>(make_rsrc((const void*)(local_row + row_bytes), odd), (int)(lane * R::kElemBytes), tail_x);
+            if (to_slot) AE::template st<MSCCLX_AUX_ST>(make_rsrc((const void*)(slot_row + row_bytes), odd), (int)(lane * R::kElemBytes), tail_x);
+          }
+        }
         a_row += a_stride; local_row += row_stride; slot_row += (u64)n * 16;
       }
       MSCCLX_CHAIN_CLOCK(prof_issued);
@@ -1209,11 +1284,8 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
 // share the resident workgroups without deadlock.
 // FOLD: steps may carry the dependencies of nop steps folded into them (a kernel of its own, so that
 // programs without such steps do not pay for the check in the poll loop).
-template <class R, bool VEC, bool LL, bool FOLD = false>
+template <class R, bool LL, bool FOLD = false>
 __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
-  static_assert(VEC || !LL, "LL lines carry 16-byte units");
-  constexpr int EB = R::kElemBytes;
-  constexpr uint64_t UB = VEC ? 16 : EB;
   // The number of launches so far is kept on the device (control word 0) and is advanced by the
   // last workgroup to finish, so a launch carries no host-side state and the same launch can be
   // replayed (stream order guarantees the next launch sees the new value).  Its lowest bit picks
@@ -1248,26 +1320,26 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
   const u64 prof_start = wall_clock64();
 #endif
   if (threadIdx.x == 0 && blockIdx.x == 0) p.sync_nxt[0] = 0;
-  if (LL && hosted == 1 && blockDim.x == 64) {
+  if (LL && hosted == 1 && blockDim.x == 64) {  // (LL is configured only for chunks of whole dwords)
 #ifdef MSCCLX_PROFILE
     u64 chain_acc[5] = {0, 0, 0, 0, 0};
-    if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin, chain_acc);
+    if constexpr (LL) run_chain<R>(p, epoch, ctx_begin, chain_acc);
     prof_fin = chain_acc[0]; prof_wait = chain_acc[1]; prof_move = chain_acc[2]; prof_ack = chain_acc[3];
     if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
 #else
-    if constexpr (LL && VEC) run_chain<R>(p, epoch, ctx_begin);
+    if constexpr (LL) run_chain<R>(p, epoch, ctx_begin);
 #endif
-  } else if (!LL && !FOLD && VEC && hosted == 1 && blockDim.x == 64) {
+  } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64) {
 #ifdef MSCCLX_PROFILE
     u64 chain_acc[5] = {0, 0, 0, 0, 0};
-    if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin, chain_acc);
+    if constexpr (!LL && !FOLD) run_chain_counters<R>(p, ctx_begin, chain_acc);
     prof_wait = chain_acc[0]; prof_move = chain_acc[1]; prof_ack = chain_acc[2]; prof_fin = chain_acc[3];
     if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
 #else
-    if constexpr (!LL && !FOLD && VEC) run_chain_counters<R>(p, ctx_begin);
+    if constexpr (!LL && !FOLD) run_chain_counters<R>(p, ctx_begin);
 #endif
   } else {
-  if (poller && lane < hosted) init_context<VEC, EB, LL>(h, c, p, epoch, ctx_begin + lane, true);
+  if (poller && lane < hosted) init_context<LL>(h, c, p, epoch, ctx_begin + lane, true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
   int cursor = 0;
   unsigned busy_rounds = 0;
@@ -1302,7 +1374,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
           const DevOp next = fetch_next_op(c, h, p);
-          finish_step<(int)UB, LL>(c, h, p, epoch, next);
+          finish_step<LL>(c, h, p, epoch, next);
           if (FOLD && c.active) mark_many_sources(c, next);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
@@ -1387,7 +1459,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
 
     // ---- the chosen context's step: move one piece ----
-    do_move<R, VEC, LL, FOLD>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
+    do_move<R, LL, FOLD>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
 #endif
@@ -1403,7 +1475,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     const u64 prof_t3 = wall_clock64();
 #endif
     if (mine) {
-      finish_step<(int)UB, LL>(c, h, p, epoch, next);
+      finish_step<LL>(c, h, p, epoch, next);
       if (FOLD && c.active) mark_many_sources(c, next);
     }
 #ifdef MSCCLX_PROFILE
@@ -1456,17 +1528,17 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
 
-template <int DT, int OP> kernel_fn pick_vec(bool vec, bool ll, bool fold) {
-  if (ll) return vec && !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, true> : nullptr;
-  if (fold) return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false, true> : nullptr;
-  return vec ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false> : (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false>;
+template <int DT, int OP> kernel_fn pick_variant(bool ll, bool fold) {
+  if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true> : nullptr;
+  if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, true>;
+  return (kernel_fn)exec_kernel<Reducer<DT, OP>, false>;
 }
-template <int DT> kernel_fn pick_op(int op, bool vec, bool ll, bool fold) {
+template <int DT> kernel_fn pick_op(int op, bool ll, bool fold) {
   switch (op) {
-    case MSCCLX_SUM: return pick_vec<DT, MSCCLX_SUM>(vec, ll, fold);
-    case MSCCLX_PROD: return pick_vec<DT, MSCCLX_PROD>(vec, ll, fold);
-    case MSCCLX_MAX: return pick_vec<DT, MSCCLX_MAX>(vec, ll, fold);
-    case MSCCLX_MIN: return pick_vec<DT, MSCCLX_MIN>(vec, ll, fold);
+    case MSCCLX_SUM: return pick_variant<DT, MSCCLX_SUM>(ll, fold);
+    case MSCCLX_PROD: return pick_variant<DT, MSCCLX_PROD>(ll, fold);
+    case MSCCLX_MAX: return pick_variant<DT, MSCCLX_MAX>(ll, fold);
+    case MSCCLX_MIN: return pick_variant<DT, MSCCLX_MIN>(ll, fold);
     default: return nullptr;
   }
 }

@@ -470,11 +470,13 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   if (cfg.slices < 0 || cfg.piece_bytes < 0 || cfg.fifo_depth < 0 || cfg.workgroups < 0 || cfg.threads < 0)
     return fail(MSCCLX_ERR_INVALID_ARG, "geometry knobs must be >= 0");
   Geometry g;
-  g.vector_path = chunk_takes_vector_path(chunk_bytes) ? 1 : 0;
-  g.unit_bytes = g.vector_path ? 16 : elem;
-  g.chunk_units = (chunk_bytes + g.unit_bytes - 1) / g.unit_bytes;  // (the vector path's last unit may be partial)
+  // Every chunk moves in 16-byte units, whatever its size: rows start wherever their chunk starts (multi-dword
+  // accesses need no alignment), the last unit of a chunk may be partial -- down to a single byte.
+  g.vector_path = 1;
+  g.unit_bytes = 16;
+  g.chunk_units = (chunk_bytes + g.unit_bytes - 1) / g.unit_bytes;
   if (cfg.protocol < 0 || cfg.protocol > MSCCLX_PROTO_LL) return fail(MSCCLX_ERR_INVALID_ARG, "unknown protocol");
-  if (cfg.protocol == MSCCLX_PROTO_LL && !g.vector_path) return fail(MSCCLX_ERR_UNSUPPORTED, "the LL protocol needs chunks that are a multiple of 4 bytes");
+  if (cfg.protocol == MSCCLX_PROTO_LL && chunk_bytes % 4) return fail(MSCCLX_ERR_UNSUPPORTED, "the LL protocol needs chunks that are a multiple of 4 bytes");
   g.staging = cfg.staging ? 1 : 0;
   const int64_t ntbs = (int64_t)plan.tbs.size();
   if (ntbs == 0) return fail(MSCCLX_ERR_BAD_IR, "the algorithm has no threadblocks");
@@ -594,7 +596,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // pipelined all-pairs 33 -> 23 us), within 2 % for the rest.  Bigger chunks lose as often as they win, and
       // a ring whose every threadblock is busy all the time (64 ranks) loses beyond one context per SIMD.
       // Chunks of up to 128 KiB too where ALL contexts are at most one per SIMD (8-rank ring on 1 MiB: 33.3 -> 31.5 us).
-      if (g.vector_path && chunk_bytes <= 128 * 1024 && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups) {
+      if (chunk_bytes <= 128 * 1024 && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups) {
         const double busy_share = chunk_bytes <= 64 * 1024 ? ratio : 1.0;
         int64_t fine = 1;
         while ((uint64_t)fine * 1024 < chunk_bytes) fine *= 2;  // pieces of at most 1 KiB
@@ -615,7 +617,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // message cost more than the hand-off saves (8-rank ring on 1 MiB: 38 us either way; on 2 MiB
       // 59 against 40 us).  Programs whose nops can be folded keep the counters: folding, and chains
       // of local reduces done as one step, are worth more there.  Only when every knob is automatic.
-      if (cfg.protocol == MSCCLX_PROTO_AUTO && g.vector_path && !cfg.staging && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups &&
+      if (cfg.protocol == MSCCLX_PROTO_AUTO && chunk_bytes % 4 == 0 && !cfg.staging && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups &&
           depth_of_dataflow >= 8 && !has_foldable_nops(plan)) {
         int64_t s = slices;
         while (chunk_bytes / (uint64_t)s > 1024 && s * 2 * ntbs <= 2 * (int64_t)num_cus && (uint64_t)(s * 2) <= g.chunk_units) s *= 2;
@@ -761,7 +763,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.fifo_byte_off = sync_bytes;
   {  // the kernel keeps slot positions as 32-bit offsets (16-byte steps on the vector path, bytes otherwise) and counter positions as 32-bit word indices
     const uint64_t fifo_bytes = g.slice_fifo_units * g.slices * fifo_unit_bytes;
-    if (fifo_bytes >= (g.vector_path ? (1ull << 36) : (1ull << 32)) || g.sync_words >= (1ull << 31))
+    if (fifo_bytes >= (1ull << 36) || g.sync_words >= (1ull << 31))
       return fail(MSCCLX_ERR_CAPACITY, "the FIFO slots or counters of this geometry exceed what the kernel can address; use fewer slices or a smaller piece_bytes");
   }
   g.workspace_bytes = sync_bytes + g.slice_fifo_units * g.slices * fifo_unit_bytes + 256;

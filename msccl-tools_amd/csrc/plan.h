@@ -105,7 +105,7 @@ struct Hosted {
   uint32_t my_flag;
   uint32_t head_out, tail_in;      // outgoing connection: the head this context advances, the tail it watches
   uint32_t head_in, tail_out;      // incoming connection: the head it watches, the tail it advances
-  uint32_t clip;                   // bytes that the slice's last unit lacks (the chunk's last slice, when a chunk is no multiple of 16 bytes)
+  uint32_t clip;                   // bytes (0 to 15) that the slice's last unit lacks: the chunk's last slice, when a chunk is no multiple of 16 bytes
   int tb, slice;                   // for the watchdog's report only
 };
 
@@ -124,7 +124,7 @@ struct Geometry {
   uint64_t chunk_units = 0;   // units (16-byte vectors or elements) per chunk
   uint32_t unit_bytes = 0;
   uint32_t piece_units = 0;
-  int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;
+  int32_t slices = 0, depth = 0, threads = 0, vector_path = 0;  // (vector_path: always 1, reported for callers of older versions)
   uint32_t slice_grain = 1;       // see slice_begin()
   int32_t staging = 0;            // 1: every message goes through a FIFO slot
   int32_t ll = 0;                 // 1: flag-in-data lines in the slots (implies staging); FIFO bytes double
@@ -172,11 +172,6 @@ struct KernelParams {
 #else
 #define MSCCLX_HOST_DEVICE
 #endif
-// The vector path moves 16-byte units.  A chunk need only be a multiple of 4 bytes for it: rows then start on
-// 4-byte boundaries (multi-dword accesses need no more), and the last unit of a chunk may be partial --
-// its buffer descriptor ends where the chunk ends, and dwords beyond a descriptor's end read as zero and
-// are not written (the range check of a raw buffer is per dword).  Anything else goes element by element.
-MSCCLX_HOST_DEVICE inline bool chunk_takes_vector_path(uint64_t chunk_bytes) { return chunk_bytes % 4 == 0; }
 // First unit of slice j of a chunk (j = slices: one past the chunk's last unit).  The chunk is dealt
 // out in groups of `grain` units (256 bytes where a chunk has at least one such group per slice, so
 // that no slice starts in the middle of a cache line; else 1); the last slice takes the remainder.

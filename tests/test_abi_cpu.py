@@ -125,14 +125,14 @@ def test_geometry_without_a_device(mscclx_lib):
     # explicit knobs
     k = p.configure(8 << 20, "int32", max_workgroups=2048, slices=16, piece_bytes=65536, fifo_depth=4, threads=256, workgroups=128)
     assert (k.slices, k.piece_bytes, k.passes, k.fifo_depth, k.threads, k.workgroups, k.max_hosted) == (16, 65536, 8, 4, 256, 128, 4)
-    # the vector path takes any multiple of 4 bytes (the chunk's last 16-byte unit is then partial) ...
+    # every chunk size moves in 16-byte units (the chunk's last unit may be partial, down to a single byte)
     info = p.configure(1000 * 4 + 4, "int32", max_workgroups=2048)
     assert info.vector_path == 1 and info.slices == 8   # tiny chunks: one slice per XCD
     assert p.configure(4, "int32", max_workgroups=2048).vector_path == 1
-    # ... anything else goes element by element
     q = Plan(parse_algo_xml(ir_samples.ring_allgather_xml(8, 4)))
-    assert q.configure(1002, "float16", max_workgroups=2048).vector_path == 0
-    assert q.configure(1001, "uint8", max_workgroups=2048).vector_path == 0
+    assert q.configure(1002, "float16", max_workgroups=2048).vector_path == 1
+    assert q.configure(1001, "uint8", max_workgroups=2048).vector_path == 1
+    assert q.configure(1, "uint8", max_workgroups=2048).vector_path == 1
     with pytest.raises(MscclxError):
         p.configure(6, "int32", max_workgroups=2048)              # not a multiple of the element
     # more threadblocks than workgroups is fine: a workgroup hosts up to 64 contexts ...
@@ -202,7 +202,7 @@ def test_protocol_choice(mscclx_lib):
     assert b.workspace_bytes - slots == a.workspace_bytes - 2 * slots  # what is left are the counters
     assert p.configure(1000 * 4 + 4, "int32", max_workgroups=2048, protocol="ll").protocol == binding.PROTOCOL_CODES["ll"]  # (a partial last unit travels as a whole line)
     with pytest.raises(MscclxError) as e:
-        p.configure(1002, "float16", max_workgroups=2048, protocol="ll")  # lines carry 16-byte units: the vector path only
+        p.configure(1002, "float16", max_workgroups=2048, protocol="ll")  # lines carry whole dwords
     assert e.value.code == binding.ERR_UNSUPPORTED
     with pytest.raises(MscclxError) as e:
         p.configure(64 << 10, "float32", max_workgroups=2048, protocol=7)

@@ -236,6 +236,38 @@ def test_chunks_that_end_inside_a_unit(chunk_elems, dtype, mode):
         assert_same(got, want)
 
 
+# chunk sizes that are no multiple of 4 bytes: rows start on odd 2-byte or 1-byte boundaries and end inside a dword
+SUB_DWORD_CASES = [(1001, "float16"), (5001, "bfloat16"), (1003, "uint8"), (1001, "int8"), (1, "uint8"), (3, "bfloat16"), (40001, "float16"),
+                   (262145, "bfloat16"), (1048579, "uint8")]
+
+
+@pytest.mark.parametrize("mode", ["in-place", "staged"])
+@pytest.mark.parametrize("chunk_elems,dtype", SUB_DWORD_CASES)
+def test_chunks_that_end_inside_a_dword(chunk_elems, dtype, mode):
+    """Chunks of 8- or 16-bit elements that are no multiple of 4 bytes move in 16-byte units too: whole dwords
+    through descriptors that end with the row's last whole dword, the 1 to 3 bytes beyond it element by
+    element -- at the row's end and, where a long row is moved from its destination's first cache line on,
+    at the end of the head in front of that line.  (Flag-in-data lines carry whole dwords: refused.)"""
+    from msccl.executor import DTYPE_SIZES, Executor, MscclxError
+    assert (chunk_elems * DTYPE_SIZES[dtype]) % 4 != 0
+    for xml in (ir_samples.ring_allreduce_xml(8, 2), ir_samples.allpairs_allreduce_xml(5), ir_samples.RRC_CPY_NOP_XML, ir_samples.ring_allgather_xml(8, 2)):
+        got, want, _, info = run_both(xml, chunk_elems, dtype, seed=chunk_elems % 89, **MODES[mode])
+        assert info.vector_path == 1
+        assert_same(got, want)
+    with pytest.raises(MscclxError):
+        Executor(ir_samples.ring_allreduce_xml(8, 2)).setup(chunk_elems * DTYPE_SIZES[dtype], dtype, protocol="ll")
+
+
+@pytest.mark.parametrize("knobs", [dict(slices=1, piece_bytes=4096), dict(slices=3, piece_bytes=16 * 7, threads=128), dict(slices=2, workgroups=1, threads=64),
+                                   dict(slices=5, threads=512), dict(slices=16, threads=64), dict(slices=4, workgroups=3, threads=256)])
+def test_sub_dword_tails_under_explicit_geometries(knobs):
+    for xml, dtype, elems in ((ir_samples.ring_allreduce_xml(8, 2), "bfloat16", 20001), (ir_samples.allpairs_allreduce_xml(5), "float16", 20003),
+                              (ir_samples.ring_allgather_xml(8, 2), "uint8", 40001)):
+        got, want, _, info = run_both(xml, elems, dtype, seed=11, protocol="simple", **knobs)
+        assert info.vector_path == 1 and info.slices == knobs["slices"]
+        assert_same(got, want)
+
+
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("first_elem,chunk_elems", [(1, 1000), (3, 1001), (2, 40004), (1, 131075)])
 def test_buffers_that_start_off_a_16_byte_boundary(first_elem, chunk_elems, mode):
