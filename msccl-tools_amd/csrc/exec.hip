@@ -27,18 +27,18 @@ namespace mscclx {
 typedef void (*kernel_fn)(const KernelParams);
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
-kernel_fn pick_kernel_group_0(int dtype, int op, bool ll, bool fold);
-kernel_fn pick_kernel_group_1(int dtype, int op, bool ll, bool fold);
-kernel_fn pick_kernel_group_2(int dtype, int op, bool ll, bool fold);
-kernel_fn pick_kernel_group_3(int dtype, int op, bool ll, bool fold);
-kernel_fn pick_kernel_group_4(int dtype, int op, bool ll, bool fold);
-static kernel_fn pick_kernel(int dtype, int op, bool ll, bool fold) {
+kernel_fn pick_kernel_group_0(int dtype, int op, bool ll, bool fold, bool ragged);
+kernel_fn pick_kernel_group_1(int dtype, int op, bool ll, bool fold, bool ragged);
+kernel_fn pick_kernel_group_2(int dtype, int op, bool ll, bool fold, bool ragged);
+kernel_fn pick_kernel_group_3(int dtype, int op, bool ll, bool fold, bool ragged);
+kernel_fn pick_kernel_group_4(int dtype, int op, bool ll, bool fold, bool ragged);
+static kernel_fn pick_kernel(int dtype, int op, bool ll, bool fold, bool ragged) {
   switch (dtype / 2) {
-    case 0: return pick_kernel_group_0(dtype, op, ll, fold);
-    case 1: return pick_kernel_group_1(dtype, op, ll, fold);
-    case 2: return pick_kernel_group_2(dtype, op, ll, fold);
-    case 3: return pick_kernel_group_3(dtype, op, ll, fold);
-    case 4: return pick_kernel_group_4(dtype, op, ll, fold);
+    case 0: return pick_kernel_group_0(dtype, op, ll, fold, ragged);
+    case 1: return pick_kernel_group_1(dtype, op, ll, fold, ragged);
+    case 2: return pick_kernel_group_2(dtype, op, ll, fold, ragged);
+    case 3: return pick_kernel_group_3(dtype, op, ll, fold, ragged);
+    case 4: return pick_kernel_group_4(dtype, op, ll, fold, ragged);
     default: return nullptr;
   }
 }
@@ -142,7 +142,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
   const mscclx_plan* plan = &plan_ref;
   const Geometry& g = plan->geo;
   const bool fold = !g.ll && has_foldable_nops(*plan);
-  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold);
+  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold, plan->chunk_bytes % 16 != 0);
   if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   DeviceImage* d = img;
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
@@ -452,11 +452,12 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
   } else {
     const bool ll = cfg.protocol == MSCCLX_PROTO_LL;
     const bool fold = !ll && has_foldable_nops(*plan);
-    int rc = query_capacity(pick_kernel(dtype, redop, ll, fold), &num_cus, capacity);
+    const bool ragged = chunk_bytes % 16 != 0;  // rows may end inside a 16-byte unit: kernels of their own
+    int rc = query_capacity(pick_kernel(dtype, redop, ll, fold, ragged), &num_cus, capacity);
     if (rc) return rc;
     if (cfg.protocol == MSCCLX_PROTO_AUTO && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
       int other[kThreadChoices];
-      rc = query_capacity(pick_kernel(dtype, redop, true, false), &num_cus, other);
+      rc = query_capacity(pick_kernel(dtype, redop, true, false, ragged), &num_cus, other);
       if (rc) return rc;
       for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
     }

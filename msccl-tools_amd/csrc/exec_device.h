@@ -644,7 +644,7 @@ __device__ __forceinline__ void mark_many_sources(Context& c, const DevOp& op) {
 // where.  LL: an incoming message is not announced by a counter; the lane watches the flag in the
 // last 8 bytes of the message instead (w1 = that word, t1 = the flag).  Lines may land in any order,
 // so this is a hint that the message is about to be complete; the threads that read it check every line.
-template <bool LL>
+template <bool LL, bool RAGGED>
 __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const KernelParams& p, uint32_t epoch, const DevOp& op) {
   const int t = (int)(op.word & 15u);
   const int cnt = (int)(op.word >> kOpCntShift);
@@ -693,8 +693,9 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     case MSCCLX_OP_REDUCE: m.a = op.src_addr + c.off; kind = kHasB; break;
     default: break;
   }
-  // the pass that reaches the end of the slice: its rows may end inside their last unit
-  m.kind = kind | (c.left <= p.piece_units ? (int)h.clip << kClipShift : 0);
+  m.kind = kind;
+  // RAGGED (chunks that are no multiple of 16 bytes): in the pass that reaches the end of the slice, rows may end inside their last unit
+  if constexpr (RAGGED) m.kind = kind | (c.left <= p.piece_units ? (int)h.clip << kClipShift : 0);
 }
 
 // The description of the step after the one `c` stands at.  It is fetched before the counters of
@@ -708,7 +709,7 @@ __device__ __forceinline__ DevOp fetch_next_op(const Context& c, const Hosted& h
 // Announce the completed step and move the context to its next one, described by `next`.
 // `writer`: this thread stores the counters (the context's lane; one thread of a wave that runs a
 // context with all its lanes).
-template <bool LL>
+template <bool LL, bool RAGGED>
 __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, const KernelParams& p, uint32_t epoch, const DevOp& next, bool writer = true) {
   const Hosted h = entry;  // one batch of LDS reads, one wait -- not one wait per field as they are needed
   if (is_send(c.type)) {
@@ -732,13 +733,13 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
     c.off += (u64)p.piece_units * 16;
   }
   if (c.pass >= h.npasses) c.active = false;
-  else describe_step<LL>(c, h, p, epoch, next);
+  else describe_step<LL, RAGGED>(c, h, p, epoch, next);
 }
 
 // Set up hosted context number `ctx`: its constants in `h` (the record worked out when the buffers were
 // bound), its state in `c`, standing at its first step.  `writer` also clears, for the next launch,
 // the counters this context alone writes.
-template <bool LL>
+template <bool LL, bool RAGGED>
 __device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int ctx, bool writer) {
   const DevCtx rec = p.ctxs[ctx];
   h = rec.h;
@@ -751,18 +752,18 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
     if (h.head_out) p.sync_nxt[h.head_out] = 0;
     if (h.tail_out) p.sync_nxt[h.tail_out] = 0;
   }
-  if (c.active) describe_step<LL>(c, h, p, epoch, p.ops[h.op_begin]);
+  if (c.active) describe_step<LL, RAGGED>(c, h, p, epoch, p.ops[h.op_begin]);
 }
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
 // incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool LL, bool FOLD = false>
+template <class R, bool LL, bool FOLD, bool RAGGED>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
   constexpr int W = 16;
   const u64 cs = p.chunk_bytes;                   // rows of a rank buffer are a chunk apart ...
   const u64 packed = (u64)m.n * W;                // ... rows in a slot are packed
-  const uint32_t clip = ((uint32_t)m.kind & kClipMask) >> kClipShift;
+  const uint32_t clip = RAGGED ? ((uint32_t)m.kind & kClipMask) >> kClipShift : 0u;  // (a constant 0 folds every cut and tail below away)
   unsigned char* const dst = (unsigned char*)m.dst;
   unsigned char* const out = (unsigned char*)m.out;
   const unsigned char* const a = (const unsigned char*)m.a;
@@ -981,7 +982,7 @@ __device__ __forceinline__ DevOp fetch_step(ConstOps e) {  // (field by field: a
 // (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for a dependency, 1 from the first
 // load of a message's lines until they are all there, 2 from there until the step's stores are issued,
 // 3 from there to the next step's first load, 4 in all)
-template <class R>
+template <class R, bool RAGGED>
 __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch, int ctx, u64* prof_acc = nullptr) {
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
@@ -990,14 +991,14 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<true>(h, first, p, epoch, ctx, writer);
+    init_context<true, RAGGED>(h, first, p, epoch, ctx, writer);
     if (!first.active) return;
     left = uniform(first.left);
     off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
   const u64 row_stride = p.chunk_bytes;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
-  const uint32_t end_clip = uniform(h.clip);  // bytes that the last unit of the slice's last pass lacks (see move_units)
+  const uint32_t end_clip = RAGGED ? uniform(h.clip) : 0u;  // bytes that the last unit of the slice's last pass lacks (see move_units)
   unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
   unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
   const u64* const flags = p.sync_cur + uniform(h.flags);
@@ -1140,7 +1141,7 @@ __device__ __forceinline__ void chain_copy_round(const __amdgpu_buffer_rsrc_t ra
 // step waits for its (up to three) counters with one round of loads, moves its rows, waits until its
 // stores are acknowledged and announces them.  Steps, waits and counters are those of the hosted
 // path, so a workgroup running this loop can talk to workgroups running that one.
-template <class R>
+template <class R, bool RAGGED>
 __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ctx, u64* prof_acc = nullptr) {
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
@@ -1149,14 +1150,14 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   u64 off;        // byte offset of this pass's piece inside every chunk
   {
     Context first;
-    init_context<false>(h, first, p, 0, ctx, writer);
+    init_context<false, RAGGED>(h, first, p, 0, ctx, writer);
     if (!first.active) return;
     left = uniform(first.left);
     off = uniform((uint64_t)first.off);
   }
   const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
   const u64 row_stride = p.chunk_bytes;  // rows of a rank buffer are a chunk apart; rows of a slot are packed
-  const uint32_t end_clip = uniform(h.clip);  // bytes that the last unit of the slice's last pass lacks (see move_units)
+  const uint32_t end_clip = RAGGED ? uniform(h.clip) : 0u;  // bytes that the last unit of the slice's last pass lacks (see move_units)
   unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
   unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
   const u64* const flags = p.sync_cur + uniform(h.flags);
@@ -1268,7 +1269,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
 // share the resident workgroups without deadlock.
 // FOLD: steps may carry the dependencies of nop steps folded into them (a kernel of its own, so that
 // programs without such steps do not pay for the check in the poll loop).
-template <class R, bool LL, bool FOLD = false>
+template <class R, bool LL, bool FOLD, bool RAGGED>
 __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
   // The number of launches so far is kept on the device (control word 0) and is advanced by the
   // last workgroup to finish, so a launch carries no host-side state and the same launch can be
@@ -1307,25 +1308,25 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
   if (LL && hosted == 1 && blockDim.x == 64) {  // (LL is configured only for chunks of whole dwords)
 #ifdef MSCCLX_PROFILE
     u64 chain_acc[5] = {0, 0, 0, 0, 0};
-    if constexpr (LL) run_chain<R>(p, epoch, ctx_begin, chain_acc);
+    if constexpr (LL) run_chain<R, RAGGED>(p, epoch, ctx_begin, chain_acc);
     prof_fin = chain_acc[0]; prof_wait = chain_acc[1]; prof_move = chain_acc[2]; prof_ack = chain_acc[3];
     if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
 #else
-    if constexpr (LL) run_chain<R>(p, epoch, ctx_begin);
+    if constexpr (LL) run_chain<R, RAGGED>(p, epoch, ctx_begin);
 #endif
-  } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64 && (p.chunk_bytes & 3u) == 0) {
+  } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64 && (!RAGGED || (p.chunk_bytes & 3u) == 0)) {
     // (the chain loops move whole dwords: a chunk of 8- or 16-bit elements that is no multiple of 4 bytes takes the
     // general loop below -- the 1 to 3 bytes at its end cost the chain loop 4 % of every launch in scalar registers)
 #ifdef MSCCLX_PROFILE
     u64 chain_acc[5] = {0, 0, 0, 0, 0};
-    if constexpr (!LL && !FOLD) run_chain_counters<R>(p, ctx_begin, chain_acc);
+    if constexpr (!LL && !FOLD) run_chain_counters<R, RAGGED>(p, ctx_begin, chain_acc);
     prof_wait = chain_acc[0]; prof_move = chain_acc[1]; prof_ack = chain_acc[2]; prof_fin = chain_acc[3];
     if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
 #else
-    if constexpr (!LL && !FOLD) run_chain_counters<R>(p, ctx_begin);
+    if constexpr (!LL && !FOLD) run_chain_counters<R, RAGGED>(p, ctx_begin);
 #endif
   } else {
-  if (poller && lane < hosted) init_context<LL>(h, c, p, epoch, ctx_begin + lane, true);
+  if (poller && lane < hosted) init_context<LL, RAGGED>(h, c, p, epoch, ctx_begin + lane, true);
   if (FOLD && poller && lane < hosted && c.active) mark_many_sources(c, p.ops[h.op_begin]);
   int cursor = 0;
   unsigned busy_rounds = 0;
@@ -1360,7 +1361,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
           const DevOp next = fetch_next_op(c, h, p);
-          finish_step<LL>(c, h, p, epoch, next);
+          finish_step<LL, RAGGED>(c, h, p, epoch, next);
           if (FOLD && c.active) mark_many_sources(c, next);
           progressed = true;
           ready = false;  // the context now stands at another step, whose conditions are not yet known
@@ -1445,7 +1446,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
 
     // ---- the chosen context's step: move one piece ----
-    do_move<R, LL, FOLD>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
+    do_move<R, LL, FOLD, RAGGED>(m, p, epoch, rseq, sseq, who_tb, who_step, who_slice, who_pass);
 #ifdef MSCCLX_PROFILE
     const u64 prof_t2 = wall_clock64();
 #endif
@@ -1461,7 +1462,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     const u64 prof_t3 = wall_clock64();
 #endif
     if (mine) {
-      finish_step<LL>(c, h, p, epoch, next);
+      finish_step<LL, RAGGED>(c, h, p, epoch, next);
       if (FOLD && c.active) mark_many_sources(c, next);
     }
 #ifdef MSCCLX_PROFILE
@@ -1514,17 +1515,18 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 // ------------------------------------------------------------------------------------------------
 typedef void (*kernel_fn)(const KernelParams);
 
-template <int DT, int OP> kernel_fn pick_variant(bool ll, bool fold) {
-  if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true> : nullptr;
-  if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, true>;
-  return (kernel_fn)exec_kernel<Reducer<DT, OP>, false>;
+// ragged: chunks that are no multiple of 16 bytes -- rows may end inside a unit; the other kernels carry none of that
+template <int DT, int OP, bool RAGGED> kernel_fn pick_variant(bool ll, bool fold) {
+  if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false, RAGGED> : nullptr;
+  if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, true, RAGGED>;
+  return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false, RAGGED>;
 }
-template <int DT> kernel_fn pick_op(int op, bool ll, bool fold) {
+template <int DT> kernel_fn pick_op(int op, bool ll, bool fold, bool ragged) {
   switch (op) {
-    case MSCCLX_SUM: return pick_variant<DT, MSCCLX_SUM>(ll, fold);
-    case MSCCLX_PROD: return pick_variant<DT, MSCCLX_PROD>(ll, fold);
-    case MSCCLX_MAX: return pick_variant<DT, MSCCLX_MAX>(ll, fold);
-    case MSCCLX_MIN: return pick_variant<DT, MSCCLX_MIN>(ll, fold);
+    case MSCCLX_SUM: return (ragged ? pick_variant<DT, MSCCLX_SUM, true>(ll, fold) : pick_variant<DT, MSCCLX_SUM, false>(ll, fold));
+    case MSCCLX_PROD: return (ragged ? pick_variant<DT, MSCCLX_PROD, true>(ll, fold) : pick_variant<DT, MSCCLX_PROD, false>(ll, fold));
+    case MSCCLX_MAX: return (ragged ? pick_variant<DT, MSCCLX_MAX, true>(ll, fold) : pick_variant<DT, MSCCLX_MAX, false>(ll, fold));
+    case MSCCLX_MIN: return (ragged ? pick_variant<DT, MSCCLX_MIN, true>(ll, fold) : pick_variant<DT, MSCCLX_MIN, false>(ll, fold));
     default: return nullptr;
   }
 }

@@ -11,10 +11,10 @@
 
 namespace mscclx {
 
-kernel_fn MSCCLX_PASTE(pick_kernel_group_, MSCCLX_KERNEL_GROUP)(int dtype, int op, bool ll, bool fold) {
+kernel_fn MSCCLX_PASTE(pick_kernel_group_, MSCCLX_KERNEL_GROUP)(int dtype, int op, bool ll, bool fold, bool ragged) {
   static_assert(2 * MSCCLX_KERNEL_GROUP + 1 < MSCCLX_NUM_DTYPES, "two element types per group");
-  if (dtype == 2 * MSCCLX_KERNEL_GROUP) return pick_op<2 * MSCCLX_KERNEL_GROUP>(op, ll, fold);
-  if (dtype == 2 * MSCCLX_KERNEL_GROUP + 1) return pick_op<2 * MSCCLX_KERNEL_GROUP + 1>(op, ll, fold);
+  if (dtype == 2 * MSCCLX_KERNEL_GROUP) return pick_op<2 * MSCCLX_KERNEL_GROUP>(op, ll, fold, ragged);
+  if (dtype == 2 * MSCCLX_KERNEL_GROUP + 1) return pick_op<2 * MSCCLX_KERNEL_GROUP + 1>(op, ll, fold, ragged);
   return nullptr;
 }
 
