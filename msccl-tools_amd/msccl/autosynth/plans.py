@@ -3,6 +3,7 @@
 are all virtual ranks of one MI355X (machines = groups of 8 virtual ranks)."""
 from msccl.autosynth.registry import register_msccl_program
 from msccl.language.ir import ThreadblockPolicy
+from msccl.programs.allgather_allpairs import allgather_allpairs
 from msccl.programs.allgather_ring import allgather_ring
 from msccl.programs.allreduce_a100_ring import allreduce_ring
 from msccl.programs.allreduce_allpairs import allreduce_allpairs
@@ -77,8 +78,16 @@ def register_mi355x_plans():
     def mi355x_ring_allreduce_large(prog, nodes):
         allreduce_ring(size=8, channels=1)
 
+    # All-gather, int32, microseconds by bytes per rank (all-pairs / ring x 4 instances): 1 MiB 18 / 31, 2 MB 26 / 51,
+    # 4 MiB 67 / 78, 8 MiB 136 / 144, 12 MB 215 / 212, 16 MiB 287 / 276, 32 MB 570 / 529.  Both move the same bytes; all-pairs
+    # is one hand-off deep, the ring seven, and the ring's pieces stream better at the large end.
+    @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=1,
+                            sizes=(0, '12MB'), threadblock_policy=manual, machines=one)
+    def mi355x_allpairs_allgather(prog, nodes):
+        allgather_allpairs(8)
+
     @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=4,
-                            threadblock_policy=manual, machines=one)
+                            sizes=('12MB', None), threadblock_policy=manual, machines=one)
     def mi355x_ring_allgather(prog, nodes):
         allgather_ring(size=8, channels=1)
 

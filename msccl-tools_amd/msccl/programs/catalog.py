@@ -50,6 +50,16 @@ def ring_allgather(num_ranks, channels=1, instances=1, protocol="Simple"):
     return _finish(prog)
 
 
+def allpairs_allgather(num_ranks, instances=1, protocol="Simple"):
+    """All-pairs all-gather (msccl.programs.allgather_allpairs): AllGather(n, 1, inplace), manual threadblocks."""
+    from msccl.programs.allgather_allpairs import allgather_allpairs
+    prog = MSCCLProgram("allgather_allpairs", fully_connected(num_ranks), AllGather(num_ranks, 1, True),
+                        instances, protocol=protocol, threadblock_policy=ThreadblockPolicy.manual)
+    with prog:
+        allgather_allpairs(num_ranks)
+    return _finish(prog)
+
+
 def hierarchical_alltoall(num_nodes, gpus_per_node, instances=1, protocol="Simple"):
     """examples/mscclang/alltoall_a100_two_step.py:8-48: AllToAll(n, 1, out of place), automatic
     threadblocks."""

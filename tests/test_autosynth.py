@@ -131,6 +131,19 @@ def test_selection_windows_are_half_open(capsys):
     assert [(a.min_bytes, a.max_bytes, a.tables.nchunksperloop) for a in load_config()] == [(0, 16000000, 64)]
 
 
+def test_mi355x_allgather_windows(capsys):
+    """All-pairs all-gather (one hand-off deep) below 12 MB per rank, the ring (4 instances) from there on."""
+    msccl.init('mi355x', 1, ('allgather', (0, None)))
+    capsys.readouterr()
+    algos = load_config()
+    assert [(a.min_bytes, a.max_bytes, a.tables.name) for a in algos] == [(0, 12000000, 'mi355x_allpairs_allgather'),
+                                                                          (12000000, float("inf"), 'mi355x_ring_allgather')]
+    small, large = algos
+    assert small.tables.ntbs == 8 * 7 and small.tables.nops == 8 * 14 and small.tables.nchunksperloop == 8   # a threadblock per peer: one send, one receive
+    assert large.tables.nchunksperloop == 32                                              # 8 chunks x 4 instances
+    assert select(algos, "allgather", 1 << 20) is small and select(algos, "allgather", 64 << 20) is large
+
+
 def test_ef_file_plan(tmp_path, capsys):
     import ir_samples
     f = tmp_path / "ring.xml"

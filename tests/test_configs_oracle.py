@@ -137,6 +137,24 @@ def test_custom_collective_examples(name):
         assert np.array_equal(bufs[r]["o"], x[0]), (name, r)
 
 
+@pytest.mark.parametrize("n,instances", [(8, 1), (5, 2), (2, 1)])
+def test_allpairs_allgather_is_a_concatenation(n, instances):
+    """The all-pairs all-gather of the mi355x plans: every rank ends with every rank's input, in rank order;
+    one hand-off deep (a threadblock per peer and instance: one send to it, one receive from it)."""
+    from msccl.programs import catalog
+    algo = oi.parse_xml(catalog.allpairs_allgather(n, instances))
+    assert algo.coll == "allgather" and algo.inplace and algo.ngpus == n
+    assert all(sorted(st.type for st in tb.steps) == ["r", "s"] for g in algo.gpus for tb in g.tbs)
+    E = 3
+    rng = np.random.default_rng(n)
+    x = [rng.integers(-2 ** 31, 2 ** 31, instances * E, dtype=np.int64).astype(np.int32) for _ in range(n)]
+    bufs = oc.place_inputs(algo, x, E, "int32")
+    oi.Interpreter(algo).run(bufs, E, "int32")
+    want = np.concatenate(x)
+    for r in range(n):
+        assert np.array_equal(bufs[r]["o"], want), r
+
+
 def test_allpairs_fold_order_float():
     algo_xml = golden_util.load("allreduce_allpairs_8r_2inst")
     algo = oi.parse_xml(algo_xml)
