@@ -60,6 +60,15 @@ def allpairs_allgather(num_ranks, instances=1, protocol="Simple"):
     return _finish(prog)
 
 
+def allpairs_alltoall(num_ranks, instances=1, protocol="Simple"):
+    """examples/mscclang/alltoall_allpairs.py:10-19: AllToAll(n, 1, out of place), automatic threadblocks."""
+    from msccl.programs.alltoall_allpairs import alltoall_allpairs
+    prog = MSCCLProgram("alltoall_allpairs", fully_connected(num_ranks), AllToAll(num_ranks, 1, inplace=False), instances, protocol=protocol)
+    with prog:
+        alltoall_allpairs(num_ranks)
+    return _finish(prog)
+
+
 def hierarchical_alltoall(num_nodes, gpus_per_node, instances=1, protocol="Simple"):
     """examples/mscclang/alltoall_a100_two_step.py:8-48: AllToAll(n, 1, out of place), automatic
     threadblocks."""

@@ -144,6 +144,18 @@ def test_mi355x_allgather_windows(capsys):
     assert select(algos, "allgather", 1 << 20) is small and select(algos, "allgather", 64 << 20) is large
 
 
+def test_mi355x_alltoall_plans(capsys):
+    """One group of 8 virtual ranks: the one-step all-to-all; two to eight groups: the hierarchical one."""
+    msccl.init('mi355x', 1, ('alltoall', '1MB'))
+    assert 'mi355x_alltoall_allpairs' in capsys.readouterr().out
+    (a,) = load_config()
+    assert a.tables.coll == "alltoall" and a.tables.ngpus == 8 and not a.tables.inplace
+    assert a.tables.nops == 2 * 8 * 7 + 8      # a send and a receive for every pair, and every rank's copy of its own chunk
+    msccl.init('mi355x', 2, ('alltoall', '1MB'))
+    assert 'mi355x_alltoall_hierarchical' in capsys.readouterr().out
+    assert load_config()[0].tables.ngpus == 16
+
+
 def test_ef_file_plan(tmp_path, capsys):
     import ir_samples
     f = tmp_path / "ring.xml"

@@ -27,9 +27,11 @@ PROGRAMS = {
     "allreduce_ring_8r_4ch_8inst": lambda: catalog.ring_allreduce(8, 4, 8),
     "allreduce_allpairs_8r_2inst": lambda: catalog.allpairs_allreduce(8, 2, protocol="LL"),
     "alltoall_three_step_3x4": lambda: catalog.three_step_alltoall(3, 4),
+    "alltoall_allpairs_4r": lambda: catalog.allpairs_alltoall(4, 1),
 }
 BYTE_IDENTICAL = ["c1_allreduce_ring_8r_1ch_1inst", "c2_allgather_ring_8r_1ch_4inst", "c4_hierarchical_allreduce_8x4_2inst_auto",
-                  "c4_hierarchical_allreduce_4x2_1inst_manual", "c5_allreduce_ring_64r_1ch_1inst", "c5_allreduce_chain_64r", "allreduce_ring_8r_4ch_8inst"]
+                  "c4_hierarchical_allreduce_4x2_1inst_manual", "c5_allreduce_ring_64r_1ch_1inst", "c5_allreduce_chain_64r", "allreduce_ring_8r_4ch_8inst",
+                  "alltoall_allpairs_4r"]
 
 
 def _anonymous(xml):

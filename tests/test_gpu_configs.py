@@ -269,6 +269,41 @@ def test_rebind_new_buffers_same_plan():
             assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (k, r)
 
 
+def test_init_to_run_alltoall_and_large_allgather(capsys):
+    """The other mi355x plans of one group of 8: the one-step all-to-all (a block transpose) and, from 12 MB per
+    rank on, the 4-instance ring all-gather -- at a size that is no multiple of 16 bytes per chunk."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    a2a_bytes, ag_bytes = 8 * 3001 * 4, 12000000 + 32 * 4     # per rank
+    msccl.init('mi355x', 1, ('alltoall', a2a_bytes), ('allgather', ag_bytes))
+    capsys.readouterr()
+    algos = load_config()
+    a2a, ag = select(algos, "alltoall", a2a_bytes), select(algos, "allgather", ag_bytes)
+    assert a2a.tables.name == "mi355x_alltoall_allpairs" and ag.tables.name == "mi355x_ring_allgather"
+    rng = np.random.default_rng(9)
+    x = [rng.integers(-2 ** 31, 2 ** 31, a2a_bytes // 4, dtype=np.int64).astype(np.int32) for _ in range(8)]
+    cb = a2a.bytes_per_rank_to_chunk_bytes(a2a_bytes)
+    assert cb == 3001 * 4
+    ex = Executor(a2a.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v) for v in x])
+    ex.run(ins, outs)
+    for r in range(8):
+        want = np.concatenate([x[s][r * 3001:(r + 1) * 3001] for s in range(8)])
+        assert np.array_equal(res[r].cpu().numpy(), want), r
+    y = [rng.integers(-2 ** 31, 2 ** 31, ag_bytes // 4, dtype=np.int64).astype(np.int32) for _ in range(8)]
+    cb = ag.bytes_per_rank_to_chunk_bytes(ag_bytes)
+    ex = Executor(ag.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v) for v in y])
+    ex.run(ins, outs)
+    want = np.concatenate(y)
+    assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(8))
+
+
 def test_init_to_run_flow(capsys):
     """msccl.init -> MSCCL_CONFIG index -> select by size -> run: the drop-in path end to end."""
     import os
