@@ -360,10 +360,11 @@ static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img,
   kp.timeout_ticks = (uint64_t)plan.timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
   kp.slice_grain = g.slice_grain;
-  {  // groups of about sqrt(workgroups), at most kFinishGroups of them
+  {  // groups of about sqrt(workgroups), at most kFinishGroups of them; up to 64 workgroups are one group
     uint32_t per = 1;
     while ((uint64_t)per * per < (uint64_t)g.workgroups) ++per;
     per = std::max<uint32_t>(per, ((uint32_t)g.workgroups + kFinishGroups - 1) / kFinishGroups);
+    if (g.workgroups <= 64) per = (uint32_t)g.workgroups;
     kp.finish_group = per;
   }
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan.tbs.size(); kp.nconns = (int)plan.conns.size();

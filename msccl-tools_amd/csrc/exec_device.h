@@ -1489,7 +1489,9 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
     if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
       publish(group_count, 0);
-      if (__hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
+      if (groups == 1) {  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
+        publish(p.sync_base, launch_no + 1);
+      } else if (__hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
         publish(p.sync_base + 1, 0);
         publish(p.sync_base, launch_no + 1);
       }
