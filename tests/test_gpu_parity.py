@@ -3,6 +3,7 @@ import numpy as np
 import pytest
 import torch
 
+import golden_util
 import ir_samples
 from oracle import collectives as oc
 from oracle import ir_interp as oi
@@ -340,6 +341,49 @@ def test_geometry_knobs(knobs):
     assert_same(got, want)
     got, want, _, _ = run_both(ir_samples.allpairs_allreduce_xml(5), 40000, "bfloat16", **knobs)
     assert_same(got, want)
+
+
+@pytest.mark.parametrize("batch", range(4))
+def test_random_sizes_dtypes_and_geometries(batch):
+    """Sixty random draws per batch of (program, element type, reduction, chunk size from 1 to 300 000 elements, message mode,
+    geometry knobs) against the interpreter, every byte compared.  A draw the library refuses must be refused
+    for a reason that the draw explains."""
+    import random
+    from msccl.executor import DTYPE_SIZES, MscclxError
+    from msccl.executor import binding
+    rnd = random.Random(1000 + batch)
+    programs = [ir_samples.ring_allreduce_xml(8, 2), ir_samples.ring_allreduce_xml(4), ir_samples.allpairs_allreduce_xml(5), ir_samples.RRC_CPY_NOP_XML,
+                ir_samples.ring_allgather_xml(8, 2), ir_samples.reduce_chain_xml(7, 8), golden_util.load("alltoall_three_step_3x4"),
+                golden_util.load("c4_hierarchical_allreduce_4x2_1inst_manual"), golden_util.load("allreduce_a100_allpairs_v2_8r")]
+    dtypes = ["float32", "bfloat16", "float16", "uint8", "int8", "int32", "float64", "int64"]
+    ran = 0
+    for case in range(60):
+        xml, dtype = rnd.choice(programs), rnd.choice(dtypes)
+        elems = rnd.choice([rnd.randint(1, 40), rnd.randint(41, 3000), rnd.randint(3001, 70000), rnd.randint(70001, 300000)])
+        mode = rnd.choice(["in-place", "staged", "ll", "auto"])
+        knobs = {} if mode == "auto" else dict(MODES[mode])
+        g = rnd.random()
+        if g < 0.25:
+            knobs.update(slices=rnd.choice([1, 2, 3, 5, 8, 16]))
+        elif g < 0.4:
+            knobs.update(slices=rnd.choice([1, 2, 4]), threads=rnd.choice([64, 128, 256, 512]))
+        elif g < 0.5:
+            knobs.update(slices=2, workgroups=rnd.choice([1, 3, 7]), threads=rnd.choice([64, 256]))
+        if rnd.random() < 0.2:
+            knobs.update(piece_bytes=rnd.choice([112, 4096, 65536]))
+        redop = rnd.choice(["sum", "sum", "max", "min", "prod"]) if dtype not in ("uint8", "int8") else rnd.choice(["sum", "max", "min"])
+        try:
+            got, want, _, info = run_both(xml, elems, dtype, seed=100 * batch + case, redop=redop, **knobs)
+        except MscclxError as e:
+            nbytes = elems * DTYPE_SIZES[dtype]
+            explained = ((e.code == binding.ERR_UNSUPPORTED and mode == "ll" and nbytes % 4) or            # lines carry whole dwords
+                         (e.code == binding.ERR_INVALID_ARG and knobs.get("slices", 0) > (nbytes + 15) // 16) or  # more slices than units
+                         (e.code == binding.ERR_CAPACITY and "workgroups" in knobs))                       # too few workgroups for the contexts
+            assert explained, (case, str(e), elems, dtype, knobs)
+            continue
+        assert_same(got, want)
+        ran += 1
+    assert ran >= 40
 
 
 def test_relaunch_reuses_counters():
