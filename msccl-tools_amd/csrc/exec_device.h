@@ -1218,15 +1218,33 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       u64 a_row = rcv ? (in_place ? op.in_addr + off : (u64)(in_ring + rslot)) : op.src_addr + off;
       const u64 a_stride = (rcv && !in_place) ? (u64)n * 16 : row_stride;
       u64 local_row = op.dst_addr + off, slot_row = (u64)(out_ring + sslot);
-      const uint32_t row_bytes = n * 16 - (left <= piece ? end_clip : 0u);  // (slot rows are n units apart, and end where their rank-buffer rows do; whole dwords: see the kernel's choice of this loop)
+      const uint32_t row_total = n * 16 - (left <= piece ? end_clip : 0u);  // (slot rows are n units apart, and end where their rank-buffer rows do)
+      // whole dwords through the descriptors; RAGGED kernels of 8- and 16-bit elements: then 1 to 3 bytes, element by element (see move_units)
+      constexpr bool kTails = RAGGED && R::kElemBytes < 4;
+      const uint32_t row_bytes = kTails ? row_total & ~3u : row_total, odd = row_total - row_bytes;
       for (uint32_t row = 0; row < cnt; ++row) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc((const void*)a_row, row_bytes), rlocal = make_rsrc((const void*)local_row, row_bytes);
         const __amdgpu_buffer_rsrc_t rslot_out = make_rsrc((const void*)slot_row, row_bytes);
+        typedef Access<(R::kElemBytes < 4 ? R::kElemBytes : 1)> AE;
+        typename AE::word tail_x{}, tail_y{};
+        if constexpr (kTails) {
+          if (odd && lane * R::kElemBytes < odd) {
+            tail_x = AE::template ld<MSCCLX_AUX_LD>(make_rsrc((const void*)(a_row + row_bytes), odd), (int)(lane * R::kElemBytes));
+            if (has_b) tail_y = AE::template ld<MSCCLX_AUX_LD>(make_rsrc((const void*)(local_row + row_bytes), odd), (int)(lane * R::kElemBytes));
+          }
+        }
         if (n <= 64) chain_copy_round<R, 1>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else if (n <= 128) chain_copy_round<R, 2>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else if (n <= 256) chain_copy_round<R, 4>(ra, rlocal, rlocal, rslot_out, lane, has_b, to_local, to_slot, nt);
         else  // (eight loads in flight per lane and operand, as the workgroup-wide mover has)
           for (uint32_t base = 0; base < n; base += 512) chain_copy_round<R, 8>(ra, rlocal, rlocal, rslot_out, base + lane, has_b, to_local, to_slot, nt);
+        if constexpr (kTails) {
+          if (odd && lane * R::kElemBytes < odd) {
+            if (has_b) tail_x = R::combine(tail_y, tail_x);
+            if (to_local) AE::template st<MSCCLX_AUX_ST>(make_rsrc((const void*)(local_row + row_bytes), odd), (int)(lane * R::kElemBytes), tail_x);
+            if (to_slot) AE::template st<MSCCLX_AUX_ST>(make_rsrc((const void*)(slot_row + row_bytes), odd), (int)(lane * R::kElemBytes), tail_x);
+          }
+        }
         a_row += a_stride; local_row += row_stride; slot_row += (u64)n * 16;
       }
       MSCCLX_CHAIN_CLOCK(prof_issued);
@@ -1314,9 +1332,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #else
     if constexpr (LL) run_chain<R, RAGGED>(p, epoch, ctx_begin);
 #endif
-  } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64 && (!RAGGED || (p.chunk_bytes & 3u) == 0)) {
-    // (the chain loops move whole dwords: a chunk of 8- or 16-bit elements that is no multiple of 4 bytes takes the
-    // general loop below -- the 1 to 3 bytes at its end cost the chain loop 4 % of every launch in scalar registers)
+  } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64) {
 #ifdef MSCCLX_PROFILE
     u64 chain_acc[5] = {0, 0, 0, 0, 0};
     if constexpr (!LL && !FOLD) run_chain_counters<R, RAGGED>(p, ctx_begin, chain_acc);
