@@ -295,6 +295,22 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
     if (odd) tail.template store<HAS_O2, NT1>(o1 + bytes, HAS_O2 ? o2 + bytes : nullptr, odd);
     return;
   }
+  if (n <= 2 * T) {
+    // Two units per thread at most: a slice a few units over a workgroup's width (chunks that do not divide evenly).  The
+    // loop below would issue its eight loads and stores per thread for them, nearly all beyond the row's end.
+    const uint32_t i = threadIdx.x, j = i + T;
+    SubDword<R, HAS_B> tail;
+    if (odd) tail.load(a + bytes, HAS_B ? b + bytes : nullptr, odd);
+    word x0 = A::template ld<XL>(ra, (int)(i * W)), x1 = A::template ld<XL>(ra, (int)(j * W));
+    if (HAS_B) {
+      const word y0 = A::template ld<XL>(rb, (int)(i * W)), y1 = A::template ld<XL>(rb, (int)(j * W));
+      x0 = R::combine(y0, x0); x1 = R::combine(y1, x1);
+    }
+    A::template st<X1>(r1, (int)(i * W), x0); A::template st<X1>(r1, (int)(j * W), x1);
+    if (HAS_O2) { A::template st<XS>(r2, (int)(i * W), x0); A::template st<XS>(r2, (int)(j * W), x1); }
+    if (odd) tail.template store<HAS_O2, NT1>(o1 + bytes, HAS_O2 ? o2 + bytes : nullptr, odd);
+    return;
+  }
   // kUnroll loads are in flight per thread either way: all of a, or half of a and half of b
   constexpr int UA = HAS_B ? (kUnroll / 2 > 0 ? kUnroll / 2 : 1) : kUnroll;
   if (!HAS_O2) {
@@ -305,8 +321,9 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
     // the destination's first line boundary).  So the row is moved in two parts: the body, whose units start
     // at that boundary, and the head in front of it -- at most 8 units, the last one cut by descriptors that
     // end where the body begins -- by the first lanes, loaded here and stored after the body.
+    // (rows of 8 KiB and more: below that a move is a matter of round trips, not of the memory system's rate, and the head is one more)
     const uint32_t head = (128u - ((uint32_t)(uintptr_t)o1 & 127u)) & 127u;
-    if (head != 0 && head < total) {
+    if (head != 0 && total >= 8192) {
       // (head and body each count their dwords from their own start: a row that starts on an odd 2-byte
       // boundary has a head of 4k + 2 bytes, and the body's dwords then sit on the destination's)
       const uint32_t hv = head & ~3u, hodd = head - hv, body = (total - head) & ~3u, bodd = total - head - body;

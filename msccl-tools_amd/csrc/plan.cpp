@@ -642,6 +642,19 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   // piece: the whole slice in one pass unless the FIFO slots of staged messages would not fit the budget
   g.slice_grain = std::max<uint32_t>(1, 256 / g.unit_bytes);
   if (g.chunk_units / g.slice_grain < (uint64_t)slices) g.slice_grain = 1;
+  // Slices of at most a kilobyte are moved one unit per lane by one wave: a 65th unit -- what the longer slices get
+  // when groups of 256 bytes do not divide evenly -- would cost every step of such a slice a second round.  Take the
+  // coarsest cut of 16, 8 ... 1 units that keeps every slice within 64 units: slices that start on cache lines are
+  // worth 10 % even at this size, a second round costs 50 %.
+  if ((g.chunk_units + (uint64_t)slices - 1) / (uint64_t)slices <= 64) {
+    auto longest = [&](uint32_t grain) {
+      uint64_t most_units = 0;
+      for (int64_t j = 0; j < slices; ++j)
+        most_units = std::max(most_units, slice_begin(g.chunk_units, grain, (int32_t)slices, (int32_t)j + 1) - slice_begin(g.chunk_units, grain, (int32_t)slices, (int32_t)j));
+      return most_units;
+    };
+    while (g.slice_grain > 1 && (g.chunk_units / g.slice_grain < (uint64_t)slices || longest(g.slice_grain) > 64)) g.slice_grain /= 2;
+  }
   uint64_t longest_slice = 0;
   for (int64_t j = 0; j < slices; ++j)
     longest_slice = std::max(longest_slice, slice_begin(g.chunk_units, g.slice_grain, (int32_t)slices, (int32_t)j + 1) -

@@ -274,6 +274,12 @@ def test_small_chunks_are_cut_one_unit_per_lane(mscclx_lib):
     # a knob that fixes the workgroups keeps the latency model's slices
     i = Plan(parse_algo_xml(golden_util.load("allreduce_a100_pcie_hierarchical_8r"))).configure(16 << 10, "float32", max_workgroups=4096, threads=128)
     assert i.slices == 4
+    # sizes that 256-byte groups do not divide: the slices are cut finer rather than let one of them run to a 65th unit
+    # (piece_bytes is the longest slice)
+    t = parse_algo_xml(golden_util.load("allreduce_a100_allpairs_8r"))
+    for chunk_bytes, longest in ((16384, 1024), (15616, 1024), (15624, 1008), (16368, 1024), (16380, 1024)):
+        i = Plan(t).configure(chunk_bytes, "float32", max_workgroups=4096)
+        assert (i.threads, i.slices, i.piece_bytes) == (64, 16, longest), (chunk_bytes, i.threads, i.slices, i.piece_bytes)
 
 
 def test_run_static_refuses_an_oversized_plan_before_touching_the_gpu(mscclx_lib):
