@@ -596,14 +596,25 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // pipelined all-pairs 33 -> 23 us), within 2 % for the rest.  Bigger chunks lose as often as they win, and
       // a ring whose every threadblock is busy all the time (64 ranks) loses beyond one context per SIMD.
       // Chunks of up to 128 KiB too where ALL contexts are at most one per SIMD (8-rank ring on 1 MiB: 33.3 -> 31.5 us).
+      // Where some threadblocks wait (waiting_ratio above 1) two busy contexts per SIMD still pay, and the slices need
+      // not be a power of two: over the same programs at 14 chunk sizes from 2 to 128 KiB, seven of them not powers of
+      // two, that took 0.9 % off the geometric mean -- PCIe-hierarchical all-reduce at 20 000-byte chunks 57 -> 40 us,
+      // all-pairs all-reduce 28 -> 23 us, two-node all-pairs at 4 KiB 73 -> 58 us; one program (the second all-pairs
+      // variant) rose by 2 to 7 %.  With no waiting at all (64-rank ring) a second context per SIMD costs 8 to 15 %.
       if (chunk_bytes <= 128 * 1024 && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups) {
         const double busy_share = chunk_bytes <= 64 * 1024 ? ratio : 1.0;
-        int64_t fine = 1;
-        while ((uint64_t)fine * 1024 < chunk_bytes) fine *= 2;  // pieces of at most 1 KiB
-        for (int64_t s : {fine, fine / 2}) {
+        const double per_cu = chunk_bytes <= 64 * 1024 && ratio > 1.0 ? 8.0 : 4.0;
+        // pieces of at most 1 KiB, else 2 KiB: a power of two up to 8 slices, a multiple of 8 (whole XCD rounds) beyond
+        auto slices_of = [&](uint64_t piece_units) {
+          const int64_t least = (int64_t)((g.chunk_units + piece_units - 1) / piece_units);
+          int64_t s = 1;
+          while (s < least && s < 8) s *= 2;
+          return s < least ? (least + 7) / 8 * 8 : s;
+        };
+        for (int64_t s : {slices_of(64), slices_of(128)}) {
           if (s <= slices || (uint64_t)s > g.chunk_units) continue;
           const int64_t contexts = s * ntbs;
-          if (contexts > capacity_by_threads[thread_index(64)] || (double)contexts > busy_share * 4.0 * (double)num_cus) continue;
+          if (contexts > capacity_by_threads[thread_index(64)] || (double)contexts > busy_share * per_cu * (double)num_cus) continue;
           slices = s;
           break;
         }

@@ -255,13 +255,16 @@ def test_geometry_between_the_benchmark_sizes(mscclx_lib):
 
 def test_small_chunks_are_cut_one_unit_per_lane(mscclx_lib):
     """Chunks of up to 64 KiB: pieces of 1 KiB (one 16-byte unit per lane of a one-wave workgroup), else 2 KiB,
-    where every context keeps a workgroup of its own and the busy ones are at most one per SIMD;
+    where every context keeps a workgroup of its own and the busy ones are at most one per SIMD (two where some
+    threadblocks wait); the slices are a power of two up to 8 and a multiple of 8 beyond;
     (workgroups, threads, slices, piece bytes, most contexts on a workgroup) on a 256-CU part."""
     want = {
         ("allreduce_a100_pcie_hierarchical_8r", 16 << 10): (2048, 64, 16, 1024, 1),   # 128 threadblocks that wait two thirds of the time
         ("pipeline_a100_allpairs_8r", 16 << 10): (2176, 64, 16, 1024, 1),
         ("allreduce_1step_4r", 64 << 10): (1024, 64, 64, 1024, 1),
-        ("allreduce_allpairs_8r_2inst", 16 << 10): (1024, 64, 8, 2048, 1),             # 1 KiB pieces would be 2048 busy contexts: 2 KiB
+        ("allreduce_allpairs_8r_2inst", 16 << 10): (2048, 64, 16, 1024, 1),            # some threadblocks wait: up to two busy contexts per SIMD
+        ("allreduce_allpairs_8r_2inst", 64 << 10): (512, 128, 4, 16384, 1),            # 8192 or 4096 contexts would be more: the latency model's 4
+        ("allreduce_a100_allpairs_8r", 20000): (1536, 64, 24, 928, 1),                  # 1250 units: 24 slices, a multiple of 8, not 32
         ("c5_allreduce_ring_64r_1ch_1inst", 16 << 10): (1024, 64, 16, 1024, 1),        # every threadblock busy: one context per SIMD ...
         ("c5_allreduce_ring_64r_1ch_1inst", 64 << 10): (512, 64, 8, 8192, 1),          # ... and no more
         ("c4_hierarchical_allreduce_8x4_2inst_auto", 4 << 10): (3840, 64, 2, 2048, 1),  # 1920 threadblocks: four slices would not get a workgroup each
