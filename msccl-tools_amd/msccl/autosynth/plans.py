@@ -65,8 +65,8 @@ def register_mi355x_plans():
     manual = ThreadblockPolicy.manual
 
     # Measured on MI355X, 8 virtual ranks, fp32 (microseconds, all-pairs / ring): 4 KiB to 512 KiB per
-    # rank 17-18 / 25-26, 1 MiB 19 / 32, 2 MiB 26 / 35, 4 MiB 39 / 44, 8 MiB 55 / 63, 16 MiB 100 / 100,
-    # 32 MiB 208 / 183, 64 MiB 373 / 348, 256 MiB 1774 / 1375.  All-pairs is three hand-offs deep, the ring fourteen; the ring moves
+    # rank 17-18 / 25-26, 1 MiB 19 / 32, 2 MiB 24 / 35, 4 MiB 37 / 45, 8 MiB 54 / 63, 16 MiB 96 / 101,
+    # 32 MiB 214 / 183, 64 MiB 372 / 348, 256 MiB 1774 / 1375.  All-pairs is three hand-offs deep, the ring fourteen; the ring moves
     # 5(n-1)/n chunks per chunk reduced, all-pairs about 4(n-1)/n + 2 on this executor.
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=1,
                             sizes=(0, '16MB'), threadblock_policy=manual, interleaved_replication=False,
