@@ -313,6 +313,22 @@ def test_partial_units_under_explicit_geometries(knobs, protocol):
         assert_same(got, want)
 
 
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("chunk_elems,dtype,slices", [(4100, "float32", 16), (14001, "float16", 16), (2047, "uint8", 1), (261, "float32", 1),
+                                                      (20000, "uint8", 16), (1025, "float64", 6), (509, "int32", 1)])
+def test_slices_of_up_to_two_units_per_lane(chunk_elems, dtype, slices, mode):
+    """One-wave workgroups whose slices are 65 to 128 units long move two units per lane in one round: whole rows,
+    rows that end inside a unit and rows that end inside a dword, in copies, reduces and reduce chains."""
+    from msccl.executor import DTYPE_SIZES
+    nbytes = chunk_elems * DTYPE_SIZES[dtype]
+    if mode == "ll" and nbytes % 4:
+        pytest.skip("flag-in-data lines carry whole dwords")
+    for xml in (ir_samples.ring_allreduce_xml(8, 2), ir_samples.allpairs_allreduce_xml(5), ir_samples.RRC_CPY_NOP_XML, ir_samples.ring_allgather_xml(8, 2)):
+        got, want, _, info = run_both(xml, chunk_elems, dtype, seed=chunk_elems % 83, threads=64, slices=slices, **MODES[mode])
+        assert info.threads == 64 and 64 * 16 < info.piece_bytes <= 128 * 16, (info.threads, info.piece_bytes)
+        assert_same(got, want)
+
+
 @pytest.mark.parametrize("knobs", [dict(), dict(slices=1, piece_bytes=4096), dict(threads=256, slices=2), dict(threads=64, slices=3)])
 @pytest.mark.parametrize("dtype,redop", [("bfloat16", "sum"), ("float32", "sum"), ("int32", "max"), ("float16", "prod")])
 @pytest.mark.parametrize("m,stride", [(7, 8), (11, 1), (2, 3)])
