@@ -299,7 +299,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
       h.nops = tb.nops; h.op_begin = tb.op_begin;
       const uint64_t u0 = slice_begin(g.chunk_units, g.slice_grain, g.slices, slice), u1 = slice_begin(g.chunk_units, g.slice_grain, g.slices, slice + 1);
       h.npasses = (unsigned)((u1 - u0 + g.piece_units - 1) / g.piece_units);
-      const uint64_t slice_fifo = (uint64_t)slice * g.slice_fifo_units * fb;  // bytes from the start of the FIFO region (a multiple of 16 on the vector path)
+      const uint64_t slice_fifo = (uint64_t)slice * g.slice_fifo_units * fb;  // bytes from the start of the FIFO region (a multiple of 16)
       const uint64_t area = (uint64_t)kSyncHeaderWords + (uint64_t)slice * g.sync_slice_words;
       const uint64_t heads = area + (uint64_t)ntb * kSyncStrideWords, tails = heads + (uint64_t)ncn * kSyncStrideWords;
       if (tails + (uint64_t)ncn * kSyncStrideWords > 0xffffffffull) return fail(MSCCLX_ERR_CAPACITY, "counter area beyond 32-bit word indices");

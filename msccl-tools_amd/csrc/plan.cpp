@@ -785,7 +785,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   g.sync_words = kSyncHeaderWords + g.sync_slice_words * g.slices;
   const uint64_t sync_bytes = ((kControlWords + 2 * g.sync_words) * 8 + 255) / 256 * 256;  // control block + two areas
   g.fifo_byte_off = sync_bytes;
-  {  // the kernel keeps slot positions as 32-bit offsets (16-byte steps on the vector path, bytes otherwise) and counter positions as 32-bit word indices
+  {  // the kernel keeps slot positions as 32-bit offsets (16-byte steps) and counter positions as 32-bit word indices
     const uint64_t fifo_bytes = g.slice_fifo_units * g.slices * fifo_unit_bytes;
     if (fifo_bytes >= (1ull << 36) || g.sync_words >= (1ull << 31))
       return fail(MSCCLX_ERR_CAPACITY, "the FIFO slots or counters of this geometry exceed what the kernel can address; use fewer slices or a smaller piece_bytes");

@@ -96,7 +96,7 @@ struct DevConn {
 struct Hosted {
   int nops, op_begin;
   unsigned npasses;
-  // Slots: offsets from the start of the FIFO region, in 16-byte steps on the vector path and in bytes otherwise; counters: 64-bit word index
+  // Slots: offsets from the start of the FIFO region, in 16-byte steps; counters: 64-bit word index
   // inside this launch's counter area.  32 bits each, so that the lot is read from LDS in one go.
   uint32_t in_slots, out_slots;    // first slot of the incoming / outgoing connection, in this slice
   uint32_t in_slot_bytes, out_slot_bytes;
@@ -152,7 +152,7 @@ struct KernelParams {
   unsigned char* fifo;
   mscclx_status* host_status;   // pinned host memory
   unsigned long long* prof;     // per-workgroup tick counters of MSCCLX_PROFILE builds, else null
-  uint64_t chunk_units;         // units per chunk; the last one may be partial on the vector path
+  uint64_t chunk_units;         // 16-byte units per chunk; the last one may be partial
   uint64_t chunk_bytes;         // rows of a rank buffer are this far apart
   uint64_t slice_fifo_units;
   uint64_t sync_slice_words;
