@@ -219,12 +219,12 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
         "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
         "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed, flag-in-data lines
-        "c5_chain": (4096, 64, 64, 4096, 1, 1),  # one buffer through 64 ranks: latency bound however big the chunk, most contexts wait
+        "c5_chain": (4096, 64, 64, 4096, 1, 1),  # one buffer through 64 ranks: latency bound however big the chunk, one rank busy at a time: lines
     }
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
-        assert i.protocol == binding.PROTOCOL_CODES["ll" if key == "c5" else "simple"], key
+        assert i.protocol == binding.PROTOCOL_CODES["ll" if key in ("c5", "c5_chain") else "simple"], key
 
 
 def test_geometry_between_the_benchmark_sizes(mscclx_lib):
