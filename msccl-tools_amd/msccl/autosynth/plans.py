@@ -111,3 +111,20 @@ def register_mi355x_plans():
                             interleaved_replication=False, machines=lambda x: x == 4)
     def mi355x_two_level_allreduce_4x8(prog, nodes):
         hierarchical_allreduce(8, 4, "auto")
+
+    # All-pairs over all 16 or 32 ranks between the sizes at which the two-level program wins: its flag-in-data lines at the
+    # small end, its fewer and longer messages at the large one.  fp32, microseconds, all-pairs / two-level -- 16 ranks:
+    # 64 KiB per rank 27 / 27, 128 KiB 27 / 29, 256 KiB 29 / 38, 1 MiB 34 / 46, 4 MiB 67 / 81, 16 MiB 207 / 228, 32 MiB 423 / 427,
+    # 64 MiB 894 / 795; 32 ranks: 128 KiB 48 / 39, 256 KiB 49 / 50, 512 KiB 52 / 59, 1 MiB 58 / 70, 2 MiB 79 / 98, 3 MiB 109 / 129,
+    # 4 MiB 137 / 138, 6 MiB 185 / 179, 16 MiB 450 / 417.
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=256, inplace=True, instances=1,
+                            sizes=('128KiB', '32MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            dependence_nop=True, machines=lambda x: x == 2, priority=1)
+    def mi355x_allpairs_allreduce_2x8(prog, nodes):
+        allreduce_allpairs(16)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=1024, inplace=True, instances=1,
+                            sizes=('256KiB', '4MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            dependence_nop=True, machines=lambda x: x == 4, priority=1)
+    def mi355x_allpairs_allreduce_4x8(prog, nodes):
+        allreduce_allpairs(32)

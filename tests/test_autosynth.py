@@ -156,6 +156,19 @@ def test_mi355x_alltoall_plans(capsys):
     assert load_config()[0].tables.ngpus == 16
 
 
+def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
+    """16 and 32 virtual ranks: all-pairs over all ranks in the middle sizes, the two-level program on either side."""
+    for groups, low, high, chunks in ((2, 128 << 10, 32 << 20, 256), (4, 256 << 10, 4 << 20, 1024)):
+        msccl.init('mi355x', groups, ('allreduce', (0, None)))
+        capsys.readouterr()
+        algos = load_config()
+        two, ap = f'mi355x_two_level_allreduce_{groups}x8', f'mi355x_allpairs_allreduce_{groups}x8'
+        assert [(a.min_bytes, a.max_bytes, a.tables.name) for a in algos] == [(0, low, two), (low, high, ap), (high, float("inf"), two)]
+        mid = select(algos, "allreduce", 1 << 20)
+        assert mid.tables.ngpus == 8 * groups and mid.tables.nchunksperloop == chunks and mid.tables.inplace
+        assert select(algos, "allreduce", 64 << 10).tables.name == two and select(algos, "allreduce", 64 << 20).tables.name == two
+
+
 def test_ef_file_plan(tmp_path, capsys):
     import ir_samples
     f = tmp_path / "ring.xml"

@@ -304,6 +304,33 @@ def test_init_to_run_alltoall_and_large_allgather(capsys):
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(8))
 
 
+@pytest.mark.parametrize("groups,elems", [(2, 251), (4, 65)])
+def test_init_to_run_allpairs_over_groups(groups, elems, capsys):
+    """16 and 32 virtual ranks in the middle sizes: msccl.init picks the all-pairs program over all ranks; int32 sums
+    (exact in any order) of chunks that are no multiple of 16 bytes."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    n = 8 * groups
+    nbytes = n * n * elems * 4                                # per rank
+    msccl.init('mi355x', groups, ('allreduce', nbytes))
+    capsys.readouterr()
+    ar = select(load_config(), "allreduce", nbytes)
+    assert ar.tables.name == f"mi355x_allpairs_allreduce_{groups}x8" and ar.tables.ngpus == n
+    rng = np.random.default_rng(groups)
+    x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64) for _ in range(n)]
+    cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
+    assert cb == elems * 4
+    ex = Executor(ar.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v.astype(np.int32)) for v in x])
+    ex.run(ins, outs)
+    want = sum(x).astype(np.int32)                              # wraps like the device's 32-bit adds
+    assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
+
+
 def test_init_to_run_flow(capsys):
     """msccl.init -> MSCCL_CONFIG index -> select by size -> run: the drop-in path end to end."""
     import os
