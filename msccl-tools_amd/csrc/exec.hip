@@ -27,12 +27,12 @@ namespace mscclx {
 typedef void (*kernel_fn)(const KernelParams);
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // The kernels are compiled in five translation units, two element types each (exec_kernels.hip).
-kernel_fn pick_kernel_group_0(int dtype, int op, bool ll, bool fold, bool ragged);
-kernel_fn pick_kernel_group_1(int dtype, int op, bool ll, bool fold, bool ragged);
-kernel_fn pick_kernel_group_2(int dtype, int op, bool ll, bool fold, bool ragged);
-kernel_fn pick_kernel_group_3(int dtype, int op, bool ll, bool fold, bool ragged);
-kernel_fn pick_kernel_group_4(int dtype, int op, bool ll, bool fold, bool ragged);
-static kernel_fn pick_kernel(int dtype, int op, bool ll, bool fold, bool ragged) {
+kernel_fn pick_kernel_group_0(int dtype, int op, bool ll, int fold, bool ragged);
+kernel_fn pick_kernel_group_1(int dtype, int op, bool ll, int fold, bool ragged);
+kernel_fn pick_kernel_group_2(int dtype, int op, bool ll, int fold, bool ragged);
+kernel_fn pick_kernel_group_3(int dtype, int op, bool ll, int fold, bool ragged);
+kernel_fn pick_kernel_group_4(int dtype, int op, bool ll, int fold, bool ragged);
+static kernel_fn pick_kernel(int dtype, int op, bool ll, int fold, bool ragged) {
   switch (dtype / 2) {
     case 0: return pick_kernel_group_0(dtype, op, ll, fold, ragged);
     case 1: return pick_kernel_group_1(dtype, op, ll, fold, ragged);
@@ -49,6 +49,7 @@ struct DeviceImage {
   std::vector<unsigned char> bytes;
   size_t off_tbs = 0, off_ops = 0, off_extras = 0, off_conns = 0, off_hosting = 0, off_ctxs = 0;
   bool one_each = false;              // workgroup w hosts context w and no other
+  bool long_folds = false;            // some step stands for more folded nops than a lane checks by itself
   std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
   std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
   kernel_fn kernel = nullptr;
@@ -142,8 +143,6 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
   const mscclx_plan* plan = &plan_ref;
   const Geometry& g = plan->geo;
   const bool fold = !g.ll && has_foldable_nops(*plan);
-  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold, plan->chunk_bytes % 16 != 0);
-  if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   DeviceImage* d = img;
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
   std::vector<DevTb> htb(ntb);
@@ -201,6 +200,20 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
     folded_ops.reserve(nop);
     d->dev_op_begin.assign(ntb, 0);
     d->dev_ir_step.clear();
+    d->long_folds = false;
+    // How many nops a step may stand for: as many as its context's own lane checks, or -- where the program has runs of
+    // more than twice that (all-pairs over 16 or 32 ranks) -- as many as the polling wave checks together.  That check
+    // runs on a kernel of its own, whose every step is some 4 % slower: a run of seven is not worth it.
+    size_t longest_run = 0;
+    for (size_t t = 0; fold && t < ntb; ++t) {
+      size_t run = 0;
+      for (int o = plan->tbs[t].op_begin; o < plan->tbs[t].op_end; ++o) {
+        const bool foldable = (hop[o].word & 15u) == MSCCLX_OP_NOP && !(hop[o].word & kOpHasdep) && o + 1 < plan->tbs[t].op_end;
+        run = foldable ? run + 1 : 0;
+        longest_run = std::max(longest_run, run);
+      }
+    }
+    const size_t most_folded = longest_run > 2 * (size_t)kLaneExtraDeps ? (size_t)kMaxExtraDeps : (size_t)kLaneExtraDeps;
     for (size_t t = 0; t < ntb; ++t) {
       const Tb& tb = plan->tbs[t];
       d->dev_op_begin[t] = (int32_t)folded_ops.size();
@@ -209,7 +222,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
       for (int o = tb.op_begin; o < tb.op_end; ++o) {
         DevOp dv = hop[o];
         const bool nop_step = (dv.word & 15u) == MSCCLX_OP_NOP;
-        if (fold && nop_step && !(dv.word & kOpHasdep) && o + 1 < tb.op_end && pending.size() / kExtraDepWords < (size_t)kMaxExtraDeps &&
+        if (fold && nop_step && !(dv.word & kOpHasdep) && o + 1 < tb.op_end && pending.size() / kExtraDepWords < most_folded &&
             dv.dep_nops < 65536 && folded < 255) {
           if (dv.dep_tb >= 0) {
             pending.push_back((uint32_t)dv.dep_tb * kSyncStrideWords);
@@ -221,6 +234,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
         const size_t first = extras.size() / kExtraDepWords;
         if (first >= (1u << 24)) return fail(MSCCLX_ERR_CAPACITY, "too many folded dependencies");
         dv.extra = (uint32_t)(first << 8) | (uint32_t)(pending.size() / kExtraDepWords);
+        if (pending.size() / kExtraDepWords > (size_t)kLaneExtraDeps) d->long_folds = true;
         dv.steps = 1 + folded;
         extras.insert(extras.end(), pending.begin(), pending.end());
         pending.clear();
@@ -286,6 +300,8 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
     hop.swap(fused);
     d->dev_ir_step.swap(fused_ir);
   }
+  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold ? (img->long_folds ? 2 : 1) : 0, plan->chunk_bytes % 16 != 0);
+  if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   // One record per hosted context, in hosting order: where its counters and slots are, its slice's bounds.
   std::vector<DevCtx> ctxs(g.ctx_tb.size());
   {
@@ -454,11 +470,17 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     const bool ll = cfg.protocol == MSCCLX_PROTO_LL;
     const bool fold = !ll && has_foldable_nops(*plan);
     const bool ragged = chunk_bytes % 16 != 0;  // rows may end inside a 16-byte unit: kernels of their own
-    int rc = query_capacity(pick_kernel(dtype, redop, ll, fold, ragged), &num_cus, capacity);
+    int rc = query_capacity(pick_kernel(dtype, redop, ll, fold ? 1 : 0, ragged), &num_cus, capacity);
     if (rc) return rc;
+    if (fold) {  // long runs of folded nops run on a kernel of their own; which one it will be is known when the tables are built
+      int other[kThreadChoices];
+      rc = query_capacity(pick_kernel(dtype, redop, ll, 2, ragged), &num_cus, other);
+      if (rc) return rc;
+      for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
+    }
     if (cfg.protocol == MSCCLX_PROTO_AUTO && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
       int other[kThreadChoices];
-      rc = query_capacity(pick_kernel(dtype, redop, true, false, ragged), &num_cus, other);
+      rc = query_capacity(pick_kernel(dtype, redop, true, 0, ragged), &num_cus, other);
       if (rc) return rc;
       for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
     }

@@ -634,19 +634,33 @@ __device__ __forceinline__ bool extras_ready(const Context& c, const Hosted& h, 
   const uint32_t n = c.extra & 255u;
   const uint2* const e = (const uint2*)p.extra_deps + (c.extra >> 8);
   const u64* const flags = p.sync_cur + h.flags;
-  uint2 entry[kMaxExtraDeps];
+  uint2 entry[kLaneExtraDeps];
 #pragma unroll
-  for (int k = 0; k < kMaxExtraDeps; ++k)
+  for (int k = 0; k < kLaneExtraDeps; ++k)
     if ((uint32_t)k < n) entry[k] = e[k];
-  u64 v[kMaxExtraDeps];
+  u64 v[kLaneExtraDeps];
 #pragma unroll
-  for (int k = 0; k < kMaxExtraDeps; ++k)
+  for (int k = 0; k < kLaneExtraDeps; ++k)
     if ((uint32_t)k < n) v[k] = load_counter(flags + entry[k].x);
   bool ok = true;
 #pragma unroll
-  for (int k = 0; k < kMaxExtraDeps; ++k)
+  for (int k = 0; k < kLaneExtraDeps; ++k)
     if ((uint32_t)k < n) ok = ok && v[k] >= (u64)(c.pass * (entry[k].y >> 16) + (entry[k].y & 0xffffu));
   return ok;
+}
+
+// The same for a context with more folded dependencies than that (up to kMaxExtraDeps = the wave's width): the whole
+// polling wave checks them, a dependency per lane -- still two rounds of loads.  Called by all 64 lanes; `owner` is the
+// lane whose context it is, and every lane gets the answer.
+__device__ __forceinline__ bool extras_ready_together(const Context& c, const Hosted& h, const KernelParams& p, int owner, int lane) {
+  const uint32_t extra = (uint32_t)__shfl((int)c.extra, owner), first_flag = (uint32_t)__shfl((int)h.flags, owner);
+  const unsigned pass = (unsigned)__shfl((int)c.pass, owner);
+  bool ok = true;
+  if ((uint32_t)lane < (extra & 255u)) {
+    const uint2 entry = ((const uint2*)p.extra_deps)[(extra >> 8) + (uint32_t)lane];
+    ok = load_counter(p.sync_cur + first_flag + entry.x) >= (u64)(pass * (entry.y >> 16) + (entry.y & 0xffffu));
+  }
+  return __ballot(!ok) == 0;
 }
 
 // FOLD kernels: an `re` with several sources (in_addr = their distance in bytes, cnt = how many).
@@ -774,7 +788,7 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
 // incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool LL, bool FOLD, bool RAGGED>
+template <class R, bool LL, int FOLD, bool RAGGED>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
   constexpr int W = 16;
@@ -1304,7 +1318,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
 // share the resident workgroups without deadlock.
 // FOLD: steps may carry the dependencies of nop steps folded into them (a kernel of its own, so that
 // programs without such steps do not pay for the check in the poll loop).
-template <class R, bool LL, bool FOLD, bool RAGGED>
+template <class R, bool LL, int FOLD, bool RAGGED>
 __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
   // The number of launches so far is kept on the device (control word 0) and is advanced by the
   // last workgroup to finish, so a launch carries no host-side state and the same launch can be
@@ -1389,7 +1403,16 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
           const u64 v2 = c.w2 ? load_counter(c.w2) : 0;
           ready = (!c.w0 || v0 >= c.t0) && (!c.w2 || v2 >= c.t2) &&
                   (!watch1 || (LL ? (uint32_t)(v1 >> 32) == (uint32_t)c.t1 : v1 >= c.t1));
-          if (FOLD && ready && (c.extra & 255u)) ready = extras_ready(c, h, p);  // the nops folded into this step
+          if (FOLD && ready && (c.extra & 255u) && (c.extra & 255u) <= (uint32_t)kLaneExtraDeps) ready = extras_ready(c, h, p);  // the nops folded into this step
+        }
+        if (FOLD == 2) {  // long runs of folded nops, context by context
+          u64 long_runs = __ballot(ready && (c.extra & 255u) > (uint32_t)kLaneExtraDeps);
+          while (long_runs) {
+            const int owner = __ffsll((long long)long_runs) - 1;
+            long_runs &= long_runs - 1;
+            const bool all_there = extras_ready_together(c, h, p, owner, lane);
+            if (lane == owner) ready = all_there;
+          }
         }
         bool progressed = false;
         if (ready && !c.moves) {  // nothing to copy: the step is complete as soon as it may start
@@ -1551,12 +1574,15 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 typedef void (*kernel_fn)(const KernelParams);
 
 // ragged: chunks that are no multiple of 16 bytes -- rows may end inside a unit; the other kernels carry none of that
-template <int DT, int OP, bool RAGGED> kernel_fn pick_variant(bool ll, bool fold) {
-  if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, false, RAGGED> : nullptr;
-  if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, true, RAGGED>;
-  return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, false, RAGGED>;
+// fold: 0 = no step stands for folded nops, 1 = some do, at most kLaneExtraDeps each, 2 = some for more (the check
+// of those costs scalar registers the other programs' poll loop has no room for: a kernel of its own)
+template <int DT, int OP, bool RAGGED> kernel_fn pick_variant(bool ll, int fold) {
+  if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, 0, RAGGED> : nullptr;
+  if (fold == 2) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 2, RAGGED>;
+  if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 1, RAGGED>;
+  return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 0, RAGGED>;
 }
-template <int DT> kernel_fn pick_op(int op, bool ll, bool fold, bool ragged) {
+template <int DT> kernel_fn pick_op(int op, bool ll, int fold, bool ragged) {
   switch (op) {
     case MSCCLX_SUM: return (ragged ? pick_variant<DT, MSCCLX_SUM, true>(ll, fold) : pick_variant<DT, MSCCLX_SUM, false>(ll, fold));
     case MSCCLX_PROD: return (ragged ? pick_variant<DT, MSCCLX_PROD, true>(ll, fold) : pick_variant<DT, MSCCLX_PROD, false>(ll, fold));

@@ -11,7 +11,7 @@
 
 namespace mscclx {
 
-kernel_fn MSCCLX_PASTE(pick_kernel_group_, MSCCLX_KERNEL_GROUP)(int dtype, int op, bool ll, bool fold, bool ragged) {
+kernel_fn MSCCLX_PASTE(pick_kernel_group_, MSCCLX_KERNEL_GROUP)(int dtype, int op, bool ll, int fold, bool ragged) {
   static_assert(2 * MSCCLX_KERNEL_GROUP + 1 < MSCCLX_NUM_DTYPES, "two element types per group");
   if (dtype == 2 * MSCCLX_KERNEL_GROUP) return pick_op<2 * MSCCLX_KERNEL_GROUP>(op, ll, fold, ragged);
   if (dtype == 2 * MSCCLX_KERNEL_GROUP + 1) return pick_op<2 * MSCCLX_KERNEL_GROUP + 1>(op, ll, fold, ragged);

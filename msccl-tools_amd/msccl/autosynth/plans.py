@@ -112,19 +112,19 @@ def register_mi355x_plans():
     def mi355x_two_level_allreduce_4x8(prog, nodes):
         hierarchical_allreduce(8, 4, "auto")
 
-    # All-pairs over all 16 or 32 ranks between the sizes at which the two-level program wins: its flag-in-data lines at the
-    # small end, its fewer and longer messages at the large one.  fp32, microseconds, all-pairs / two-level -- 16 ranks:
-    # 64 KiB per rank 27 / 27, 128 KiB 27 / 29, 256 KiB 29 / 38, 1 MiB 34 / 46, 4 MiB 67 / 81, 16 MiB 207 / 228, 32 MiB 423 / 427,
-    # 64 MiB 894 / 795; 32 ranks: 128 KiB 48 / 39, 256 KiB 49 / 50, 512 KiB 52 / 59, 1 MiB 58 / 70, 2 MiB 79 / 98, 3 MiB 109 / 129,
-    # 4 MiB 137 / 138, 6 MiB 185 / 179, 16 MiB 450 / 417.
+    # All-pairs over all 16 or 32 ranks up to the sizes at which the two-level program's fewer and longer messages win (and, on
+    # 32 ranks, from the size below which its flag-in-data lines do).  fp32, microseconds, all-pairs / two-level -- 16 ranks:
+    # 4 to 64 KiB per rank 22-23 / 26-28, 256 KiB 24 / 38, 1 MiB 29 / 46, 4 MiB 62 / 82, 16 MiB 204 / 227, 24 MiB 335 / 338,
+    # 32 MiB 433 / 418; 32 ranks: 4 KiB 37 / 32, 32 KiB 36 / 34, 64 KiB 35 / 35, 128 KiB 34 / 39, 256 KiB 35 / 51, 1 MiB 45 / 70,
+    # 4 MiB 119 / 139, 6 MiB 182 / 179, 8 MiB 231 / 229.
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=256, inplace=True, instances=1,
-                            sizes=('128KiB', '32MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=(0, '24MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 2, priority=1)
     def mi355x_allpairs_allreduce_2x8(prog, nodes):
         allreduce_allpairs(16)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=1024, inplace=True, instances=1,
-                            sizes=('256KiB', '4MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=('64KiB', '5MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 4, priority=1)
     def mi355x_allpairs_allreduce_4x8(prog, nodes):
         allreduce_allpairs(32)

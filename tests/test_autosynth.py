@@ -157,16 +157,17 @@ def test_mi355x_alltoall_plans(capsys):
 
 
 def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
-    """16 and 32 virtual ranks: all-pairs over all ranks in the middle sizes, the two-level program on either side."""
-    for groups, low, high, chunks in ((2, 128 << 10, 32 << 20, 256), (4, 256 << 10, 4 << 20, 1024)):
+    """16 and 32 virtual ranks: all-pairs over all ranks up to 24 MiB per rank (16 ranks) or between 64 KiB and 5 MiB
+    (32 ranks), the two-level program elsewhere."""
+    for groups, windows, chunks in ((2, [(0, 24 << 20, 'allpairs'), (24 << 20, float("inf"), 'two_level')], 256),
+                                    (4, [(0, 64 << 10, 'two_level'), (64 << 10, 5 << 20, 'allpairs'), (5 << 20, float("inf"), 'two_level')], 1024)):
         msccl.init('mi355x', groups, ('allreduce', (0, None)))
         capsys.readouterr()
         algos = load_config()
-        two, ap = f'mi355x_two_level_allreduce_{groups}x8', f'mi355x_allpairs_allreduce_{groups}x8'
-        assert [(a.min_bytes, a.max_bytes, a.tables.name) for a in algos] == [(0, low, two), (low, high, ap), (high, float("inf"), two)]
+        assert [(a.min_bytes, a.max_bytes, a.tables.name) for a in algos] == [(lo, hi, f'mi355x_{kind}_allreduce_{groups}x8') for lo, hi, kind in windows]
         mid = select(algos, "allreduce", 1 << 20)
         assert mid.tables.ngpus == 8 * groups and mid.tables.nchunksperloop == chunks and mid.tables.inplace
-        assert select(algos, "allreduce", 64 << 10).tables.name == two and select(algos, "allreduce", 64 << 20).tables.name == two
+        assert select(algos, "allreduce", 64 << 20).tables.name == f'mi355x_two_level_allreduce_{groups}x8'
 
 
 def test_ef_file_plan(tmp_path, capsys):
