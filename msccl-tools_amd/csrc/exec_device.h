@@ -411,8 +411,8 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
 }
 
 // dst = ((dst (+) a0) (+) a1) ... (+) a[m-1] over n units of W bytes; source k starts `stride` bytes
-// after source k-1.  All sources of a unit are in flight together and folded in order, so the result
-// is bit for bit that of m reduce steps -- which would read and write dst m times.
+// after source k-1.  The sources of a unit are in flight together, eight at a time, and folded in order, so the
+// result is bit for bit that of m reduce steps -- which would read and write dst m times.
 template <class R, int W, bool NT1>
 __device__ __forceinline__ void move_reduce_many(unsigned char* dst, const unsigned char* a, uint32_t stride, int m, uint32_t n, uint32_t clip) {
   typedef Access<W> A;
@@ -425,13 +425,15 @@ __device__ __forceinline__ void move_reduce_many(unsigned char* dst, const unsig
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(a, (uint32_t)(m - 1) * stride + bytes);
   for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
     word acc = A::template ld<XL>(rd, (int)(i * W));
-    word s[kMaxReduceSources];
+    for (int first = 0; first < m; first += kReduceSourcesAtOnce) {  // (one round for the 7 peers of an 8-rank all-pairs program)
+      word s[kReduceSourcesAtOnce];
 #pragma unroll
-    for (int k = 0; k < kMaxReduceSources; ++k)
-      if (k < m) s[k] = A::template lds<XL>(rs, (int)(i * W), (int)((uint32_t)k * stride));
+      for (int k = 0; k < kReduceSourcesAtOnce; ++k)
+        if (first + k < m) s[k] = A::template lds<XL>(rs, (int)(i * W), (int)((uint32_t)(first + k) * stride));
 #pragma unroll
-    for (int k = 0; k < kMaxReduceSources; ++k)
-      if (k < m) acc = R::combine(acc, s[k]);
+      for (int k = 0; k < kReduceSourcesAtOnce; ++k)
+        if (first + k < m) acc = R::combine(acc, s[k]);
+    }
     A::template st<X1>(rd, (int)(i * W), acc);
   }
 }

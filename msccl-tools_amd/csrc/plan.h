@@ -73,7 +73,8 @@ constexpr int kOpCntShift = 8;
 // A run of `re` steps with one chunk each, the same destination and sources a fixed distance apart is
 // done as one step on the device -- dst = (..((dst + src0) + src1)..) + src[m-1]: an `re` whose
 // in_addr holds the distance between sources in bytes (0 for an ordinary `re`) and whose cnt holds m.
-constexpr int kMaxReduceSources = 8;
+constexpr int kMaxReduceSources = 64;      // sources of one such step, at most ...
+constexpr int kReduceSourcesAtOnce = 8;    // ... of which this many are in flight together
 constexpr int kMaxExtraDeps = 64;        // nop steps folded into the step that follows them, at most: one for each lane of the polling wave
 constexpr int kLaneExtraDeps = 6;        // up to this many a context's own lane checks; longer runs the wave checks together
 constexpr int kExtraDepWords = 2;        // one folded dependency: counter word (from the slice's first flag); step + 1 | steps per pass of that threadblock << 16

@@ -112,19 +112,19 @@ def register_mi355x_plans():
     def mi355x_two_level_allreduce_4x8(prog, nodes):
         hierarchical_allreduce(8, 4, "auto")
 
-    # All-pairs over all 16 or 32 ranks up to the sizes at which the two-level program's fewer and longer messages win (and, on
-    # 32 ranks, from the size below which its flag-in-data lines do).  fp32, microseconds, all-pairs / two-level -- 16 ranks:
-    # 4 to 64 KiB per rank 22-23 / 26-28, 256 KiB 24 / 38, 1 MiB 29 / 46, 4 MiB 62 / 82, 16 MiB 204 / 227, 24 MiB 335 / 338,
-    # 32 MiB 433 / 418; 32 ranks: 4 KiB 37 / 32, 32 KiB 36 / 34, 64 KiB 35 / 35, 128 KiB 34 / 39, 256 KiB 35 / 51, 1 MiB 45 / 70,
-    # 4 MiB 119 / 139, 6 MiB 182 / 179, 8 MiB 231 / 229.
+    # All-pairs over all 16 or 32 ranks up to the sizes at which the two-level program's fewer and longer messages win; below
+    # 4 / 16 KiB per rank its 256 / 1024 chunks would be smaller than an element.  fp32, microseconds, all-pairs / two-level --
+    # 16 ranks: 16 KiB per rank 21 / 26, 1 MiB 28 / 47, 4 MiB 62 / 82, 16 MiB 202 / 228, 24 MiB 336 / 338, 32 MiB 427 / 420;
+    # 32 ranks: 16 KiB 31 / 33, 64 KiB 30 / 35, 256 KiB 35 / 51, 1 MiB 42 / 70, 4 MiB 114 / 137, 6 MiB 174 / 180, 8 MiB 223 / 227,
+    # 16 MiB 450 / 417.
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=256, inplace=True, instances=1,
-                            sizes=(0, '24MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=('4KiB', '24MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 2, priority=1)
     def mi355x_allpairs_allreduce_2x8(prog, nodes):
         allreduce_allpairs(16)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=1024, inplace=True, instances=1,
-                            sizes=('64KiB', '5MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=('16KiB', '8MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 4, priority=1)
     def mi355x_allpairs_allreduce_4x8(prog, nodes):
         allreduce_allpairs(32)

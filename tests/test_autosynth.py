@@ -157,10 +157,10 @@ def test_mi355x_alltoall_plans(capsys):
 
 
 def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
-    """16 and 32 virtual ranks: all-pairs over all ranks up to 24 MiB per rank (16 ranks) or between 64 KiB and 5 MiB
+    """16 and 32 virtual ranks: all-pairs over all ranks from 4 KiB to 24 MiB per rank (16 ranks) or from 16 KiB to 8 MiB
     (32 ranks), the two-level program elsewhere."""
-    for groups, windows, chunks in ((2, [(0, 24 << 20, 'allpairs'), (24 << 20, float("inf"), 'two_level')], 256),
-                                    (4, [(0, 64 << 10, 'two_level'), (64 << 10, 5 << 20, 'allpairs'), (5 << 20, float("inf"), 'two_level')], 1024)):
+    for groups, windows, chunks in ((2, [(0, 4 << 10, 'two_level'), (4 << 10, 24 << 20, 'allpairs'), (24 << 20, float("inf"), 'two_level')], 256),
+                                    (4, [(0, 16 << 10, 'two_level'), (16 << 10, 8 << 20, 'allpairs'), (8 << 20, float("inf"), 'two_level')], 1024)):
         msccl.init('mi355x', groups, ('allreduce', (0, None)))
         capsys.readouterr()
         algos = load_config()

@@ -331,7 +331,7 @@ def test_slices_of_up_to_two_units_per_lane(chunk_elems, dtype, slices, mode):
 
 @pytest.mark.parametrize("knobs", [dict(), dict(slices=1, piece_bytes=4096), dict(threads=256, slices=2), dict(threads=64, slices=3)])
 @pytest.mark.parametrize("dtype,redop", [("bfloat16", "sum"), ("float32", "sum"), ("int32", "max"), ("float16", "prod")])
-@pytest.mark.parametrize("m,stride", [(7, 8), (11, 1), (2, 3)])
+@pytest.mark.parametrize("m,stride", [(7, 8), (11, 1), (2, 3), (31, 1), (17, 2)])
 def test_reduce_chains_as_one_step(m, stride, dtype, redop, knobs):
     """Runs of reduce steps into one destination are done as one step with several sources (at most 8:
     11 in a row make two), in the order of the IR -- which the rounding of bfloat16 sums and fp16 products
