@@ -313,6 +313,18 @@ def test_partial_units_under_explicit_geometries(knobs, protocol):
         assert_same(got, want)
 
 
+@pytest.mark.parametrize("knobs", [dict(), dict(slices=2, workgroups=40, threads=64), dict(threads=256, slices=3), dict(staging=1, slices=4, workgroups=300)])
+def test_long_nop_runs_and_reduce_chains(knobs):
+    """All-pairs over 16 ranks: every threadblock waits for 15 peers through runs of 14 nops, which one step stands for
+    (its dependencies checked by the polling wave together, also where a workgroup hosts many contexts), and folds
+    their 15 chunks with one step of 15 sources."""
+    from msccl.programs import catalog
+    xml = catalog.allpairs_allreduce(16, 1)
+    for dtype, elems in (("float32", 33), ("bfloat16", 1001)):
+        got, want, _, info = run_both(xml, elems, dtype, seed=5, protocol="simple", **knobs)
+        assert_same(got, want)
+
+
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("chunk_elems,dtype,slices", [(4100, "float32", 16), (14001, "float16", 16), (2047, "uint8", 1), (261, "float32", 1),
                                                       (20000, "uint8", 16), (1025, "float64", 6), (509, "int32", 1)])
