@@ -187,6 +187,8 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
           dv.word |= kOpInPlace;
           dv.in_addr = (uint64_t)(uintptr_t)bufs[(size_t)sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf)] +
                        (uint64_t)(from_src ? sender.srcoff : sender.dstoff) * plan->chunk_bytes;
+          const Tb& sender_tb = plan->tbs[plan->conns[tb.recv_conn].send_tb];
+          if (from_src && op.match_send == sender_tb.op_begin && sender.depid < 0) dv.steps |= kStepsPayloadAtLaunch;
         }
       }
     }
@@ -235,7 +237,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
         if (first >= (1u << 24)) return fail(MSCCLX_ERR_CAPACITY, "too many folded dependencies");
         dv.extra = (uint32_t)(first << 8) | (uint32_t)(pending.size() / kExtraDepWords);
         if (pending.size() / kExtraDepWords > (size_t)kLaneExtraDeps) d->long_folds = true;
-        dv.steps = 1 + folded;
+        dv.steps = (dv.steps & kStepsPayloadAtLaunch) | (1 + folded);
         extras.insert(extras.end(), pending.begin(), pending.end());
         pending.clear();
         folded = 0;

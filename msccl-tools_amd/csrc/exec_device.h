@@ -705,7 +705,7 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     if (LL) {
       c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
       c.t1 = ll_flag(epoch, c.rseq);
-    } else {
+    } else if (!(in_place && (op.steps & kStepsPayloadAtLaunch))) {
       c.w1 = p.sync_cur + h.head_in;
       c.t1 = c.rseq + 1;
     }
@@ -1219,7 +1219,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
     {  // what the step waits for: a step of another threadblock, the incoming message, a free outgoing slot -- one round of loads for all
       const u64* const w0 = op.dep_tb >= 0 ? flags + (uint32_t)op.dep_tb * kSyncStrideWords : nullptr;
       const u64 t0 = (u64)pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1;
-      const u64* const w1 = rcv_bit ? in_head : nullptr;
+      const u64* const w1 = (rcv_bit && !(op.steps & kStepsPayloadAtLaunch)) ? in_head : nullptr;  // (the bit is only set on payloads read in place)
       const u64 t1 = (u64)rseq + 1;
       const u64* const w2 = (snd_bit && sseq >= depth) ? out_tail : nullptr;
       const u64 t2 = (u64)sseq + 1 - depth;

@@ -70,6 +70,11 @@ struct DevOp {
 static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
 constexpr uint32_t kOpHasdep = 1u << 4, kOpOutStaged = 1u << 5, kOpNtStore = 1u << 6, kOpInPlace = 1u << 7;
 constexpr int kOpCntShift = 8;
+// Bit 31 of DevOp::steps, on a receive that reads its payload in place: the matching send is the first step of its
+// threadblock and waits for nothing, so the payload is what the sender's buffer holds when the launch starts --
+// there is no announcement to wait for.  (Every later writer of those chunks comes after this receive, or the
+// payload would not be read in place at all; and a step without predecessors lies on no path between two steps.)
+constexpr uint32_t kStepsPayloadAtLaunch = 1u << 31;
 // A run of `re` steps with one chunk each, the same destination and sources a fixed distance apart is
 // done as one step on the device -- dst = (..((dst + src0) + src1)..) + src[m-1]: an `re` whose
 // in_addr holds the distance between sources in bytes (0 for an ordinary `re`) and whose cnt holds m.
