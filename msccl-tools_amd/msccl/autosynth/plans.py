@@ -92,15 +92,15 @@ def register_mi355x_plans():
     def mi355x_ring_allgather(prog, nodes):
         allgather_ring(size=8, channels=1)
 
-    # One group of 8: the one-step all-to-all, every message read where its sender keeps it (8 KiB to 1 MiB per rank
-    # 8-10 us, 16 MiB 52 us, 64 MiB 204 us = 66 % of the HBM peak, 256 MiB 715 us = 75 %; instances make no difference).
-    @register_msccl_program(fully_connected(8), 'alltoall', 'mi355x', machines=one)
+    # The one-step all-to-all, every message read where its sender keeps it, for any number of groups: 8 ranks 8-10 us from
+    # 8 KiB to 1 MiB per rank, 16 MiB 52 us, 64 MiB 204 us = 66 % of the HBM peak, 256 MiB 715 us = 75 % (instances make no
+    # difference).  The hierarchical program gathers per destination group first, which pays on links between machines; between
+    # virtual ranks of one GPU it is a second pass over the data.  uint8, microseconds, one-step / hierarchical -- 16 ranks:
+    # 64 KiB per rank 9 / 15, 1 MiB 12 / 23, 16 MiB 116 / 135, 64 MiB 399 / 515; 32 ranks: 9 / 21, 19 / 38, 203 / 298, 793 / 1178;
+    # 64 ranks: 12 / 38, 31 / 70, 407 / 720 (16 MiB).
+    @register_msccl_program(fully_connected(8), 'alltoall', 'mi355x', machines=lambda x: 1 <= x <= 8)
     def mi355x_alltoall_allpairs(prog, nodes):
-        alltoall_allpairs(8)
-
-    @register_msccl_program(fully_connected(8), 'alltoall', 'mi355x', machines=lambda x: 2 <= x <= 8)
-    def mi355x_alltoall_hierarchical(prog, nodes):
-        alltoall_hierarchical(num_nodes=nodes, gpus_per_node=8)
+        alltoall_allpairs(8 * nodes)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=16, inplace=True, instances=2,
                             interleaved_replication=False, machines=lambda x: x == 2)

@@ -36,7 +36,7 @@ def test_msccl_init(capsys):
 
     msccl.init('mi355x', 2, ('alltoall', '1MB'))
     out, _ = capsys.readouterr()
-    assert 'mi355x_alltoall_hierarchical' in out
+    assert 'mi355x_alltoall_allpairs' in out
     assert 'MSCCL_CONFIG' in os.environ
     assert 'NCCL_IB_AR_THRESHOLD' not in os.environ
     assert os.environ['NCCL_ALGO'] == 'MSCCL,RING,TREE'
@@ -145,15 +145,19 @@ def test_mi355x_allgather_windows(capsys):
 
 
 def test_mi355x_alltoall_plans(capsys):
-    """One group of 8 virtual ranks: the one-step all-to-all; two to eight groups: the hierarchical one."""
+    """The one-step all-to-all for any number of groups of 8 virtual ranks (between ranks of one GPU the hierarchical
+    program's gathering step is a second pass over the data); the ndv4 machine type keeps msccl-tools' hierarchical plans."""
     msccl.init('mi355x', 1, ('alltoall', '1MB'))
     assert 'mi355x_alltoall_allpairs' in capsys.readouterr().out
     (a,) = load_config()
     assert a.tables.coll == "alltoall" and a.tables.ngpus == 8 and not a.tables.inplace
     assert a.tables.nops == 2 * 8 * 7 + 8      # a send and a receive for every pair, and every rank's copy of its own chunk
     msccl.init('mi355x', 2, ('alltoall', '1MB'))
-    assert 'mi355x_alltoall_hierarchical' in capsys.readouterr().out
-    assert load_config()[0].tables.ngpus == 16
+    assert 'mi355x_alltoall_allpairs' in capsys.readouterr().out
+    (a,) = load_config()
+    assert a.tables.ngpus == 16 and a.tables.nops == 2 * 16 * 15 + 16
+    msccl.init('ndv4', 8, ('alltoall', '2MB'))
+    assert 'ndv4_alltoall_hierarchical' in capsys.readouterr().out
 
 
 def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):

@@ -331,6 +331,31 @@ def test_init_to_run_allpairs_over_groups(groups, elems, capsys):
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
 
 
+def test_init_to_run_alltoall_over_two_groups(capsys):
+    """16 virtual ranks: msccl.init picks the one-step all-to-all here too -- a block transpose, chunks of 1003 int32."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    n, e = 16, 1003
+    nbytes = n * e * 4
+    msccl.init('mi355x', 2, ('alltoall', nbytes))
+    capsys.readouterr()
+    a2a = select(load_config(), "alltoall", nbytes)
+    assert a2a.tables.name == "mi355x_alltoall_allpairs" and a2a.tables.ngpus == n
+    rng = np.random.default_rng(16)
+    x = [rng.integers(-2 ** 31, 2 ** 31, n * e, dtype=np.int64).astype(np.int32) for _ in range(n)]
+    cb = a2a.bytes_per_rank_to_chunk_bytes(nbytes)
+    assert cb == e * 4
+    ex = Executor(a2a.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v) for v in x])
+    ex.run(ins, outs)
+    for r in range(n):
+        assert np.array_equal(res[r].cpu().numpy(), np.concatenate([x[s][r * e:(r + 1) * e] for s in range(n)])), r
+
+
 def test_init_to_run_flow(capsys):
     """msccl.init -> MSCCL_CONFIG index -> select by size -> run: the drop-in path end to end."""
     import os
