@@ -82,15 +82,18 @@ def register_mi355x_plans():
     # All-gather, int32, microseconds by bytes per rank (all-pairs / ring x 4 instances): 1 MiB 18 / 31, 2 MB 26 / 51,
     # 4 MiB 67 / 78, 8 MiB 136 / 144, 12 MB 215 / 212, 16 MiB 287 / 276, 32 MB 570 / 529.  Both move the same bytes; all-pairs
     # is one hand-off deep, the ring seven, and the ring's pieces stream better at the large end.
+    # Two and four groups, all 16 or 32 ranks in one all-pairs program or one ring, the same way -- 16 ranks: 64 KiB per rank
+    # 12 / 33, 1 MiB 50 / 82, 4 MiB 271 / 294, 8 MiB 565 / 579, 16 MiB 1152 / 1150; 32 ranks: 64 KiB 19 / 70, 1 MiB 297 / 299,
+    # 4 MiB 1145 / 1183, 8 MiB 2343 / 2359, 16 MiB 5038 / 4705.
     @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=1,
-                            sizes=(0, '12MB'), threadblock_policy=manual, machines=one)
+                            sizes=(0, '12MB'), threadblock_policy=manual, machines=lambda x: x in (1, 2, 4))
     def mi355x_allpairs_allgather(prog, nodes):
-        allgather_allpairs(8)
+        allgather_allpairs(8 * nodes)
 
     @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=4,
-                            sizes=('12MB', None), threadblock_policy=manual, machines=one)
+                            sizes=('12MB', None), threadblock_policy=manual, machines=lambda x: x in (1, 2, 4))
     def mi355x_ring_allgather(prog, nodes):
-        allgather_ring(size=8, channels=1)
+        allgather_ring(size=8 * nodes, channels=1)
 
     # The one-step all-to-all, every message read where its sender keeps it, for any number of groups: 8 ranks 8-10 us from
     # 8 KiB to 1 MiB per rank, 16 MiB 52 us, 64 MiB 204 us = 66 % of the HBM peak, 256 MiB 715 us = 75 % (instances make no

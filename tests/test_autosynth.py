@@ -142,6 +142,12 @@ def test_mi355x_allgather_windows(capsys):
     assert small.tables.ntbs == 8 * 7 and small.tables.nops == 8 * 14 and small.tables.nchunksperloop == 8   # a threadblock per peer: one send, one receive
     assert large.tables.nchunksperloop == 32                                              # 8 chunks x 4 instances
     assert select(algos, "allgather", 1 << 20) is small and select(algos, "allgather", 64 << 20) is large
+    # two groups: the same two programs over all 16 ranks
+    msccl.init('mi355x', 2, ('allgather', (0, None)))
+    capsys.readouterr()
+    small, large = load_config()
+    assert (small.tables.name, small.tables.ngpus, small.tables.ntbs) == ('mi355x_allpairs_allgather', 16, 16 * 15)
+    assert (large.tables.name, large.tables.ngpus, large.tables.nchunksperloop) == ('mi355x_ring_allgather', 16, 64)
 
 
 def test_mi355x_alltoall_plans(capsys):

@@ -331,6 +331,30 @@ def test_init_to_run_allpairs_over_groups(groups, elems, capsys):
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
 
 
+def test_init_to_run_allgather_over_two_groups(capsys):
+    """16 virtual ranks: the all-pairs all-gather below 12 MB per rank -- every output is the concatenation of the inputs."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    n, e = 16, 2501
+    nbytes = e * 4
+    msccl.init('mi355x', 2, ('allgather', nbytes))
+    capsys.readouterr()
+    ag = select(load_config(), "allgather", nbytes)
+    assert ag.tables.name == "mi355x_allpairs_allgather" and ag.tables.ngpus == n
+    rng = np.random.default_rng(61)
+    x = [rng.integers(-2 ** 31, 2 ** 31, e, dtype=np.int64).astype(np.int32) for _ in range(n)]
+    cb = ag.bytes_per_rank_to_chunk_bytes(nbytes)
+    ex = Executor(ag.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v) for v in x])
+    ex.run(ins, outs)
+    want = np.concatenate(x)
+    assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
+
+
 def test_init_to_run_alltoall_over_two_groups(capsys):
     """16 virtual ranks: msccl.init picks the one-step all-to-all here too -- a block transpose, chunks of 1003 int32."""
     import os
