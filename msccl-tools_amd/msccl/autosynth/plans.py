@@ -121,10 +121,17 @@ def register_mi355x_plans():
     # 32 ranks: 16 KiB 31 / 33, 64 KiB 30 / 35, 256 KiB 35 / 51, 1 MiB 42 / 70, 4 MiB 114 / 137, 6 MiB 174 / 180, 8 MiB 223 / 227,
     # 16 MiB 450 / 417.
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=256, inplace=True, instances=1,
-                            sizes=('4KiB', '24MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=('4KiB', '16MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 2, priority=1)
     def mi355x_allpairs_allreduce_2x8(prog, nodes):
         allreduce_allpairs(16)
+
+    # 16 ranks, large messages: one ring over all ranks (4 instances) against the two-level program, 16 MiB per rank 194 / 212,
+    # 32 MiB 377 / 412, 128 MiB 1403 / 1498 (all-pairs: 202, 427).  On 32 ranks the two are level (128 MiB 2890 / 2917, 8 MiB 235 / 219).
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=16, inplace=True, instances=4,
+                            sizes=('16MiB', None), threadblock_policy=manual, machines=lambda x: x == 2, priority=1)
+    def mi355x_ring_allreduce_2x8(prog, nodes):
+        allreduce_ring(size=16, channels=1)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=1024, inplace=True, instances=1,
                             sizes=('16KiB', '8MiB'), threadblock_policy=manual, interleaved_replication=False,

@@ -167,9 +167,9 @@ def test_mi355x_alltoall_plans(capsys):
 
 
 def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
-    """16 and 32 virtual ranks: all-pairs over all ranks from 4 KiB to 24 MiB per rank (16 ranks) or from 16 KiB to 8 MiB
-    (32 ranks), the two-level program elsewhere."""
-    for groups, windows, chunks in ((2, [(0, 4 << 10, 'two_level'), (4 << 10, 24 << 20, 'allpairs'), (24 << 20, float("inf"), 'two_level')], 256),
+    """16 and 32 virtual ranks: all-pairs over all ranks from 4 KiB to 16 MiB per rank (16 ranks; one ring over all ranks
+    above) or from 16 KiB to 8 MiB (32 ranks), the two-level program elsewhere."""
+    for groups, windows, chunks in ((2, [(0, 4 << 10, 'two_level'), (4 << 10, 16 << 20, 'allpairs'), (16 << 20, float("inf"), 'ring')], 256),
                                     (4, [(0, 16 << 10, 'two_level'), (16 << 10, 8 << 20, 'allpairs'), (8 << 20, float("inf"), 'two_level')], 1024)):
         msccl.init('mi355x', groups, ('allreduce', (0, None)))
         capsys.readouterr()
@@ -177,7 +177,7 @@ def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
         assert [(a.min_bytes, a.max_bytes, a.tables.name) for a in algos] == [(lo, hi, f'mi355x_{kind}_allreduce_{groups}x8') for lo, hi, kind in windows]
         mid = select(algos, "allreduce", 1 << 20)
         assert mid.tables.ngpus == 8 * groups and mid.tables.nchunksperloop == chunks and mid.tables.inplace
-        assert select(algos, "allreduce", 64 << 20).tables.name == f'mi355x_two_level_allreduce_{groups}x8'
+        assert select(algos, "allreduce", 64 << 20).tables.name == f'mi355x_{windows[-1][2]}_allreduce_{groups}x8'
 
 
 def test_ef_file_plan(tmp_path, capsys):
