@@ -143,34 +143,46 @@ def test_nan_operands(dtype, redop):
         assert np.array_equal(got[~rn].view(np.uint8), ref[~rn].view(np.uint8)), r  # and the same bits everywhere else
 
 
+SIXTEEN_BIT_PARTNERS = {
+    "bfloat16": [0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x3F80, 0xBF80, 0x3F81, 0x3B80, 0x3B81, 0x3780, 0x3781, 0x4000,
+                 0x40FF, 0x437F, 0x7F7F, 0xFF7F, 0x7F00, 0x7F80, 0xFF80, 0x7FC0, 0x0100, 0x8100, 0x3F00, 0x3EFF, 0x4B80, 0xCB80,
+                 0x5F80, 0x1F80, 0x2F81, 0x6F7F],
+    "float16": [0x0000, 0x8000, 0x0001, 0x8001, 0x03FF, 0x0400, 0x3C00, 0xBC00, 0x3C01, 0x1400, 0x1401, 0x1000, 0x1001, 0x4000,
+                0x47FF, 0x5BFF, 0x7BFF, 0xFBFF, 0x7800, 0x7C00, 0xFC00, 0x7E00, 0x0800, 0x8800, 0x3800, 0x37FF, 0x6400, 0xE400,
+                0x6C00, 0x0C00, 0x2C01, 0x73FF],
+}
+
+
 @pytest.mark.parametrize("redop", ["sum", "prod"])
-def test_every_bf16_value_against_chosen_partners(redop):
-    """Rounding of bf16 results (the device uses the conversion instruction, the oracle the integer formula): every one
-    of the 65536 bf16 bit patterns -- zeros, denormals, infinities, NaNs -- combined with 32 partners that lead to exact
-    results, ties, carries into the exponent, overflow and underflow.  Bits equal wherever the oracle has a number, NaN
-    exactly where it has a NaN."""
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_every_16_bit_float_against_chosen_partners(dtype, redop):
+    """Rounding of 16-bit results (the device uses the conversion instructions, the oracle the integer formula for bf16
+    and NumPy's cast for fp16): every one of the 65536 bit patterns -- zeros, denormals, infinities, NaNs -- combined
+    with 32 partners that lead to exact results, ties, carries into the exponent, overflow and underflow.  Bits equal
+    wherever the oracle has a number, NaN exactly where it has a NaN."""
     from msccl.executor import Executor, collective_buffers
-    partners = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x3F80, 0xBF80, 0x3F81, 0x3B80, 0x3B81, 0x3780, 0x3781, 0x4000,
-                         0x40FF, 0x437F, 0x7F7F, 0xFF7F, 0x7F00, 0x7F80, 0xFF80, 0x7FC0, 0x0100, 0x8100, 0x3F00, 0x3EFF, 0x4B80, 0xCB80,
-                         0x5F80, 0x1F80, 0x2F81, 0x6F7F], np.uint16)
+    partners = np.array(SIXTEEN_BIT_PARTNERS[dtype], np.uint16)
     every = np.arange(65536, dtype=np.uint32).astype(np.uint16)
-    x = [np.tile(every, partners.size), np.repeat(partners, 65536)]
+    bits = [np.tile(every, partners.size), np.repeat(partners, 65536)]
+    x = bits if dtype == "bfloat16" else [v.view(np.float16) for v in bits]
+    as_float = oi.bf16_bits_to_f32 if dtype == "bfloat16" else (lambda v: v.astype(np.float32))
     xml = ir_samples.ring_allreduce_xml(2)
     algo = oi.parse_xml(xml)
     E = x[0].size // 2
-    want = oc.place_inputs(algo, x, E, "bfloat16")
-    oi.Interpreter(algo).run(want, E, "bfloat16", redop)
+    want = oc.place_inputs(algo, x, E, dtype)
+    oi.Interpreter(algo).run(want, E, dtype, redop)
     ex = Executor(xml)
-    print(f"case: every bf16 value, redop={redop}", flush=True)
-    ex.setup(E * 2, "bfloat16", redop)
-    ins, outs, _ = collective_buffers(ex.tables, E * 2, "bfloat16", inputs=[to_torch(v, "bfloat16") for v in x])
+    print(f"case: every {dtype} value, redop={redop}", flush=True)
+    ex.setup(E * 2, dtype, redop)
+    ins, outs, _ = collective_buffers(ex.tables, E * 2, dtype, inputs=[to_torch(v, dtype) for v in x])
     ex.run(ins, outs)
     torch.cuda.synchronize()
     for r in range(2):
-        got, ref = to_numpy(ins[r], "bfloat16"), want[r]["i"]
-        gn, rn = np.isnan(oi.bf16_bits_to_f32(got)), np.isnan(oi.bf16_bits_to_f32(ref))
+        got, ref = to_numpy(ins[r], dtype), want[r]["i"]
+        gn, rn = np.isnan(as_float(got)), np.isnan(as_float(ref))
         assert np.array_equal(gn, rn), (r, int(gn.sum()), int(rn.sum()))
-        assert np.array_equal(got[~rn], ref[~rn]), (r, np.flatnonzero((got != ref) & ~rn)[:8])
+        gb, rb = got.view(np.uint16), ref.view(np.uint16)
+        assert np.array_equal(gb[~rn], rb[~rn]), (r, np.flatnonzero((gb != rb) & ~rn)[:8])
 
 
 @pytest.mark.parametrize("protocol", PROTOCOLS)
