@@ -126,6 +126,19 @@ def register_mi355x_plans():
     def mi355x_allpairs_allreduce_2x8(prog, nodes):
         allreduce_allpairs(16)
 
+    # Eight groups (64 ranks), fp32, microseconds, two-level / one ring over all ranks (the ring is 126 hand-offs deep, the
+    # two-level program 28): 16 KiB per rank 66 / 170, 256 KiB 73 / 171, 1 MiB 104 / 257, 4 MiB 262 / 358, 8 MiB 419 / 486,
+    # 16 MiB 796 / 768, 24 MiB 1162 / 1132, 64 MiB 3086 / 3008.
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=2,
+                            sizes=(0, '12MiB'), interleaved_replication=False, machines=lambda x: x == 8)
+    def mi355x_two_level_allreduce_8x8(prog, nodes):
+        hierarchical_allreduce(8, 8, "auto")
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=1,
+                            sizes=('12MiB', None), threadblock_policy=manual, machines=lambda x: x == 8)
+    def mi355x_ring_allreduce_8x8(prog, nodes):
+        allreduce_ring(size=64, channels=1)
+
     # 16 ranks, large messages: one ring over all ranks (4 instances) against the two-level program, 16 MiB per rank 194 / 212,
     # 32 MiB 377 / 412, 128 MiB 1403 / 1498 (all-pairs: 202, 427).  On 32 ranks the two are level (128 MiB 2890 / 2917, 8 MiB 235 / 219).
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=16, inplace=True, instances=4,

@@ -180,6 +180,16 @@ def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
         assert select(algos, "allreduce", 64 << 20).tables.name == f'mi355x_{windows[-1][2]}_allreduce_{groups}x8'
 
 
+def test_mi355x_allreduce_windows_of_eight_groups(capsys):
+    """64 virtual ranks: the two-level program (28 hand-offs deep) below 12 MiB per rank, one ring over all ranks (126) above."""
+    msccl.init('mi355x', 8, ('allreduce', (0, None)))
+    capsys.readouterr()
+    small, large = load_config()
+    assert (small.min_bytes, small.max_bytes, small.tables.name, small.tables.ngpus) == (0, 12 << 20, 'mi355x_two_level_allreduce_8x8', 64)
+    assert (large.min_bytes, large.tables.name, large.tables.ngpus, large.tables.nchunksperloop) == (12 << 20, 'mi355x_ring_allreduce_8x8', 64, 64)
+    assert select([small, large], "allreduce", 256 << 10) is small
+
+
 def test_ef_file_plan(tmp_path, capsys):
     import ir_samples
     f = tmp_path / "ring.xml"

@@ -331,6 +331,29 @@ def test_init_to_run_allpairs_over_groups(groups, elems, capsys):
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
 
 
+def test_init_to_run_allreduce_over_eight_groups(capsys):
+    """64 virtual ranks at 256 KiB per rank: msccl.init picks the two-level all-reduce (int32 sums, exact in any order)."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    n, nbytes = 64, 256 << 10
+    msccl.init('mi355x', 8, ('allreduce', nbytes))
+    capsys.readouterr()
+    ar = select(load_config(), "allreduce", nbytes)
+    assert ar.tables.name == "mi355x_two_level_allreduce_8x8" and ar.tables.ngpus == n
+    rng = np.random.default_rng(64)
+    x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64) for _ in range(n)]
+    cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
+    ex = Executor(ar.tables)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v.astype(np.int32)) for v in x])
+    ex.run(ins, outs)
+    want = sum(x).astype(np.int32)
+    assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
+
+
 def test_init_to_run_allgather_over_two_groups(capsys):
     """16 virtual ranks: the all-pairs all-gather below 12 MB per rank -- every output is the concatenation of the inputs."""
     import os
