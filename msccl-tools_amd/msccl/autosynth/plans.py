@@ -95,6 +95,18 @@ def register_mi355x_plans():
     def mi355x_ring_allgather(prog, nodes):
         allgather_ring(size=8 * nodes, channels=1)
 
+    # Eight groups (64 ranks, 63 messages into every rank): all-pairs / ring, 16 KiB per rank 20 / 114, 64 KiB 95 / 175,
+    # 128 KiB 174 / 192, 192 KiB 256 / 244, 1 MiB 1251 / 1207, 4 MiB 5348 / 4769.
+    @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=1,
+                            sizes=(0, '160KiB'), threadblock_policy=manual, machines=lambda x: x == 8)
+    def mi355x_allpairs_allgather_8x8(prog, nodes):
+        allgather_allpairs(64)
+
+    @register_msccl_program(fully_connected(8), 'allgather', 'mi355x', chunk_factor=1, inplace=True, instances=1,
+                            sizes=('160KiB', None), threadblock_policy=manual, machines=lambda x: x == 8)
+    def mi355x_ring_allgather_8x8(prog, nodes):
+        allgather_ring(size=64, channels=1)
+
     # The one-step all-to-all, every message read where its sender keeps it, for any number of groups: 8 ranks 8-10 us from
     # 8 KiB to 1 MiB per rank, 16 MiB 52 us, 64 MiB 204 us = 66 % of the HBM peak, 256 MiB 715 us = 75 % (instances make no
     # difference).  The hierarchical program gathers per destination group first, which pays on links between machines; between

@@ -148,6 +148,12 @@ def test_mi355x_allgather_windows(capsys):
     small, large = load_config()
     assert (small.tables.name, small.tables.ngpus, small.tables.ntbs) == ('mi355x_allpairs_allgather', 16, 16 * 15)
     assert (large.tables.name, large.tables.ngpus, large.tables.nchunksperloop) == ('mi355x_ring_allgather', 16, 64)
+    # eight groups: 63 messages into every rank -- the ring from 160 KiB per rank on
+    msccl.init('mi355x', 8, ('allgather', (0, None)))
+    capsys.readouterr()
+    small, large = load_config()
+    assert (small.max_bytes, small.tables.name, small.tables.ngpus) == (160 << 10, 'mi355x_allpairs_allgather_8x8', 64)
+    assert (large.min_bytes, large.tables.name, large.tables.ngpus) == (160 << 10, 'mi355x_ring_allgather_8x8', 64)
 
 
 def test_mi355x_alltoall_plans(capsys):
