@@ -139,10 +139,17 @@ def register_mi355x_plans():
         allreduce_allpairs(16)
 
     # Eight groups (64 ranks), fp32, microseconds, two-level / one ring over all ranks (the ring is 126 hand-offs deep, the
-    # two-level program 28): 16 KiB per rank 66 / 170, 256 KiB 73 / 171, 1 MiB 104 / 257, 4 MiB 262 / 358, 8 MiB 419 / 486,
+    # two-level program 28): 16 KiB per rank 47 / 170, 256 KiB 73 / 171, 1 MiB 104 / 257, 4 MiB 262 / 358, 8 MiB 419 / 486,
     # 16 MiB 796 / 768, 24 MiB 1162 / 1132, 64 MiB 3086 / 3008.
+    # One instance of the two-level program has half the threadblocks, each with a workgroup of its own, and runs on flag-in-data
+    # lines up to 64 KiB per rank: 47-49 us against 68-69 with two instances; 256 KiB to 4 MiB the same; 8 MiB 450 against 413.
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=1,
+                            sizes=(0, '4MiB'), interleaved_replication=False, machines=lambda x: x == 8)
+    def mi355x_two_level_allreduce_8x8_small(prog, nodes):
+        hierarchical_allreduce(8, 8, "auto")
+
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=2,
-                            sizes=(0, '12MiB'), interleaved_replication=False, machines=lambda x: x == 8)
+                            sizes=('4MiB', '12MiB'), interleaved_replication=False, machines=lambda x: x == 8)
     def mi355x_two_level_allreduce_8x8(prog, nodes):
         hierarchical_allreduce(8, 8, "auto")
 

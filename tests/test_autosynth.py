@@ -187,13 +187,16 @@ def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
 
 
 def test_mi355x_allreduce_windows_of_eight_groups(capsys):
-    """64 virtual ranks: the two-level program (28 hand-offs deep) below 12 MiB per rank, one ring over all ranks (126) above."""
+    """64 virtual ranks: the two-level program (28 hand-offs deep; one instance below 4 MiB per rank, two above) below
+    12 MiB, one ring over all ranks (126 deep) from there on."""
     msccl.init('mi355x', 8, ('allreduce', (0, None)))
     capsys.readouterr()
-    small, large = load_config()
-    assert (small.min_bytes, small.max_bytes, small.tables.name, small.tables.ngpus) == (0, 12 << 20, 'mi355x_two_level_allreduce_8x8', 64)
-    assert (large.min_bytes, large.tables.name, large.tables.ngpus, large.tables.nchunksperloop) == (12 << 20, 'mi355x_ring_allreduce_8x8', 64, 64)
-    assert select([small, large], "allreduce", 256 << 10) is small
+    algos = load_config()
+    assert [(a.min_bytes, a.max_bytes, a.tables.name, a.tables.nchunksperloop) for a in algos] == [
+        (0, 4 << 20, 'mi355x_two_level_allreduce_8x8_small', 64), (4 << 20, 12 << 20, 'mi355x_two_level_allreduce_8x8', 128),
+        (12 << 20, float("inf"), 'mi355x_ring_allreduce_8x8', 64)]
+    assert all(a.tables.ngpus == 64 for a in algos)
+    assert select(algos, "allreduce", 256 << 10) is algos[0]
 
 
 def test_ef_file_plan(tmp_path, capsys):

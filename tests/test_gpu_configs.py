@@ -342,7 +342,7 @@ def test_init_to_run_allreduce_over_eight_groups(capsys):
     msccl.init('mi355x', 8, ('allreduce', nbytes))
     capsys.readouterr()
     ar = select(load_config(), "allreduce", nbytes)
-    assert ar.tables.name == "mi355x_two_level_allreduce_8x8" and ar.tables.ngpus == n
+    assert ar.tables.name == "mi355x_two_level_allreduce_8x8_small" and ar.tables.ngpus == n
     rng = np.random.default_rng(64)
     x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64) for _ in range(n)]
     cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
