@@ -10,7 +10,11 @@
  * buffer a plain device pointer; no C++ or torch types cross this boundary.
  *
  * Ownership: the caller owns the rank buffers and the workspace; the library owns the plan (host
- * tables and their device copies) and never frees caller memory.
+ * tables and their device copies) and never frees caller memory.  Between a bind and the last wait
+ * on that binding the workspace's contents belong to the plan: nobody else may write there.  A
+ * workspace may be handed from plan to plan (every bind stamps it, and a plan that finds another
+ * plan's stamp clears it again), but whoever writes into it by other means must clear its first
+ * 64 bytes too, or the next bind of the plan that armed it will trust what it holds.
  * Errors: 0 on success, a negative mscclx_error otherwise; mscclx_last_error() returns the text of
  * the calling thread's last failure.  No exception crosses the ABI.
  * Threading: a plan is not thread-safe; launches are stream-ordered; launches of one plan must all
@@ -173,9 +177,11 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
  * in-place NCCL call; buffers that overlap in memory need a plan configured with staging=1, else
  * MSCCLX_ERR_ALIASED).  A buffer must start on a boundary of its element type; a view into a
  * larger tensor is fine.
- * Uploads the plan tables to the current device and clears the workspace.
- * Binding again after a launch has been waited for (new buffers, same geometry) re-uses the
- * device-side allocations: one upload of the tables, no allocation. */
+ * Uploads the plan tables to the current device and arms the workspace (counters zero, the plan's
+ * stamp in control word 2).  Binding again after a launch has been waited for (new buffers, same
+ * geometry) re-uses the device-side allocations -- one upload of the tables, no allocation -- and
+ * clears the workspace again only if it must: another address, a lost launch before, or a stamp
+ * that is no longer this plan's because another plan was bound to the same memory in between. */
 int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void* const* scratch,
                      void* workspace, size_t workspace_bytes);
 
@@ -189,7 +195,10 @@ int mscclx_plan_poll(mscclx_plan* plan, void* stream, mscclx_status* status);
 /* Asks the running launch (and any launch of this plan queued behind it) to give up: every
  * workgroup sees the request while it polls and leaves, every wave exits normally.  Returns once
  * the request is on the device; mscclx_plan_wait then returns MSCCLX_ERR_ABORTED, the rank buffers
- * hold partial results, and the next launch re-arms the counters. */
+ * hold partial results, and the next mscclx_plan_launch re-arms the counters.  A launch replayed from
+ * a HIP graph passes by that re-arming: the first replay after an abort may still find the request,
+ * ends at once and is reported as MSCCLX_ERR_ABORTED by the wait that follows it; the replay after
+ * that runs normally (every launch clears the counters the next one uses). */
 int mscclx_plan_abort(mscclx_plan* plan);
 /* Bytes of the device array behind mscclx_plan_run_static (one copy per GPU, held until the process ends). */
 #define MSCCLX_STATIC_SCRATCH_BYTES (32u << 20)

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -63,6 +64,7 @@ struct DeviceState {
   DeviceImage image;                     // (bytes are dropped after the upload)
   mscclx_status* host_status = nullptr;  // pinned, device-visible
   unsigned char* workspace = nullptr;
+  unsigned long long stamp = 0;          // what this binding wrote into the workspace's stamp word when it armed it
   bool dirty = false;  // counters must be cleared before the next launch (after a failed or aborted launch)
   bool abort_requested = false;
   hipStream_t side = nullptr;            // for the host's abort request while the launch stream is busy
@@ -557,7 +559,7 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
     d->tables_capacity = img.bytes.size();
     HIP_TRY(hipHostMalloc((void**)&d->host_status, sizeof(mscclx_status), hipHostMallocDefault));
     HIP_TRY(hipHostMalloc((void**)&d->abort_word_host, sizeof(unsigned long long), hipHostMallocDefault));
-    *d->abort_word_host = 1ull;
+    *d->abort_word_host = kAbortByHost;
     HIP_TRY(hipStreamCreateWithFlags(&d->side, hipStreamNonBlocking));
     HIP_TRY(hipEventCreate(&d->ev0));
     HIP_TRY(hipEventCreate(&d->ev1));
@@ -569,8 +571,20 @@ int mscclx_plan_bind(mscclx_plan* plan, void* const* in, void* const* out, void*
   d->ready = false;
   HIP_TRY(hipMemcpy(d->tables, img.bytes.data(), img.bytes.size(), hipMemcpyHostToDevice));
   std::memset(d->host_status, 0, sizeof(mscclx_status));
-  if (fresh || d->dirty || d->workspace != (unsigned char*)workspace) {
+  // The workspace is armed (counters zero; LL: slots too) when this plan first sees it, after a lost launch, and when
+  // the stamp this plan left in it is gone: another plan's bind has cleared and stamped it in between, and its
+  // counters and slots, laid out for that plan, mean nothing here.
+  bool arm = fresh || d->dirty || d->workspace != (unsigned char*)workspace;
+  if (!arm) {
+    unsigned long long seen = 0;
+    HIP_TRY(hipMemcpy(&seen, (unsigned long long*)workspace + kStampWord, sizeof seen, hipMemcpyDeviceToHost));
+    arm = seen != d->stamp;
+  }
+  if (arm) {
+    static std::atomic<unsigned long long> next_stamp{1};
+    d->stamp = (next_stamp.fetch_add(1) << 20) | ((unsigned long long)(uintptr_t)d >> 4 & 0xfffffull) | 1ull;  // (never 0)
     HIP_TRY(hipMemset(workspace, 0, armed_bytes(g)));
+    HIP_TRY(hipMemcpy((unsigned long long*)workspace + kStampWord, &d->stamp, sizeof d->stamp, hipMemcpyHostToDevice));
     HIP_TRY(hipDeviceSynchronize());
     d->dirty = false;
   }
@@ -594,6 +608,7 @@ int mscclx_plan_launch(mscclx_plan* plan, void* stream) {
     HIP_TRY(hipStreamSynchronize(s));
     HIP_TRY(hipStreamSynchronize(d->side));
     HIP_TRY(hipMemset(d->workspace, 0, armed_bytes(g)));  // LL: launches count from 0 again, old lines must go
+    HIP_TRY(hipMemcpy((unsigned long long*)d->workspace + kStampWord, &d->stamp, sizeof d->stamp, hipMemcpyHostToDevice));
     HIP_TRY(hipDeviceSynchronize());
     std::memset(d->host_status, 0, sizeof(mscclx_status));
     d->dirty = false;
@@ -662,8 +677,12 @@ static int finish_wait(mscclx_plan* plan, mscclx_status* status) {
     }
   }
 #endif
-  if (d->abort_requested) {
+  // (st.code is ABORTED when a launch found the request on the device by itself: one replayed from a HIP graph
+  // after an abort, which passes by the re-arming in mscclx_plan_launch -- the replay after it runs normally,
+  // because every launch, aborted or not, clears the counters of the area the next one uses)
+  if (d->abort_requested || st.code == MSCCLX_ERR_ABORTED) {
     d->dirty = true;
+    d->abort_requested = false;
     if (status) { *status = st; status->code = MSCCLX_ERR_ABORTED; }
     std::memset(d->host_status, 0, sizeof(mscclx_status));
     return fail(MSCCLX_ERR_ABORTED, "the launch was aborted by mscclx_plan_abort; the rank buffers hold partial results");

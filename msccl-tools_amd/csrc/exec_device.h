@@ -505,7 +505,7 @@ struct LLWatch {
 
 // (arguments by value: a struct handed to a function that is not inlined would have to live in memory)
 __device__ __noinline__ void ll_give_up(u64* abort_word, mscclx_status* hs, int tb, int step, int slice, u64 pass, int waiting_on = 1) {
-  if (atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
+  if (atomicCAS(abort_word, 0ull, kAbortByWatchdog) == 0ull) {
     hs->tb = tb; hs->step = step; hs->slice = slice; hs->pass = (int64_t)pass; hs->waiting_on = waiting_on;
     __threadfence_system();
     __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_TIMEOUT, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1459,7 +1459,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
               // report the first context that is still waiting
               const u64 stuck = __ballot(c.active);
               const int who = __ffsll((long long)stuck) - 1;
-              if (lane == who && atomicCAS(abort_word, 0ull, 1ull) == 0ull) {
+              if (lane == who && atomicCAS(abort_word, 0ull, kAbortByWatchdog) == 0ull) {
                 int what = 3;
                 if (c.w0 && load_counter(c.w0) < c.t0) what = 0;
                 else if (c.w1 && (LL ? (uint32_t)(load_counter(c.w1) >> 32) != (uint32_t)c.t1 : load_counter(c.w1) < c.t1)) what = 1;
@@ -1539,7 +1539,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
       prof_ack += prof_t3 - prof_t2;
       prof_fin += prof_t4 - prof_t3;
       // the first kProfTrace moves of the workgroup: start (10 ns ticks since the workgroup began), duration up to the barrier, lane
-      if (prof_moves < kProfTrace)
+      if (p.prof && prof_moves < kProfTrace)
         p.prof[(size_t)blockIdx.x * kProfWords + 8 + prof_moves] = ((prof_t1 - prof_start) << 32) | (((prof_t3 - prof_t1) & 0xffffffull) << 8) | (u64)(choice & 0xff);
       ++prof_moves;
     }
@@ -1555,10 +1555,17 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
     if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
       publish(group_count, 0);
-      if (groups == 1) {  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
-        publish(p.sync_base, launch_no + 1);
-      } else if (__hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
+      bool last = groups == 1;  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
+      if (!last && __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
         publish(p.sync_base + 1, 0);
+        last = true;
+      }
+      if (last) {
+        // A launch that ran under a host's abort request says so itself: whoever replays it from a HIP graph passes
+        // by the host code that would have re-armed the counters, and must still learn that it did not run.
+        if (load_counter(abort_word) == kAbortByHost &&
+            __hip_atomic_load(&p.host_status->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
+          __hip_atomic_store(&p.host_status->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
         publish(p.sync_base, launch_no + 1);
       }
     }

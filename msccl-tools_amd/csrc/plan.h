@@ -198,6 +198,11 @@ constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
 // Workgroups report the end of a launch group by group: one counter for all of them would put one
 // returning atomic per workgroup on a single address at the end of every launch (measured 10 ns
 // each: 5 us of a 512-workgroup launch).
+constexpr int kStampWord = 2;  // control word 2: which plan's binding armed this workspace (see mscclx_plan_bind)
+// Values of an area's abort word: raised by a workgroup whose watchdog expired (which then reports the step it
+// waited for), or by mscclx_plan_abort from the host (reported by the launch's last workgroup, so that a launch
+// replayed from a HIP graph onto a raised word still tells the host that it did not run).
+constexpr unsigned long long kAbortByWatchdog = 1, kAbortByHost = 2;
 constexpr int kFinishGroups = 64;
 constexpr int kFinishStrideWords = 16;
 constexpr int kControlWords = 8 + kFinishGroups * kFinishStrideWords;

@@ -68,18 +68,29 @@ _LOCAL_SRC = {OP_CODES[k] for k in ("s", "cpy", "re")}
 _LOCAL_DST = {OP_CODES[k] for k in ("r", "rcs", "rrs", "rrc", "rrcs", "cpy", "re")}
 
 
-def _scratch_behind_output(row, o_chunks):
+def _scratch_behind_output(rows, o_chunks, where):
     """ncclize(use_scratch=False) writes a rank's scratch references as output offsets past the
     output's own chunks ("scratch at the end of output", msccl/ncclize.py:690-697) while still
-    declaring o_chunks and s_chunks separately.  Such a local reference is taken back to the
-    scratch buffer, so the caller's output buffer keeps the size the collective gives it.  (On 's'
-    and receive steps the other side's location is informational and is left alone.)"""
-    ty, sb, so, db, do, cnt, depid, deps, hasdep = row
-    if ty in _LOCAL_SRC and sb == BUF_CODES["o"] and so >= o_chunks:
-        sb, so = BUF_CODES["s"], so - o_chunks
-    if ty in _LOCAL_DST and db == BUF_CODES["o"] and do >= o_chunks:
-        db, do = BUF_CODES["s"], do - o_chunks
-    return (ty, sb, so, db, do, cnt, depid, deps, hasdep)
+    declaring o_chunks and s_chunks separately, and never names buffer 's'.  In such a rank -- one
+    that declares scratch and none of whose steps names 's' -- a local reference past the output's
+    end is taken back to the scratch buffer, so the caller's output buffer keeps the size the
+    collective gives it.  (On 's' and receive steps the other side's location is informational and
+    is left alone.)  Everywhere else an output offset out of range stays what it is: malformed,
+    refused when the plan is made.  A step that straddles the output's end is refused here."""
+    s_code, o_code = BUF_CODES["s"], BUF_CODES["o"]
+    if any((row[0] in _LOCAL_SRC and row[1] == s_code) or (row[0] in _LOCAL_DST and row[3] == s_code) for row in rows):
+        return rows
+    out = []
+    for k, (ty, sb, so, db, do, cnt, depid, deps, hasdep) in enumerate(rows):
+        for is_local, buf, off in ((ty in _LOCAL_SRC, sb, so), (ty in _LOCAL_DST, db, do)):
+            if is_local and buf == o_code and off < o_chunks < off + cnt:
+                raise IRError(f"{where} step {k}: chunks [{off}, {off + cnt}) straddle the end of the output buffer ({o_chunks} chunks)")
+        if ty in _LOCAL_SRC and sb == o_code and so >= o_chunks:
+            sb, so = s_code, so - o_chunks
+        if ty in _LOCAL_DST and db == o_code and do >= o_chunks:
+            db, do = s_code, do - o_chunks
+        out.append((ty, sb, so, db, do, cnt, depid, deps, hasdep))
+    return out
 
 
 def parse_algo_xml(text):
@@ -129,10 +140,10 @@ def parse_algo_xml(text):
                 op_rows.append((OP_CODES[ty], BUF_CODES[sb], _int(st, "srcoff", -1), BUF_CODES[db], _int(st, "dstoff", -1),
                                 _int(st, "cnt", 1 if ty != "nop" else 0), _int(st, "depid", -1), _int(st, "deps", -1),
                                 _int(st, "hasdep", 0)))
-            if rank_chunks[r, 2] > 0:
-                for k in range(begin, len(op_rows)):
-                    op_rows[k] = _scratch_behind_output(op_rows[k], int(rank_chunks[r, 1]))
             tb_rows.append((r, _int(t, "send"), _int(t, "recv"), _int(t, "chan"), begin, len(op_rows)))
+        if rank_chunks[r, 2] > 0 and tb_rows and len(tbs):
+            first = tb_rows[len(tb_rows) - len(tbs)][4]
+            op_rows[first:] = _scratch_behind_output(op_rows[first:], int(rank_chunks[r, 1]), f"gpu {r}:")
     return AlgoTables(
         name=root.get("name", ""), proto=root.get("proto", "Simple"), coll=root.get("coll", "custom"),
         inplace=bool(_int(root, "inplace", 0)), nchannels=_int(root, "nchannels", 0),

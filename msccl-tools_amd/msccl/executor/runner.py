@@ -45,6 +45,7 @@ class Executor:
         self._scratch = None
         self._workspace = None
         self._bound = None
+        self._staged_for_aliasing = False
         self.host_seconds = {}   # host time of the last configure / bind call into the library
 
     # -- geometry ---------------------------------------------------------------------------------
@@ -61,6 +62,7 @@ class Executor:
         self.dtype = dtype_name(dtype)
         self.chunk_bytes = int(chunk_bytes)
         self._setup_args = (chunk_bytes, dtype, redop, dict(knobs))
+        self._staged_for_aliasing = False
         with torch.cuda.device(self.device):
             t0 = time.perf_counter()
             self.info = self.plan.configure(self.chunk_bytes, self.dtype, redop, **knobs)
@@ -92,15 +94,40 @@ class Executor:
             ptrs.append(b.data_ptr())
         return ptrs
 
-    def bind(self, inputs, outputs):
+    def _spans_overlap(self, ins, outs):
+        """Do any two rank buffers the algorithm addresses share memory?  (What mscclx_plan_bind refuses
+        with ALIASED unless every message is staged.)"""
+        t = self.tables
+        spans = []
+        for col, ptrs in ((0, ins), (1, outs), (2, [0 if s is None else s.data_ptr() for s in self._scratch])):
+            for r, ptr in enumerate(ptrs):
+                need = int(t.rank_chunks[r, col]) * self.chunk_bytes
+                if need:
+                    spans.append((ptr, ptr + need))
+        spans.sort()
+        return any(b[0] < a[1] for a, b in zip(spans, spans[1:]))
+
+    def bind(self, inputs, outputs, allow_aliased=False):
+        """Attach rank buffers.  Buffers that the IR names separately but that share memory (an in-place
+        call on an out-of-place algorithm) are refused with MscclxError(ALIASED) unless
+        allow_aliased=True: the plan is then configured again with every message copied through a FIFO
+        slot.  That only takes away the executor's own reads of payloads where the sender keeps them; whether
+        the *program* still computes the collective when two of its buffers are one is the caller's
+        to know (it does for NCCL's in-place all-gather convention on an all-gather whose every write
+        of a chunk writes that chunk's final value; it does not where a receive overwrites what a
+        later step of the same rank still reads).  A later bind of buffers that do not overlap goes back
+        to the knobs setup() was called with."""
         if self.info is None:
             raise RuntimeError("call setup() first")
         key = (tuple(0 if b is None else b.data_ptr() for b in (inputs or [])),
-               tuple(0 if b is None else b.data_ptr() for b in (outputs or [])))
+               tuple(0 if b is None else b.data_ptr() for b in (outputs or [])), bool(allow_aliased))
         if key == self._bound:
             return
         ins = self._check_buffers(inputs, 0, "input")
         outs = self._check_buffers(outputs, 1, "output")
+        chunk_bytes, dtype, redop, knobs = self._setup_args
+        if self._staged_for_aliasing and not self._spans_overlap(ins, outs):
+            self.setup(chunk_bytes, dtype, redop, **knobs)
         scr = [0 if s is None else s.data_ptr() for s in self._scratch]
         try:
             with torch.cuda.device(self.device):
@@ -108,13 +135,11 @@ class Executor:
                 self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
                 self.host_seconds["bind"] = time.perf_counter() - t0
         except MscclxError as e:
-            if e.code != ERR_ALIASED:
+            if e.code != ERR_ALIASED or not allow_aliased:
                 raise
-            # the caller aliases buffers the IR names separately (an in-place call): payloads can no
-            # longer be read in place, so every message goes through a FIFO slot
-            chunk_bytes, dtype, redop, knobs = self._setup_args
-            knobs["staging"] = 1
-            self.setup(chunk_bytes, dtype, redop, **knobs)
+            self.setup(chunk_bytes, dtype, redop, **dict(knobs, staging=1))
+            self._setup_args = (chunk_bytes, dtype, redop, knobs)   # what the caller asked for, to go back to
+            self._staged_for_aliasing = True
             scr = [0 if t is None else t.data_ptr() for t in self._scratch]
             with torch.cuda.device(self.device):
                 self.plan.bind(ins, outs, scr, self._workspace.data_ptr(), self._workspace.numel())
@@ -143,8 +168,8 @@ class Executor:
         with torch.cuda.device(self.device):
             self.plan.abort()
 
-    def run(self, inputs, outputs):
-        self.bind(inputs, outputs)
+    def run(self, inputs, outputs, allow_aliased=False):
+        self.bind(inputs, outputs, allow_aliased=allow_aliased)
         self.launch()
         self.wait()
         return outputs

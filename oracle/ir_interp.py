@@ -135,6 +135,28 @@ class Algo:
     __slots__ = ("name", "proto", "nchannels", "nchunksperloop", "ngpus", "coll", "inplace", "gpus")
 
 
+def _scratch_behind_output(gpu):
+    """ncclize(use_scratch=False) addresses a rank's scratch as output chunks past o_chunks
+    (msccl/ncclize.py:690-697, "scratch at the end of output") and then never names buffer 's':
+    in a rank that declares scratch and names 's' nowhere, local references past the output's end
+    mean scratch.  Any other out-of-range offset is left as written (and fails when executed)."""
+    local_src, local_dst = ("s", "cpy", "re"), RECV_TYPES + ("cpy", "re")
+    steps = [st for tb in gpu.tbs for st in tb.steps]
+    if not gpu.s_chunks or any((st.type in local_src and st.srcbuf == "s") or (st.type in local_dst and st.dstbuf == "s") for st in steps):
+        return
+    for tb in gpu.tbs:
+        for k, st in enumerate(tb.steps):
+            for local, buf, off in ((st.type in local_src, "srcbuf", "srcoff"), (st.type in local_dst, "dstbuf", "dstoff")):
+                at = getattr(st, off)
+                if not (local and getattr(st, buf) == "o"):
+                    continue
+                if at < gpu.o_chunks < at + st.cnt:
+                    raise ValueError(f"gpu {gpu.id}: a step's chunks [{at}, {at + st.cnt}) straddle the end of the output buffer")
+                if at >= gpu.o_chunks:
+                    st = st._replace(**{buf: "s", off: at - gpu.o_chunks})
+            tb.steps[k] = st
+
+
 def parse_xml(text):
     """Parse <algo> XML (ir.py:320-391 / ncclize.py:658-718) into Algo/Gpu/Tb/Step."""
     root = ET.fromstring(text)
@@ -156,15 +178,10 @@ def parse_xml(text):
             for st in t.findall("step"):
                 ty = st.get("type")
                 sb, so, db, do = st.get("srcbuf"), int(st.get("srcoff")), st.get("dstbuf"), int(st.get("dstoff"))
-                # ncclize(use_scratch=False) addresses a rank's scratch as output chunks past o_chunks
-                # (msccl/ncclize.py:690-697, "scratch at the end of output"): local references only
-                if gpu.s_chunks and ty in ("s", "cpy", "re") and sb == "o" and so >= gpu.o_chunks:
-                    sb, so = "s", so - gpu.o_chunks
-                if gpu.s_chunks and ty in RECV_TYPES + ("cpy", "re") and db == "o" and do >= gpu.o_chunks:
-                    db, do = "s", do - gpu.o_chunks
                 tb.steps.append(Step(int(st.get("s")), ty, sb, so, db, do, int(st.get("cnt")),
                                      int(st.get("depid")), int(st.get("deps")), int(st.get("hasdep"))))
             gpu.tbs.append(tb)
+        _scratch_behind_output(gpu)
         a.gpus.append(gpu)
     a.gpus.sort(key=lambda g: g.id)
     if [g.id for g in a.gpus] != list(range(a.ngpus)):

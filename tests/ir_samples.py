@@ -206,3 +206,15 @@ def ncclize_style_allreduce_xml():
             _tb(2, -1, -1, 0, [_step(0, "cpy", "i", 0, "o", 0, 1, hasdep=1)]),
         ])
     return _algo("ncclize_allreduce", "allreduce", 0, 3, 1, 1, [g0, leaf(1), leaf(2)])
+
+
+def relay_through_scratch_xml(out_off=0, out_cnt=1, name_scratch=True):
+    """2 ranks, out of place: rank 0 sends i[0..1] to rank 1, which receives them into scratch
+    (name_scratch: as s[0..1], the way the MSCCLang emitter writes scratch; else as o[1..2], "scratch at
+    the end of output", the way ncclize(use_scratch=False) does) and copies `out_cnt` of them to
+    o[out_off..].  Rank 1 declares one output chunk and two scratch chunks."""
+    sbuf, soff = ("s", 0) if name_scratch else ("o", 1)
+    g0 = _gpu(0, 2, 0, 0, [_tb(0, 1, -1, 0, [_step(0, "s", "i", 0, sbuf, soff, 2)])])
+    g1 = _gpu(1, 0, 1, 2, [_tb(0, -1, 0, 0, [_step(0, "r", "i", 0, sbuf, soff, 2, hasdep=1)]),
+                           _tb(1, -1, -1, 0, [_step(0, "cpy", sbuf, soff, "o", out_off, out_cnt, depid=0, deps=0)])])
+    return _algo("relay_through_scratch", "custom", 0, 2, 1, 2, [g0, g1])

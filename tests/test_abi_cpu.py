@@ -79,6 +79,32 @@ def test_plan_create_rejects_bad_ir(mscclx_lib, old, new, needle):
     assert needle in e.value.message
 
 
+def test_output_offsets_out_of_range_are_not_taken_for_scratch(mscclx_lib):
+    """Only a rank that declares scratch and never names buffer 's' -- what ncclize(use_scratch=False)
+    writes -- has its output offsets past o_chunks read as scratch.  A document that names 's' keeps
+    its out-of-range output offset and is refused; a step that straddles the output's end is refused
+    in either style."""
+    ok = parse_algo_xml(ir_samples.relay_through_scratch_xml(name_scratch=False))
+    assert ok.ops[1:, [1, 2, 3, 4]].tolist() == [[0, 0, 2, 0], [2, 0, 1, 0]]   # r -> s[0..1]; cpy s[0] -> o[0]
+    Plan(ok)
+    Plan(parse_algo_xml(ir_samples.relay_through_scratch_xml()))
+    t = parse_algo_xml(ir_samples.relay_through_scratch_xml(out_off=1))      # names 's': o[1] stays o[1], past the output's one chunk
+    assert t.ops[2, [3, 4]].tolist() == [1, 1]
+    with pytest.raises(MscclxError) as e:
+        Plan(t)
+    assert e.value.code == binding.ERR_BAD_IR and "outside" in e.value.message
+    with pytest.raises(IRError) as e:
+        parse_algo_xml(ir_samples.relay_through_scratch_xml(out_off=0, out_cnt=2, name_scratch=False))
+    assert "straddle" in str(e.value)
+    from oracle import ir_interp as oi
+    with pytest.raises(ValueError):
+        oi.parse_xml(ir_samples.relay_through_scratch_xml(out_off=0, out_cnt=2, name_scratch=False))
+    a = oi.parse_xml(ir_samples.relay_through_scratch_xml(out_off=1))
+    assert (a.gpus[1].tbs[1].steps[0].dstbuf, a.gpus[1].tbs[1].steps[0].dstoff) == ("o", 1)
+    a = oi.parse_xml(ir_samples.relay_through_scratch_xml(name_scratch=False))
+    assert (a.gpus[1].tbs[0].steps[0].dstbuf, a.gpus[1].tbs[0].steps[0].dstoff) == ("s", 0)
+
+
 def test_two_senders_on_one_connection_rejected(mscclx_lib):
     xml = ir_samples.ring_allreduce_xml(4, instances=2).replace('chan="1"', 'chan="0"')
     with pytest.raises(MscclxError) as e:

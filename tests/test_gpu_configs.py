@@ -202,9 +202,10 @@ def test_aliased_buffers_fall_back_to_staging():
     """An in-place call on an out-of-place algorithm aliases buffers the IR names separately: here every
     rank's 'i' is chunk r of its own 'o' (NCCL's in-place all-gather convention) on an out-of-place
     ring all-gather whose copy threadblock moves i[0] to o[r].  Reading payloads in place assumes
-    distinct memory, so bind refuses with ALIASED and the runner re-plans with every message staged;
-    the aliased run must still deliver the concatenation, and on a program where aliasing makes a
-    receive overwrite what a send of the same rank still has to read, nothing but the refusal is promised."""
+    distinct memory, so bind refuses with ALIASED, and so does the runner unless the caller passes
+    allow_aliased=True; it then re-plans with every message staged, and this program (every write of a
+    chunk writes its final value) must still deliver the concatenation.  On a program where aliasing
+    makes a receive overwrite what a send of the same rank still has to read, nothing but the refusal is promised."""
     import ir_samples
     from msccl.executor import Executor, MscclxError
     from msccl.executor.binding import ERR_ALIASED
@@ -223,12 +224,21 @@ def test_aliased_buffers_fall_back_to_staging():
     with pytest.raises(MscclxError) as e:                        # the C ABI itself refuses ...
         ex.plan.bind([t.data_ptr() for t in ins], [t.data_ptr() for t in outs], [0] * n, ex._workspace.data_ptr(), ex._workspace.numel())
     assert e.value.code == ERR_ALIASED
+    with pytest.raises(MscclxError) as e:                        # ... and so does the runner, unless told otherwise
+        ex.run(ins, outs)
+    assert e.value.code == ERR_ALIASED
     print("case: aliased all-gather, staged", flush=True)
-    ex.run(ins, outs)                                            # ... and the runner falls back to staging
+    ex.run(ins, outs, allow_aliased=True)                        # the caller vouches for the program: every message staged
     assert ex.info.zero_copy_messages == 0 and ex.info.staged_messages > 0
     torch.cuda.synchronize()
     for r in range(n):
         assert np.array_equal(outs[r].cpu().numpy(), want), r
+    # buffers that do not overlap, on the same Executor: back to the knobs setup() was given
+    outs3 = [torch.zeros(n * E, dtype=torch.int32, device="cuda:0") for _ in range(n)]
+    ex.run([torch.from_numpy(v).cuda() for v in x], outs3, allow_aliased=True)
+    assert ex.info.zero_copy_messages > 0
+    for r in range(n):
+        assert np.array_equal(outs3[r].cpu().numpy(), want), r
     # the same data out of place, payloads read in place: the same result
     ex2 = Executor(xml)
     ex2.setup(E * 4, "int32", protocol="simple")
