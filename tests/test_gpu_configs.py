@@ -63,6 +63,21 @@ def test_config_reduced_size_vs_oracle(key, source, mode):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
 
 
+@pytest.mark.parametrize("key", ["c1", "c2", "c5", "c5_chain"])
+def test_config_full_size_vs_oracle_on_the_benchmark_inputs(key):
+    """The configurations whose whole execution the interpreter finishes in seconds, at FULL size, on
+    exactly the inputs the benchmark definition names (NumPy streams default_rng(1000 * cfg + rank)),
+    under the automatic geometry -- what `bench.py` times -- against the interpreter, bit for bit."""
+    w = WORKLOADS[key]
+    xml = w.build()
+    x = [numpy_input(w, r) for r in range(w.ranks)]
+    got, info = device_run(xml, w, x)
+    print(f"{key}: {info.workgroups} workgroups x {info.threads} threads, {info.slices} slices, pieces of {info.piece_bytes} bytes, protocol {info.protocol}", flush=True)
+    want = oracle_run(xml, w, x)
+    for r in range(w.ranks):
+        assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
+
+
 @pytest.mark.parametrize("name", golden_util.names() + golden_util.ncclize_names())
 def test_reference_emitted_programs_vs_oracle(name):
     """Every program msccl-tools' compiler (tests/golden/reference_xml) and its second emitter, ncclize
@@ -247,6 +262,40 @@ def test_aliased_buffers_fall_back_to_staging():
     assert ex2.info.zero_copy_messages > 0
     for r in range(n):
         assert torch.equal(outs2[r], outs[r]), r
+
+
+def test_workspace_handed_from_plan_to_plan_and_back():
+    """One workspace, two plans with different layouts of it, bound in turn: A runs, B is bound to the same
+    memory and runs, A is bound again -- same address, nothing it knows of has failed -- and must find that its
+    counters are no longer its own (B's bind stamped the workspace) and clear them before it runs."""
+    import ir_samples
+    from msccl.executor import Executor, collective_buffers
+    E = 3000
+    plans = {}
+    for name, xml in (("A", ir_samples.ring_allreduce_xml(8, 2)), ("B", ir_samples.allpairs_allreduce_xml(5))):
+        ex = Executor(xml)
+        ex.setup(E * 4, "float32", protocol="simple")
+        plans[name] = (ex, oi.parse_xml(xml))
+    shared = torch.empty(max(int(ex.info.workspace_bytes) for ex, _ in plans.values()), dtype=torch.uint8, device="cuda:0")
+    for turn, name in enumerate("ABABBA"):
+        ex, algo = plans[name]
+        ex._workspace = shared
+        ex._bound = None
+        n = algo.ngpus
+        rng = np.random.default_rng(900 + turn)
+        x = [rng.random(algo.gpus[0].i_chunks * E, dtype=np.float32) * 2 - 1 for _ in range(n)]
+        ins, outs, res = collective_buffers(ex.tables, E * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+        print(f"case: shared workspace, turn {turn}, plan {name}", flush=True)
+        for _ in range(1 + turn % 2):                       # (an odd and an even number of launches: both counter areas get used)
+            for r in range(n):
+                ins[r].copy_(torch.from_numpy(x[r]))
+            ex.run(ins, outs)
+            ex._bound = None
+        torch.cuda.synchronize()
+        want = oc.place_inputs(algo, x, E, "float32")
+        oi.Interpreter(algo).run(want, E, "float32")
+        for r in range(n):
+            assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (turn, name, r)
 
 
 def test_rebind_new_buffers_same_plan():

@@ -632,6 +632,57 @@ def test_abort_from_the_host():
     assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0])
 
 
+def test_graph_replay_after_an_abort():
+    """A launch captured in a HIP graph, replayed after mscclx_plan_abort ended a launch: the replay passes by the
+    host code that re-arms the counters.  The first replay may still find the abort request on the device -- it
+    then ends at once and the wait after it says ABORTED, never OK with a buffer that was not filled -- and the
+    replay after that runs and delivers."""
+    from msccl.executor import Executor, MscclxError, collective_buffers
+    from msccl.executor.binding import ERR_ABORTED
+    xml = ir_samples.slow_producer_xml(200)
+    nbytes = 64 << 20
+    ex = Executor(xml)
+    ex.setup(nbytes, "uint8", slices=1, piece_bytes=nbytes)
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            ex.launch()
+        print("case: replay before the abort", flush=True)
+        graph.replay()
+        ex.wait()
+        assert torch.equal(outs[1].cpu(), x[0])
+        outs[1].zero_()
+        torch.cuda.synchronize()
+        print("case: replay, aborted from the host", flush=True)
+        graph.replay()
+        assert ex.poll()
+        ex.abort()
+        with pytest.raises(MscclxError) as e:
+            ex.wait()
+        assert e.value.code == ERR_ABORTED
+        assert not torch.equal(outs[1].cpu(), x[0])
+        delivered = 0
+        for attempt in range(3):
+            outs[1].zero_()
+            torch.cuda.synchronize()
+            print(f"case: replay {attempt} after the abort", flush=True)
+            graph.replay()
+            try:
+                ex.wait()
+            except MscclxError as err:                        # only the first replay may be refused, and only this way
+                assert err.code == ERR_ABORTED and attempt == 0 and delivered == 0, (attempt, err)
+                continue
+            assert torch.equal(outs[1].cpu(), x[0]) and torch.equal(outs[0].cpu(), x[0]), attempt
+            delivered += 1
+        assert delivered >= 2
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("threads", [0, 64])
 def test_watchdog_in_ll_mode(threads):
     """Flag-in-data lines, one context per workgroup (threads=64: a workgroup of one wave, which runs
