@@ -7,6 +7,9 @@ from msccl.programs.allgather_allpairs import allgather_allpairs
 from msccl.programs.allgather_ring import allgather_ring
 from msccl.programs.allreduce_a100_ring import allreduce_ring
 from msccl.programs.allreduce_allpairs import allreduce_allpairs
+from msccl.programs.allreduce_allpairs_two_level import allreduce_allpairs_two_level
+from msccl.programs.reducescatter_allpairs import reducescatter_allpairs
+from msccl.programs.reducescatter_ring import reducescatter_ring
 from msccl.programs.alltoall_a100_8kp1 import alltoall_three_step
 from msccl.programs.alltoall_allpairs import alltoall_allpairs
 from msccl.programs.alltoall_a100_yifan import alltoall_hierarchical
@@ -138,18 +141,18 @@ def register_mi355x_plans():
     def mi355x_allpairs_allreduce_2x8(prog, nodes):
         allreduce_allpairs(16)
 
-    # Eight groups (64 ranks), fp32, microseconds, two-level / one ring over all ranks (the ring is 126 hand-offs deep, the
-    # two-level program 28): 16 KiB per rank 47 / 170, 256 KiB 73 / 171, 1 MiB 104 / 257, 4 MiB 262 / 358, 8 MiB 419 / 486,
-    # 16 MiB 796 / 768, 24 MiB 1162 / 1132, 64 MiB 3086 / 3008.
-    # One instance of the two-level program has half the threadblocks, each with a workgroup of its own, and runs on flag-in-data
-    # lines up to 64 KiB per rank: 47-49 us against 68-69 with two instances; 256 KiB to 4 MiB the same; 8 MiB 450 against 413.
+    # Eight groups (64 ranks), fp32, microseconds, all-pairs inside the groups and across them (seven moving steps deep) /
+    # two-level program x 2 instances (28 hand-offs deep) / one ring over all ranks (126 deep): 16 KiB per rank 30 / 66 / 170,
+    # 64 KiB 31 / 67 / 169, 256 KiB 42 / 73 / 172, 1 MiB 77 / 106 / 256, 2 MiB 123 / 159 / 299, 4 MiB 239 / 258 / 361,
+    # 8 MiB 457 / 419 / 486, 12 MiB 746 / 604 / 628, 16 MiB 1025 / 794 / 767, 32 MiB 2092 / 1600 / 1524.  (One instance of the
+    # two-level program on flag-in-data lines, the plan for the small sizes before: 47-49 us up to 64 KiB.)
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=1,
-                            sizes=(0, '4MiB'), interleaved_replication=False, machines=lambda x: x == 8)
-    def mi355x_two_level_allreduce_8x8_small(prog, nodes):
-        hierarchical_allreduce(8, 8, "auto")
+                            sizes=(0, '6MiB'), threadblock_policy=manual, dependence_nop=True, machines=lambda x: x == 8)
+    def mi355x_allpairs_two_level_allreduce_8x8(prog, nodes):
+        allreduce_allpairs_two_level(8, 8)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=64, inplace=True, instances=2,
-                            sizes=('4MiB', '12MiB'), interleaved_replication=False, machines=lambda x: x == 8)
+                            sizes=('6MiB', '12MiB'), interleaved_replication=False, machines=lambda x: x == 8)
     def mi355x_two_level_allreduce_8x8(prog, nodes):
         hierarchical_allreduce(8, 8, "auto")
 
@@ -166,7 +169,42 @@ def register_mi355x_plans():
         allreduce_ring(size=16, channels=1)
 
     @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=1024, inplace=True, instances=1,
-                            sizes=('16KiB', '8MiB'), threadblock_policy=manual, interleaved_replication=False,
+                            sizes=('256KiB', '8MiB'), threadblock_policy=manual, interleaved_replication=False,
                             dependence_nop=True, machines=lambda x: x == 4, priority=1)
     def mi355x_allpairs_allreduce_4x8(prog, nodes):
         allreduce_allpairs(32)
+
+    # Below that, all-pairs inside the groups and across them: 16 or 32 chunks where all-pairs over all ranks has 256 or 1024, so
+    # it also serves the sizes at which those would be smaller than an element.  fp32, microseconds, this / all-pairs over all
+    # ranks / two-level -- 32 ranks: 16 KiB per rank 26 / 31 / 34, 64 KiB 26 / 29 / 35, 256 KiB 30 / 30 / 49, 1 MiB 51 / 41 / 69;
+    # 16 ranks: 4 KiB 24 / 22 / 26, 64 KiB 24 / 21 / 28 (all-pairs over all 16 ranks stays ahead wherever its chunks hold an element).
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=32, inplace=True, instances=1,
+                            sizes=(0, '256KiB'), threadblock_policy=manual, dependence_nop=True, machines=lambda x: x == 4, priority=1)
+    def mi355x_allpairs_two_level_allreduce_4x8(prog, nodes):
+        allreduce_allpairs_two_level(4, 8)
+
+    @register_msccl_program(fully_connected(8), 'allreduce', 'mi355x', chunk_factor=16, inplace=True, instances=1,
+                            sizes=(0, '4KiB'), threadblock_policy=manual, dependence_nop=True, machines=lambda x: x == 2, priority=1)
+    def mi355x_allpairs_two_level_allreduce_2x8(prog, nodes):
+        allreduce_allpairs_two_level(2, 8)
+
+    # Reduce-scatter in place (rank r's result is its own input chunks [r * cf, (r + 1) * cf)): all-pairs through scratch, one
+    # hand-off and one fold deep, below about 12 MB per rank, the ring from there on.  fp32, microseconds, all-pairs / ring --
+    # 8 ranks: 8 KiB per rank 13 / 16, 1 MiB 15 / 19, 4 MiB 26 / 28, 8 MiB 37 / 42, 16 MiB 68 / 64, 64 MiB 246 / 209, 256 MiB 1099 / 825;
+    # 16 ranks: 64 KiB 14 / 27, 4 MiB 40 / 61, 8 MiB 67 / 77, 16 MiB 132 / 123, 64 MiB 574 / 439; 32 ranks: 64 KiB 20 / 48, 4 MiB 67 / 119,
+    # 8 MiB 134 / 152, 16 MiB 288 / 243; 64 ranks: 64 KiB 44 / 90, 4 MiB 130 / 238, 8 MiB 290 / 304, 16 MiB 615 / 499.
+    def reduce_scatter_plans(groups, switch):
+        n = 8 * groups
+
+        @register_msccl_program(fully_connected(8), 'reduce_scatter', 'mi355x', chunk_factor=n, inplace=True, instances=1,
+                                sizes=(0, switch), threadblock_policy=manual, dependence_nop=True, machines=lambda x: x == groups)
+        def mi355x_allpairs_reduce_scatter(prog, nodes):
+            reducescatter_allpairs(n)
+
+        @register_msccl_program(fully_connected(8), 'reduce_scatter', 'mi355x', chunk_factor=1, inplace=True, instances=1,
+                                sizes=(switch, None), threadblock_policy=manual, machines=lambda x: x == groups)
+        def mi355x_ring_reduce_scatter(prog, nodes):
+            reducescatter_ring(size=n, channels=1)
+
+    for groups, switch in ((1, '12MB'), (2, '12MB'), (4, '12MB'), (8, '10MiB')):
+        reduce_scatter_plans(groups, switch)

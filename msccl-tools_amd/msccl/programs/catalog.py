@@ -7,7 +7,7 @@ collective's post-condition symbolically and returns the MSCCL-IR XML.
 from __future__ import annotations
 
 from msccl.language import MSCCLProgram, ThreadblockPolicy
-from msccl.language.collectives import AllGather, AllReduce, AllToAll
+from msccl.language.collectives import AllGather, AllReduce, AllToAll, ReduceScatter
 from msccl.topologies import fully_connected
 
 
@@ -110,4 +110,40 @@ def three_step_alltoall(num_nodes, gpus_per_node, instances=1, protocol="Simple"
     prog = MSCCLProgram("alltoall_three_step", fully_connected(n), AllToAll(n, 1, False), 1, protocol=protocol)
     with prog:
         alltoall_three_step(num_nodes, gpus_per_node, instances=instances)
+    return _finish(prog)
+
+
+def ring_reduce_scatter(num_ranks, channels=1, instances=1, protocol="Simple"):
+    """Ring reduce-scatter (msccl.programs.reducescatter_ring): ReduceScatter(n, 1, inplace), manual threadblocks."""
+    from msccl.programs.reducescatter_ring import reducescatter_ring
+    prog = MSCCLProgram(f"reducescatter_ring_{channels}channelsperring", fully_connected(num_ranks), ReduceScatter(num_ranks, 1, True),
+                        instances, protocol=protocol, threadblock_policy=ThreadblockPolicy.manual)
+    with prog:
+        reducescatter_ring(num_ranks, channels)
+    return _finish(prog)
+
+
+def allpairs_reduce_scatter(num_ranks, protocol="Simple"):
+    """All-pairs reduce-scatter (msccl.programs.reducescatter_allpairs): ReduceScatter(n, n, inplace), manual
+    threadblocks and hoisted reduce dependencies as for the all-pairs all-reduce (msccl-tools'
+    msccl/autosynth/ndv4_plans.py:12-22).  One instance only: replication cuts the program's n-chunk copies
+    and its one-chunk reduces differently (msccl/language/rank_dag.py:337-340), and rank r's result would
+    no longer be the contiguous block the collective defines as its output."""
+    from msccl.programs.reducescatter_allpairs import reducescatter_allpairs
+    prog = MSCCLProgram("reducescatter_allpairs", fully_connected(num_ranks), ReduceScatter(num_ranks, num_ranks, True), 1,
+                        protocol=protocol, threadblock_policy=ThreadblockPolicy.manual, dependence_nop=True)
+    with prog:
+        reducescatter_allpairs(num_ranks)
+    return _finish(prog)
+
+
+def allpairs_two_level_allreduce(num_groups, group_size, protocol="Simple"):
+    """All-pairs inside groups and across them (msccl.programs.allreduce_allpairs_two_level): AllReduce(n, n, inplace),
+    manual threadblocks, dependencies of the folds hoisted as for the all-pairs all-reduce."""
+    from msccl.programs.allreduce_allpairs_two_level import allreduce_allpairs_two_level
+    n = num_groups * group_size
+    prog = MSCCLProgram("allreduce_allpairs_two_level", fully_connected(n), AllReduce(n, n, True), 1, protocol=protocol,
+                        threadblock_policy=ThreadblockPolicy.manual, dependence_nop=True)
+    with prog:
+        allreduce_allpairs_two_level(num_groups, group_size)
     return _finish(prog)

@@ -136,3 +136,28 @@ def allpairs_allreduce_orders(n, instances=1):
         r = c // n
         orders.append([r] + [p for p in range(n) if p != r])
     return orders * instances
+
+
+def expected_reduce_scatter(inputs, chunks_per_rank, fold_orders, dtype, redop="sum"):
+    """Reduce-scatter (msccl/language/collectives.py:198-218): out_r[c] = fold over ranks of in_i[r*cf + c],
+    cf = chunks_per_rank, with an explicit fold order per input chunk index r*cf + c."""
+    n = len(inputs)
+    E = np.asarray(inputs[0]).size // (n * chunks_per_rank)
+    outs = []
+    for r in range(n):
+        res = np.empty(chunks_per_rank * E, np.asarray(inputs[0]).dtype)
+        for c in range(chunks_per_rank):
+            k = r * chunks_per_rank + c
+            ops = [np.asarray(inputs[i]).ravel()[k * E:(k + 1) * E] for i in range(n)]
+            res[c * E:(c + 1) * E] = fold(fold_orders[k], ops, dtype, redop)
+        outs.append(res)
+    return outs
+
+
+def ring_reduce_scatter_orders(n, instances=1):
+    """Fold order of the ring reduce-scatter whose chunk k walks k+1 -> k+2 -> ... -> k: ranks k+1, k+2, ...,
+    k (mod n), left to right.  Interleaved replication: chunk k*inst + i follows chunk k."""
+    orders = []
+    for k in range(n):
+        orders.extend([[(k + 1 + m) % n for m in range(n)]] * instances)
+    return orders

@@ -11,7 +11,11 @@ Only msccl.language and msccl.topologies are needed, so the top-level package is
 empty stand-in module object (its __init__ is not executed) and `lxml.etree` is served by the
 standard library's ElementTree, of which the emitter uses Element/SubElement/set/indent/tostring.
 
-usage: python tests/golden/make_reference_xml.py [/root/reference]
+tests/golden/reference_random_xml/*.xml.gz: the same compiler on random programs of tests/random_programs.py
+(instruction fusion on), among them programs it leaves malformed (sends without receives) or with a race:
+what this package's compiler is compared with, byte for byte, on shapes no example has.
+
+usage: python tests/golden/make_reference_xml.py [/root/reference] [--only SUBSTRING]
 """
 import contextlib
 import gzip
@@ -22,7 +26,14 @@ import sys
 import types
 import xml.etree.ElementTree as ET
 
+ONLY = sys.argv[sys.argv.index("--only") + 1] if "--only" in sys.argv else None
+if ONLY is not None:
+    del sys.argv[sys.argv.index("--only"):sys.argv.index("--only") + 2]
 REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+RANDOM_OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_random_xml")
+# fused random programs: well-formed ones, three that come out with unmatched sends and receives (7, 11, 19), two with a
+# race (12, 32), two with an `rrs` (216, 270)
+RANDOM_SEEDS = [0, 1, 2, 3, 4, 5, 6, 7, 11, 12, 19, 32, 216, 270]
 OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_xml")
 sys.dont_write_bytecode = True
 
@@ -115,7 +126,38 @@ def main():
             assert Check()
             XML()
 
+    def reduce_scatter_ring(n, channels, instances):
+        # this repository's msccl/programs/reducescatter_ring.py, through msccl-tools' compiler
+        from msccl.language import chunk, Buffer
+        from msccl.language.collectives import ReduceScatter
+        with MSCCLProgram("reducescatter_ring", fully_connected(n), ReduceScatter(n, 1, True), instances, threadblock_policy=ThreadblockPolicy.manual):
+            for hop in range(n - 1):
+                for k in range(n):
+                    lane = k % channels
+                    here, there = (k + 1 + hop) % n, (k + 2 + hop) % n
+                    chunk(there, Buffer.input, k).reduce(chunk(here, Buffer.input, k), ch=lane, recvtb=lane, sendtb=lane)
+            assert Check()
+            XML()
+
+    def reduce_scatter_allpairs(n):
+        # this repository's msccl/programs/reducescatter_allpairs.py, through msccl-tools' compiler
+        from msccl.language import chunk, Buffer
+        from msccl.language.collectives import ReduceScatter
+        with MSCCLProgram("reducescatter_allpairs", fully_connected(n), ReduceScatter(n, n, True), 1, threadblock_policy=ThreadblockPolicy.manual,
+                          dependence_nop=True):
+            for src in range(n):
+                for dst in range(n):
+                    if src != dst:
+                        chunk(src, Buffer.input, dst * n, size=n).copy(dst, "scratch", sendtb=dst, recvtb=src)
+            for r in range(n):
+                for k in range(n * (n - 1)):
+                    chunk(r, Buffer.input, r * n + k % n).reduce(chunk(r, "scratch", k), sendtb=k % n)
+            assert Check()
+            XML()
+
     jobs = {
+        "reducescatter_ring_8r_1ch_4inst": lambda: from_program(lambda: reduce_scatter_ring(8, 1, 4)),
+        "reducescatter_allpairs_8r": lambda: from_program(lambda: reduce_scatter_allpairs(8)),
         "c1_allreduce_ring_8r_1ch_1inst": lambda: from_program(lambda: ring(8, 1, 1)),
         "c2_allgather_ring_8r_1ch_4inst": lambda: from_example("allgather_ring.py", [8, 1, 4, "--protocol", "Simple"]),
         "c3_alltoall_two_step_2x8": lambda: from_example("alltoall_a100_two_step.py", [2, 8]),
@@ -149,6 +191,8 @@ def main():
     }
     os.makedirs(OUT, exist_ok=True)
     for name, job in jobs.items():
+        if ONLY is not None and ONLY not in name:
+            continue
         try:
             xml = job()
         except (SystemExit, Exception) as e:  # some examples are written against an older DSL and fail upstream too
@@ -159,5 +203,41 @@ def main():
         print(f"{name}: {len(xml)} bytes")
 
 
+def random_programs():
+    """tests/random_programs.py's generator, traced and compiled by msccl-tools' msccl.language.  Every seed is
+    compiled in six processes: msccl-tools walks sets of objects hashed by address (rank_dag.py:156-174,
+    tb_assignment.py:100-128), so where an order is not otherwise fixed its output changes from process to process;
+    every distinct document is kept (random_<seed>_fused, random_<seed>_fused_alt1, ...)."""
+    import subprocess
+    os.makedirs(RANDOM_OUT, exist_ok=True)
+    for seed in RANDOM_SEEDS:
+        name = f"random_{seed}_fused"
+        if ONLY is not None and ONLY not in name:
+            continue
+        variants = []
+        for _ in range(6):
+            out = subprocess.run([sys.executable, os.path.abspath(__file__), REF, "--random-child", str(seed)], capture_output=True, text=True, check=True).stdout
+            if out not in variants:
+                variants.append(out)
+        for old in os.listdir(RANDOM_OUT):
+            if old.startswith(name + "_alt") or old == name + ".xml.gz":
+                os.remove(os.path.join(RANDOM_OUT, old))
+        for k, xml in enumerate(sorted(variants)):
+            with open(os.path.join(RANDOM_OUT, name + (f"_alt{k}" if k else "") + ".xml.gz"), "wb") as f:
+                f.write(gzip.compress(xml.encode(), 9, mtime=0))
+        print(f"{name}: {len(variants)} distinct document(s), {len(variants[0])} bytes")
+
+
+def random_child(seed):
+    install_entry_points()
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import random_programs as rp
+    sys.stdout.write(normalise(rp.random_program(seed, fusion=True)[0]))
+
+
 if __name__ == "__main__":
-    main()
+    if "--random-child" in sys.argv:
+        random_child(int(sys.argv[sys.argv.index("--random-child") + 1]))
+    else:
+        main()
+        random_programs()

@@ -174,9 +174,10 @@ def test_mi355x_alltoall_plans(capsys):
 
 def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
     """16 and 32 virtual ranks: all-pairs over all ranks from 4 KiB to 16 MiB per rank (16 ranks; one ring over all ranks
-    above) or from 16 KiB to 8 MiB (32 ranks), the two-level program elsewhere."""
-    for groups, windows, chunks in ((2, [(0, 4 << 10, 'two_level'), (4 << 10, 16 << 20, 'allpairs'), (16 << 20, float("inf"), 'ring')], 256),
-                                    (4, [(0, 16 << 10, 'two_level'), (16 << 10, 8 << 20, 'allpairs'), (8 << 20, float("inf"), 'two_level')], 1024)):
+    above) or from 256 KiB to 8 MiB (32 ranks; the two-level program above), all-pairs inside the groups and across them
+    below -- 16 or 32 chunks, so it also serves what is too small for the 256 or 1024 chunks of all-pairs over all ranks."""
+    for groups, windows, chunks in ((2, [(0, 4 << 10, 'allpairs_two_level'), (4 << 10, 16 << 20, 'allpairs'), (16 << 20, float("inf"), 'ring')], 256),
+                                    (4, [(0, 256 << 10, 'allpairs_two_level'), (256 << 10, 8 << 20, 'allpairs'), (8 << 20, float("inf"), 'two_level')], 1024)):
         msccl.init('mi355x', groups, ('allreduce', (0, None)))
         capsys.readouterr()
         algos = load_config()
@@ -184,19 +185,41 @@ def test_mi355x_allreduce_windows_of_two_and_four_groups(capsys):
         mid = select(algos, "allreduce", 1 << 20)
         assert mid.tables.ngpus == 8 * groups and mid.tables.nchunksperloop == chunks and mid.tables.inplace
         assert select(algos, "allreduce", 64 << 20).tables.name == f'mi355x_{windows[-1][2]}_allreduce_{groups}x8'
+        small = select(algos, "allreduce", 1 << 10)
+        assert small.tables.nchunksperloop == 8 * groups and small.tables.rank_chunks[0].tolist() == [8 * groups, 0, 7 * groups + groups - 1]
 
 
 def test_mi355x_allreduce_windows_of_eight_groups(capsys):
-    """64 virtual ranks: the two-level program (28 hand-offs deep; one instance below 4 MiB per rank, two above) below
-    12 MiB, one ring over all ranks (126 deep) from there on."""
+    """64 virtual ranks: all-pairs inside the groups and across them (seven moving steps deep) below 6 MiB per rank, the
+    two-level program (28 hand-offs deep, two instances) up to 12 MiB, one ring over all ranks (126 deep) from there on."""
     msccl.init('mi355x', 8, ('allreduce', (0, None)))
     capsys.readouterr()
     algos = load_config()
     assert [(a.min_bytes, a.max_bytes, a.tables.name, a.tables.nchunksperloop) for a in algos] == [
-        (0, 4 << 20, 'mi355x_two_level_allreduce_8x8_small', 64), (4 << 20, 12 << 20, 'mi355x_two_level_allreduce_8x8', 128),
+        (0, 6 << 20, 'mi355x_allpairs_two_level_allreduce_8x8', 64), (6 << 20, 12 << 20, 'mi355x_two_level_allreduce_8x8', 128),
         (12 << 20, float("inf"), 'mi355x_ring_allreduce_8x8', 64)]
     assert all(a.tables.ngpus == 64 for a in algos)
     assert select(algos, "allreduce", 256 << 10) is algos[0]
+
+
+def test_mi355x_reduce_scatter_plans(capsys):
+    """Reduce-scatter, in place: all-pairs through scratch below 12 MB per rank (10 MiB on 64 ranks), the ring from there on;
+    registered through msccl-tools' own decorator (msccl/autosynth/registry.py:65-99, collective 'reduce_scatter')."""
+    from msccl.autosynth.registry import synthesis_plans
+    windows = sorted((low, high) for _, _, machines, (low, high), _, _ in synthesis_plans[('reduce_scatter', 'mi355x')] if machines(8))
+    assert windows == [(0, 10 << 20), (10 << 20, float("inf"))]      # (64 ranks: listed, not compiled here -- 4096 chunks a rank)
+    for groups, switch in ((1, 12 * 10 ** 6), (2, 12 * 10 ** 6)):
+        n = 8 * groups
+        msccl.init('mi355x', groups, (msccl.Collective.reduce_scatter, (0, None)))
+        out = capsys.readouterr().out
+        assert 'mi355x_allpairs_reduce_scatter' in out and 'mi355x_ring_reduce_scatter' in out
+        small, large = load_config()
+        assert (small.min_bytes, small.max_bytes, small.tables.name) == (0, switch, 'mi355x_allpairs_reduce_scatter')
+        assert (large.min_bytes, large.max_bytes, large.tables.name) == (switch, float("inf"), 'mi355x_ring_reduce_scatter')
+        for a, chunks, scratch in ((small, n * n, n * (n - 1)), (large, n, 0)):
+            assert a.tables.coll == "reduce_scatter" and a.tables.inplace and a.tables.ngpus == n
+            assert a.tables.rank_chunks[0].tolist() == [chunks, 0, scratch]
+        assert select(load_config(), "reduce_scatter", 1 << 20) is not None
 
 
 def test_ef_file_plan(tmp_path, capsys):

@@ -77,6 +77,43 @@ def test_config_schedule_invariance(seed):
             assert np.array_equal(base[r].view(np.uint8), rnd[r].view(np.uint8))
 
 
+REDUCE_SCATTERS = {
+    # name of the fixture, this package's builder, input chunks per rank, chunks of the result per rank, fold orders
+    "ring": ("reducescatter_ring_8r_1ch_4inst", lambda: _catalog().ring_reduce_scatter(8, 1, 4), 32, 4, lambda: oc.ring_reduce_scatter_orders(8, 4)),
+    "allpairs": ("reducescatter_allpairs_8r", lambda: _catalog().allpairs_reduce_scatter(8), 64, 8, lambda: oc.allpairs_allreduce_orders(8)),
+}
+
+
+def _catalog():
+    from msccl.programs import catalog
+    return catalog
+
+
+@pytest.mark.parametrize("source", ["msccl-tools", "this-package"])
+@pytest.mark.parametrize("program", sorted(REDUCE_SCATTERS))
+def test_reduce_scatter_matches_closed_form(program, source):
+    """Reduce-scatter in place (msccl/language/collectives.py:172-225): rank r ends with
+    out_r[c] = fold over ranks of in_i[r * cf + c] in its input chunks [r * cf, (r + 1) * cf), in the order the
+    program's text fixes (ring: ranks k+1, k+2, ..., k; all-pairs: the owner, then its peers ascending) -- fp32,
+    bit for bit, and another order gives other bits."""
+    fixture, build, nchunks, per_rank, orders = REDUCE_SCATTERS[program]
+    xml = golden_util.load(fixture) if source == "msccl-tools" else build()
+    algo = oi.parse_xml(xml)
+    assert algo.coll == "reduce_scatter" and algo.inplace and algo.gpus[0].i_chunks == nchunks and algo.gpus[0].o_chunks == 0
+    E = 11
+    rng = np.random.default_rng(31)
+    x = [(rng.random(nchunks * E, dtype=np.float32) * 2 - 1) for _ in range(8)]
+    bufs = oc.place_inputs(algo, x, E, "float32")
+    oi.Interpreter(algo).run(bufs, E, "float32")
+    got = oc.extract_outputs(algo, bufs, E)
+    want = oc.expected_reduce_scatter(x, per_rank, orders(), "float32")
+    other = oc.expected_reduce_scatter(x, per_rank, [list(range(8))[::-1]] * nchunks, "float32")
+    for r in range(8):
+        assert got[r].size == per_rank * E
+        assert np.array_equal(got[r].view(np.uint32), want[r].view(np.uint32)), (program, source, r)
+    assert any(not np.array_equal(want[r].view(np.uint32), other[r].view(np.uint32)) for r in range(8))
+
+
 # every other reference-emitted program: integer data, where any summation order gives the same bits
 OTHERS = {
     "allreduce_ring_8r_4ch_8inst": ("allreduce", 8, 64),

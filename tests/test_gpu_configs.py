@@ -78,6 +78,38 @@ def test_config_full_size_vs_oracle_on_the_benchmark_inputs(key):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
 
 
+@pytest.mark.parametrize("mode", sorted(MODES))
+@pytest.mark.parametrize("source", ["msccl-tools", "this-package"])
+@pytest.mark.parametrize("program", ["ring", "allpairs"])
+def test_reduce_scatter_in_place(program, source, mode):
+    """Reduce-scatter programs, in place (rank r's result is its own input chunks [r * cf, (r + 1) * cf),
+    msccl/language/collectives.py:220-225): collective_buffers' view of the result against the interpreter's,
+    and against the closed form with the fold order the program's text fixes; bf16, so that the order shows."""
+    from msccl.executor import Executor, collective_buffers
+    from test_configs_oracle import REDUCE_SCATTERS
+    fixture, build, nchunks, per_rank, orders = REDUCE_SCATTERS[program]
+    xml = golden_util.load(fixture) if source == "msccl-tools" else build()
+    algo = oi.parse_xml(xml)
+    E = 2600 + (1 if mode == "in-place" else 0)           # chunks of 5200 or 5202 bytes (the latter end inside a dword)
+    rng = np.random.default_rng(63)
+    x = [oi.f32_to_bf16_bits(rng.standard_normal(nchunks * E, dtype=np.float32)) for _ in range(8)]
+    ex = Executor(xml)
+    print(f"case: reduce-scatter {program} from {source}, mode={mode}", flush=True)
+    ex.setup(E * 2, "bfloat16", **MODES[mode])
+    ins, outs, res = collective_buffers(ex.tables, E * 2, "bfloat16", inputs=[to_torch(v, "bfloat16") for v in x])
+    assert all(o is None for o in outs) and all(res[r].data_ptr() == ins[r].data_ptr() + r * per_rank * E * 2 for r in range(8))
+    ex.run(ins, outs)
+    torch.cuda.synchronize()
+    bufs = oc.place_inputs(algo, x, E, "bfloat16")
+    oi.Interpreter(algo).run(bufs, E, "bfloat16")
+    want = oc.extract_outputs(algo, bufs, E)
+    closed = oc.expected_reduce_scatter(x, per_rank, orders(), "bfloat16")
+    for r in range(8):
+        got = to_numpy(res[r], "bfloat16")
+        assert np.array_equal(got, want[r]) and np.array_equal(got, closed[r]), (program, source, mode, r)
+        assert np.array_equal(to_numpy(ins[r], "bfloat16"), bufs[r]["i"]), (program, source, mode, r, "whole buffer")
+
+
 @pytest.mark.parametrize("name", golden_util.names() + golden_util.ncclize_names())
 def test_reference_emitted_programs_vs_oracle(name):
     """Every program msccl-tools' compiler (tests/golden/reference_xml) and its second emitter, ncclize
@@ -390,8 +422,36 @@ def test_init_to_run_allpairs_over_groups(groups, elems, capsys):
     assert all(np.array_equal(res[r].cpu().numpy(), want) for r in range(n))
 
 
+@pytest.mark.parametrize("groups,nbytes,plan", [(1, 8 * 8 * 501 * 4, "allpairs"), (1, 12000000 + 32, "ring"), (2, 16 * 16 * 33 * 4, "allpairs")])
+def test_init_to_run_reduce_scatter(groups, nbytes, plan, capsys):
+    """msccl.init -> MSCCL_CONFIG -> select -> run for reduce-scatter, in place: rank r ends with the sums of its own
+    1/n of the buffer, where it lies in its input (int32: exact in any order)."""
+    import os
+    import msccl
+    from msccl.executor import Executor, collective_buffers, load_config, select
+    for k in ("MSCCL_CONFIG", "NCCL_ALGO"):
+        os.environ.pop(k, None)
+    n = 8 * groups
+    msccl.init('mi355x', groups, ('reduce_scatter', nbytes))
+    capsys.readouterr()
+    rs = select(load_config(), "reduce_scatter", nbytes)
+    assert rs.tables.name == f"mi355x_{plan}_reduce_scatter" and rs.tables.ngpus == n and rs.tables.inplace
+    rng = np.random.default_rng(groups)
+    x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64) for _ in range(n)]
+    cb = rs.bytes_per_rank_to_chunk_bytes(nbytes)
+    ex = Executor(rs.tables)
+    print(f"case: reduce-scatter from msccl.init, {n} ranks, {nbytes} bytes per rank, chunks of {cb} bytes", flush=True)
+    ex.setup(cb, "int32")
+    ins, outs, res = collective_buffers(ex.tables, cb, "int32", inputs=[torch.from_numpy(v.astype(np.int32)) for v in x])
+    ex.run(ins, outs)
+    total = sum(x).astype(np.int32)                             # wraps like the device's 32-bit adds
+    per = nbytes // 4 // n
+    for r in range(n):
+        assert np.array_equal(res[r].cpu().numpy(), total[r * per:(r + 1) * per]), r
+
+
 def test_init_to_run_allreduce_over_eight_groups(capsys):
-    """64 virtual ranks at 256 KiB per rank: msccl.init picks the two-level all-reduce (int32 sums, exact in any order)."""
+    """64 virtual ranks at 256 KiB per rank: msccl.init picks all-pairs inside the groups and across them (int32 sums, exact in any order)."""
     import os
     import msccl
     from msccl.executor import Executor, collective_buffers, load_config, select
@@ -401,7 +461,7 @@ def test_init_to_run_allreduce_over_eight_groups(capsys):
     msccl.init('mi355x', 8, ('allreduce', nbytes))
     capsys.readouterr()
     ar = select(load_config(), "allreduce", nbytes)
-    assert ar.tables.name == "mi355x_two_level_allreduce_8x8_small" and ar.tables.ngpus == n
+    assert ar.tables.name == "mi355x_allpairs_two_level_allreduce_8x8" and ar.tables.ngpus == n
     rng = np.random.default_rng(64)
     x = [rng.integers(-2 ** 31, 2 ** 31, nbytes // 4, dtype=np.int64) for _ in range(n)]
     cb = ar.bytes_per_rank_to_chunk_bytes(nbytes)
