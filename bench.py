@@ -23,7 +23,8 @@ which matters for the two latency-bound workloads (a launch on an idle GPU pays 
 metric/value: algbw in GB/s (nccl-tests convention, S / t).  "roofline": algorithmic bytes per launch
 / mean launch duration against the 8 TB/s HBM peak.  "cpu_baseline": the NumPy interpreter of the
 same IR on this box's host cores (reported, not a target).  "host_us": what a caller pays on the host
-for plan creation, configuration, binding and launching.  "roofline.streaming_reference": what torch's own
+for plan creation, configuration, binding and launching the first time, and what the executor cache
+(msccl.executor.cache) makes of the same request when it comes again.  "roofline.streaming_reference": what torch's own
 copy and add kernels reach on the same box over 1 GiB arrays (read + write bytes), a yardstick beside the peak.
 """
 import argparse
@@ -139,13 +140,16 @@ def fold_orders(key):
 
 def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_costs=False, knobs=None):
     import torch
-    from msccl.executor import Executor, collective_buffers, parse_algo_xml
+    import gc
+    from msccl.executor import Executor, cache, collective_buffers
     from msccl.executor.workloads import WORKLOADS, torch_input
     w = WORKLOADS[key] if bytes_per_rank is None else WORKLOADS[key].scaled(bytes_per_rank)
     xml = WORKLOADS[key].build()
     host = {}
+    cache.clear()
+    gc.collect()  # (a collection of the garbage the previous workload left would otherwise land in whichever step allocates next)
     t0 = time.perf_counter()
-    tables = parse_algo_xml(xml)
+    tables = cache.tables_for(xml)
     host["parse_xml"] = time.perf_counter() - t0
     t0 = time.perf_counter()
     ex = Executor(tables, device=device)
@@ -177,6 +181,21 @@ def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_
         ex.bind(ins, outs)
         host["bind_again"] = min(host["bind_again"], ex.host_seconds["bind"])
         del ins2, outs2
+        # the executor cache: the first request for (document, chunk size, type, knobs) builds everything above once
+        # more; the same request again is a lookup -- by the text's hash, or by the tables the caller kept
+        gc.collect()
+        t0 = time.perf_counter()
+        kept = cache.executor_for(xml, w.chunk_bytes, w.dtype, device=device, **(knobs or {}))
+        host["executor_for_first"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        again = cache.executor_for(xml, w.chunk_bytes, w.dtype, device=device, **(knobs or {}))
+        host["executor_for_again_from_text"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        again2 = cache.executor_for(tables, w.chunk_bytes, w.dtype, device=device, **(knobs or {}))
+        host["executor_for_again_from_tables"] = time.perf_counter() - t0
+        assert again is kept and again2 is kept
+        del kept, again, again2
+        cache.clear()
     for _ in range(warmup):
         restore()
         ex.launch()
@@ -349,7 +368,7 @@ def main():
         for key in sorted(WORKLOADS):
             if key == args.config:
                 continue
-            r = run_workload(key, max(5, args.steps // 2), args.warmup, host_costs=key in ("c4", "c5"))
+            r = run_workload(key, max(5, args.steps // 2), args.warmup, host_costs=key in ("c3", "c4", "c5"))
             line["others"][key] = {k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items() if k != "geometry"}
             line["others"][key].update(r["geometry"])
             line["others"][key]["traffic"] = traffic.get(key)

@@ -10,4 +10,7 @@ def __getattr__(name):
     if name in ("Executor", "collective_buffers", "dtype_name"):
         from . import runner
         return getattr(runner, name)
+    if name in ("executor_for", "tables_for"):
+        from . import cache
+        return getattr(cache, name)
     raise AttributeError(name)

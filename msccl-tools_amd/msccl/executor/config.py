@@ -8,7 +8,7 @@ import math
 import os
 import xml.etree.ElementTree as ET
 
-from .ir_tables import AlgoTables, IRError, load_algo
+from .ir_tables import AlgoTables, IRError
 
 
 @dataclasses.dataclass
@@ -31,6 +31,14 @@ class LoadedAlgo:
         return nbytes // chunks
 
 
+def _load(path):
+    """The tables of the document at `path`: parsed once per distinct text (msccl.init writes a new temporary file for
+    the same program every time it is called)."""
+    from .cache import tables_for
+    with open(path, "r") as f:
+        return tables_for(f.read())
+
+
 def load_config(path=None):
     """Parse the index at `path` (default: $MSCCL_CONFIG) and every algorithm it lists."""
     path = path or os.environ.get("MSCCL_CONFIG")
@@ -45,7 +53,7 @@ def load_config(path=None):
         if p is None:
             raise IRError(f"{path}: <load> without path")
         algos.append(LoadedAlgo(p, int(load.get("minBytes", "0")), float(load.get("maxBytes", "inf")),
-                                load.get("proto", "Simple"), load_algo(p)))
+                                load.get("proto", "Simple"), _load(p)))
     return algos
 
 

@@ -32,6 +32,7 @@ class AlgoTables:
     rank_chunks: np.ndarray  # [ngpus, 3] int32: i_chunks, o_chunks, s_chunks
     tbs: np.ndarray          # [ntbs, 6] int32: rank, send, recv, chan, op_begin, op_end
     ops: np.ndarray          # [nops, 9] int32: type, srcbuf, srcoff, dstbuf, dstoff, cnt, depid, deps, hasdep
+    document_key: str = ""   # hash of the XML text these tables were parsed from (set by msccl.executor.cache.tables_for)
 
     @property
     def ntbs(self):

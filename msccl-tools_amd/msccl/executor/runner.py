@@ -36,7 +36,11 @@ class Executor:
     """plan = Executor(xml_or_tables); plan.setup(chunk_bytes, dtype); plan.run(inputs, outputs)."""
 
     def __init__(self, algo, device="cuda:0"):
-        self.tables = algo if isinstance(algo, AlgoTables) else parse_algo_xml(algo)
+        if isinstance(algo, AlgoTables):
+            self.tables = algo
+        else:  # XML text: parsed once per distinct document
+            from .cache import tables_for
+            self.tables = tables_for(algo)
         self.device = torch.device(device)
         self.plan = Plan(self.tables)
         self.info = None

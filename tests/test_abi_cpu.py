@@ -321,3 +321,20 @@ def test_run_static_refuses_an_oversized_plan_before_touching_the_gpu(mscclx_lib
     with pytest.raises(MscclxError) as e:
         p.run_static(fake, [0] * t.ngpus, [0] * t.ngpus)
     assert e.value.code == binding.ERR_CAPACITY and "MSCCLX_STATIC_SCRATCH_BYTES" in e.value.message
+
+
+def test_documents_are_parsed_once(mscclx_lib):
+    """Tables are kept by the hash of the document's text: the same text again (another Executor, another temporary file
+    written by msccl.init for the same program) costs a hash, not a parse; another text gets tables of its own."""
+    from msccl.executor import cache
+    cache.clear()
+    xml = ir_samples.ring_allreduce_xml(8)
+    a = cache.tables_for(xml)
+    assert cache.tables_for(xml) is a and a.document_key == cache.document_key(xml) and len(a.document_key) == 40
+    other = cache.tables_for(xml.replace('name="', 'name="x'))
+    assert other is not a and other.document_key != a.document_key and (other.ops == a.ops).all()
+    for k in range(cache.MAX_DOCUMENTS + 3):                         # bounded: the entry unused for longest goes
+        cache.tables_for(xml.replace('name="', f'name="{k}_'))
+    assert len(cache._tables) == cache.MAX_DOCUMENTS and a.document_key not in cache._tables
+    with pytest.raises(ValueError):
+        cache.executor_for(parse_algo_xml(xml), 1024, "float32")     # tables that did not come from the cache carry no key

@@ -63,11 +63,12 @@ def test_config_reduced_size_vs_oracle(key, source, mode):
         assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (key, r)
 
 
-@pytest.mark.parametrize("key", ["c1", "c2", "c5", "c5_chain"])
+@pytest.mark.parametrize("key", ["c1", "c2", "c3", "c4", "c5", "c5_chain"])
 def test_config_full_size_vs_oracle_on_the_benchmark_inputs(key):
-    """The configurations whose whole execution the interpreter finishes in seconds, at FULL size, on
-    exactly the inputs the benchmark definition names (NumPy streams default_rng(1000 * cfg + rank)),
-    under the automatic geometry -- what `bench.py` times -- against the interpreter, bit for bit."""
+    """Every configuration at FULL size, on exactly the inputs the benchmark definition names (NumPy
+    streams default_rng(1000 * cfg + rank)), under the automatic geometry -- what `bench.py` times --
+    against the interpreter, bit for bit.  (The largest, 32 ranks x 128 MiB of bf16, takes the interpreter
+    a few seconds and drawing its inputs most of a minute.)"""
     w = WORKLOADS[key]
     xml = w.build()
     x = [numpy_input(w, r) for r in range(w.ranks)]
@@ -328,6 +329,38 @@ def test_workspace_handed_from_plan_to_plan_and_back():
         oi.Interpreter(algo).run(want, E, "float32")
         for r in range(n):
             assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (turn, name, r)
+
+
+def test_executor_cache_hands_back_a_working_executor():
+    """msccl.executor.cache.executor_for: the same (document, chunk size, type, knobs) again gives the executor made the
+    first time -- in microseconds -- and it still delivers on new buffers; another chunk size gets an executor of its own."""
+    import time
+    import ir_samples
+    from msccl.executor import cache, collective_buffers
+    cache.clear()
+    xml = ir_samples.allpairs_allreduce_xml(6)
+    algo = oi.parse_xml(xml)
+    E = 2000
+    first = cache.executor_for(xml, E * 4, "float32")
+    t0 = time.perf_counter()
+    again = cache.executor_for(xml, E * 4, "float32")
+    lookup = time.perf_counter() - t0
+    assert again is first and lookup < 2e-3
+    assert cache.executor_for(cache.tables_for(xml), E * 4, torch.float32) is first            # by tables, dtype given as torch's
+    other = cache.executor_for(xml, 2 * E * 4, "float32")
+    assert other is not first and other.tables is first.tables
+    for ex, elems, seed in ((first, E, 1), (other, 2 * E, 2), (again, E, 3)):
+        rng = np.random.default_rng(seed)
+        x = [rng.random(6 * elems, dtype=np.float32) * 2 - 1 for _ in range(6)]
+        ins, outs, res = collective_buffers(ex.tables, elems * 4, "float32", inputs=[torch.from_numpy(v) for v in x])
+        print(f"case: cached executor, chunks of {elems} floats", flush=True)
+        ex.run(ins, outs)
+        torch.cuda.synchronize()
+        want = oc.place_inputs(algo, x, elems, "float32")
+        oi.Interpreter(algo).run(want, elems, "float32")
+        for r in range(6):
+            assert np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r]["i"].view(np.uint32)), (seed, r)
+    cache.clear()
 
 
 def test_rebind_new_buffers_same_plan():
