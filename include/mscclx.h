@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MSCCLX_VERSION 3
+#define MSCCLX_VERSION 4
 
 typedef enum {
   MSCCLX_OK = 0,
@@ -79,6 +79,13 @@ typedef enum {
  * the data itself -- twice the slot traffic, about half the latency per hop; meant for small pieces
  * (the trade msccl-tools names with proto="LL", msccl/language/__init__.py:38-39). */
 typedef enum { MSCCLX_PROTO_AUTO = 0, MSCCLX_PROTO_SIMPLE = 1, MSCCLX_PROTO_LL = 2 } mscclx_protocol;
+
+/* The step loop a launch runs (reported, not chosen: it follows from the geometry).  HOSTED: workgroups of any size that
+ * host several (threadblock, slice) contexts each and poll for all of them.  The CHAIN loops serve one-wave workgroups
+ * with one context each -- the shape of latency-bound launches: LINES for flag-in-data lines, COUNTERS for counters,
+ * FOLD for counters in programs whose nop steps are folded into the steps behind them (msccl/language/ir.py:296-311
+ * gives a step one dependency and puts a nop in front of it for every other: the all-pairs family). */
+typedef enum { MSCCLX_LOOP_HOSTED = 0, MSCCLX_LOOP_CHAIN_LINES = 1, MSCCLX_LOOP_CHAIN_COUNTERS = 2, MSCCLX_LOOP_CHAIN_FOLD = 3 } mscclx_loop;
 
 typedef enum { MSCCLX_SUM = 0, MSCCLX_PROD = 1, MSCCLX_MAX = 2, MSCCLX_MIN = 3, MSCCLX_NUM_REDOPS = 4 } mscclx_redop;
 
@@ -132,6 +139,8 @@ typedef struct {
   int32_t protocol;    /* MSCCLX_PROTO_SIMPLE or MSCCLX_PROTO_LL                    */
   int32_t waiting_ratio_x100; /* 100 * threadblocks * depth of the dataflow / moving steps: 100 = every threadblock always has work (a ring) */
   int32_t dataflow_depth;     /* moving steps on the longest chain through step order, dependencies and messages */
+  int32_t kernel_loop; /* mscclx_loop: which of the kernels' step loops this geometry runs */
+  int32_t reserved;
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

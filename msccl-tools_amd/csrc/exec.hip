@@ -6,6 +6,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <utility>
 #include <string>
@@ -51,6 +52,7 @@ struct DeviceImage {
   size_t off_tbs = 0, off_ops = 0, off_extras = 0, off_conns = 0, off_hosting = 0, off_ctxs = 0;
   bool one_each = false;              // workgroup w hosts context w and no other
   bool long_folds = false;            // some step stands for more folded nops than a lane checks by itself
+  bool chain_fold = false;            // folded nops on one-wave workgroups with one context each: exec_kernel_chain_fold
   std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
   std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
   kernel_fn kernel = nullptr;
@@ -85,18 +87,31 @@ void destroy_device_state(DeviceState* d) {
   delete d;
 }
 
+// Resident workgroups of kernel k on the current device, per thread count.  Asked of the runtime once per (device, kernel):
+// the answers never change, and the queries (device properties, five occupancy calculations) cost milliseconds.
 static int query_capacity(kernel_fn k, int* num_cus, int capacity[kThreadChoices]) {
+  struct Known { int num_cus; int capacity[kThreadChoices]; };
+  static std::mutex mutex;
+  static std::map<std::pair<int, const void*>, Known> known;
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
-  hipDeviceProp_t prop;
-  HIP_TRY(hipGetDeviceProperties(&prop, dev));
-  *num_cus = prop.multiProcessorCount;
-  const int threads[kThreadChoices] = {64, 128, 256, 512, 1024};
-  for (int i = 0; i < kThreadChoices; ++i) {
-    int per_cu = 0;
-    HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, threads[i], 0));
-    capacity[i] = per_cu * prop.multiProcessorCount;
+  std::lock_guard<std::mutex> lock(mutex);
+  auto it = known.find({dev, (const void*)k});
+  if (it == known.end()) {
+    Known kn{};
+    int cus = 0;
+    HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    kn.num_cus = cus;
+    const int threads[kThreadChoices] = {64, 128, 256, 512, 1024};
+    for (int i = 0; i < kThreadChoices; ++i) {
+      int per_cu = 0;
+      HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, threads[i], 0));
+      kn.capacity[i] = per_cu * cus;
+    }
+    it = known.emplace(std::make_pair(dev, (const void*)k), kn).first;
   }
+  *num_cus = it->second.num_cus;
+  for (int i = 0; i < kThreadChoices; ++i) capacity[i] = it->second.capacity[i];
   return MSCCLX_OK;
 }
 
@@ -146,6 +161,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
   const Geometry& g = plan->geo;
   const bool fold = !g.ll && has_foldable_nops(*plan);
   DeviceImage* d = img;
+  d->chain_fold = fold && one_wave_each(g);
   const size_t ntb = plan->tbs.size(), nop = plan->ops.size(), ncn = plan->conns.size();
   std::vector<DevTb> htb(ntb);
   std::vector<DevOp> hop(nop);
@@ -190,7 +206,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
           dv.in_addr = (uint64_t)(uintptr_t)bufs[(size_t)sender_rank * 3 + (from_src ? sender.srcbuf : sender.dstbuf)] +
                        (uint64_t)(from_src ? sender.srcoff : sender.dstoff) * plan->chunk_bytes;
           const Tb& sender_tb = plan->tbs[plan->conns[tb.recv_conn].send_tb];
-          if (from_src && op.match_send == sender_tb.op_begin && sender.depid < 0) dv.steps |= kStepsPayloadAtLaunch;
+          if (from_src && op.match_send == sender_tb.op_begin && sender.depid < 0) dv.steps |= kStepsNoAnnouncement;
         }
       }
     }
@@ -217,7 +233,9 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
         longest_run = std::max(longest_run, run);
       }
     }
-    const size_t most_folded = longest_run > 2 * (size_t)kLaneExtraDeps ? (size_t)kMaxExtraDeps : (size_t)kLaneExtraDeps;
+    // (exec_kernel_chain_fold checks a dependency per lane whatever their number: every run is folded, up to what its lanes hold)
+    const size_t most_folded = d->chain_fold ? (size_t)kMaxChainFoldDeps - 1
+                                             : longest_run > 2 * (size_t)kLaneExtraDeps ? (size_t)kMaxExtraDeps : (size_t)kLaneExtraDeps;
     for (size_t t = 0; t < ntb; ++t) {
       const Tb& tb = plan->tbs[t];
       d->dev_op_begin[t] = (int32_t)folded_ops.size();
@@ -239,7 +257,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
         if (first >= (1u << 24)) return fail(MSCCLX_ERR_CAPACITY, "too many folded dependencies");
         dv.extra = (uint32_t)(first << 8) | (uint32_t)(pending.size() / kExtraDepWords);
         if (pending.size() / kExtraDepWords > (size_t)kLaneExtraDeps) d->long_folds = true;
-        dv.steps = (dv.steps & kStepsPayloadAtLaunch) | (1 + folded);
+        dv.steps = (dv.steps & kStepsNoAnnouncement) | (1 + folded);
         extras.insert(extras.end(), pending.begin(), pending.end());
         pending.clear();
         folded = 0;
@@ -304,7 +322,54 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
     hop.swap(fused);
     d->dev_ir_step.swap(fused_ir);
   }
-  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, fold ? (img->long_folds ? 2 : 1) : 0, plan->chunk_bytes % 16 != 0);
+  if (d->chain_fold && !g.staging) {
+    // Receives take over the waits of sends that only announce.  S: an `s` whose payload is read in place; R: the receive
+    // that reads it.  S moves nothing: it waits for its dependencies (its own and those of the nops folded into it) and
+    // for the steps in front of it in its threadblock, then raises the connection's head -- one hand-off, which R spares
+    // by waiting for the same counters itself.  Everything that happened before S still happens before R; every later
+    // writer of the payload comes after R on the program's happens-before graph, or the payload would not be read in
+    // place at all.  The step in front of S must publish its threadblock's flag for this.
+    std::vector<int32_t> dev_of_ir(nop, -1);  // row of an IR step in plan->ops -> its step in the device's list
+    for (size_t t = 0; t < ntb; ++t)
+      for (int32_t i = htb[t].op_begin; i < htb[t].op_begin + htb[t].nops; ++i) dev_of_ir[(size_t)(plan->tbs[t].op_begin + d->dev_ir_step[(size_t)i])] = i;
+    for (size_t t = 0; t < ntb; ++t) {
+      const Tb& tb = plan->tbs[t];
+      for (int32_t i = htb[t].op_begin; i < htb[t].op_begin + htb[t].nops; ++i) {
+        DevOp& rv = hop[(size_t)i];
+        if (!is_recv_type((int)(rv.word & 15u)) || !(rv.word & kOpInPlace) || (rv.steps & kStepsNoAnnouncement)) continue;
+        const Op& rop = plan->ops[(size_t)(tb.op_begin + d->dev_ir_step[(size_t)i])];
+        const int32_t si = rop.match_send >= 0 ? dev_of_ir[(size_t)rop.match_send] : -1;
+        if (si < 0) continue;
+        const DevOp& sv = hop[(size_t)si];
+        if ((sv.word & 15u) != MSCCLX_OP_SEND || (sv.word & kOpOutStaged)) continue;  // (an rcs / rrcs writes its payload itself: it must have run)
+        const size_t st = (size_t)plan->conns[(size_t)tb.recv_conn].send_tb;       // the sending threadblock's row
+        const int32_t s_first = htb[st].op_begin, s_steps = htb[st].nops;
+        const uint32_t s_ir_steps = (uint32_t)(plan->tbs[st].op_end - plan->tbs[st].op_begin);
+        const uint32_t s_folded = (sv.steps & ~kStepsNoAnnouncement) - 1;                       // nops folded into S
+        const uint32_t before_s = (uint32_t)d->dev_ir_step[(size_t)si] - s_folded;              // IR steps of the threadblock in front of S and its nops
+        const bool waits_for_steps = before_s > 0 || g.passes > 1;
+        const size_t mine = rv.extra & 255u, theirs = sv.extra & 255u;
+        const size_t total = mine + theirs + (sv.dep_tb >= 0 ? 1 : 0) + (waits_for_steps ? 1 : 0);
+        if (total > (size_t)kMaxChainFoldDeps || s_ir_steps >= 65536u || (sv.dep_tb >= 0 && sv.dep_nops >= 65536)) continue;
+        const size_t first = extras.size() / kExtraDepWords;
+        if (first + total >= (1u << 24)) continue;
+        for (size_t k = 0; k < mine * kExtraDepWords; ++k) extras.push_back(extras[(size_t)(rv.extra >> 8) * kExtraDepWords + k]);
+        for (size_t k = 0; k < theirs * kExtraDepWords; ++k) extras.push_back(extras[(size_t)(sv.extra >> 8) * kExtraDepWords + k]);
+        if (sv.dep_tb >= 0) {
+          extras.push_back((uint32_t)sv.dep_tb * kSyncStrideWords);
+          extras.push_back(((uint32_t)sv.dep_step + 1) | ((uint32_t)sv.dep_nops << 16));
+        }
+        if (waits_for_steps) {
+          extras.push_back((uint32_t)st * kSyncStrideWords);
+          extras.push_back(before_s | (s_ir_steps << 16));
+          hop[(size_t)(si > s_first ? si - 1 : s_first + s_steps - 1)].word |= kOpHasdep;  // the step in front of S (the last one, of the pass before, when S is the first)
+        }
+        rv.extra = (uint32_t)(first << 8) | (uint32_t)total;
+        rv.steps |= kStepsNoAnnouncement;
+      }
+    }
+  }
+  img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, d->chain_fold ? 3 : fold ? (img->long_folds ? 2 : 1) : 0, plan->chunk_bytes % 16 != 0);
   if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   // One record per hosted context, in hosting order: where its counters and slots are, its slice's bounds.
   std::vector<DevCtx> ctxs(g.ctx_tb.size());
@@ -481,6 +546,9 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
       rc = query_capacity(pick_kernel(dtype, redop, ll, 2, ragged), &num_cus, other);
       if (rc) return rc;
       for (int i = 0; i < kThreadChoices; ++i) capacity[i] = std::min(capacity[i], other[i]);
+      rc = query_capacity(pick_kernel(dtype, redop, ll, 3, ragged), &num_cus, other);  // one-wave workgroups with one context each run on exec_kernel_chain_fold
+      if (rc) return rc;
+      capacity[0] = std::min(capacity[0], other[0]);
     }
     if (cfg.protocol == MSCCLX_PROTO_AUTO && !fold) {  // the geometry may choose LL lines by itself: what fits must fit either kernel
       int other[kThreadChoices];
@@ -508,6 +576,9 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
     info->waiting_ratio_x100 = (int32_t)std::min(2.0e9, g.waiting_ratio * 100.0 + 0.5);
     info->dataflow_depth = g.dataflow_depth;
+    info->kernel_loop = !one_wave_each(g) ? MSCCLX_LOOP_HOSTED : g.ll ? MSCCLX_LOOP_CHAIN_LINES
+                        : has_foldable_nops(*plan) ? MSCCLX_LOOP_CHAIN_FOLD : MSCCLX_LOOP_CHAIN_COUNTERS;
+    info->reserved = 0;
     info->threads = g.threads;
     info->slices = g.slices;
     info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);

@@ -713,7 +713,7 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     if (LL) {
       c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
       c.t1 = ll_flag(epoch, c.rseq);
-    } else if (!(in_place && (op.steps & kStepsPayloadAtLaunch))) {
+    } else if (!(in_place && (op.steps & kStepsNoAnnouncement))) {
       c.w1 = p.sync_cur + h.head_in;
       c.t1 = c.rseq + 1;
     }
@@ -1227,7 +1227,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
     {  // what the step waits for: a step of another threadblock, the incoming message, a free outgoing slot -- one round of loads for all
       const u64* const w0 = op.dep_tb >= 0 ? flags + (uint32_t)op.dep_tb * kSyncStrideWords : nullptr;
       const u64 t0 = (u64)pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1;
-      const u64* const w1 = (rcv_bit && !(op.steps & kStepsPayloadAtLaunch)) ? in_head : nullptr;  // (the bit is only set on payloads read in place)
+      const u64* const w1 = (rcv_bit && !(op.steps & kStepsNoAnnouncement)) ? in_head : nullptr;  // (the bit is only set on payloads read in place)
       const u64 t1 = (u64)rseq + 1;
       const u64* const w2 = (snd_bit && sseq >= depth) ? out_tail : nullptr;
       const u64 t2 = (u64)sseq + 1 - depth;
@@ -1321,6 +1321,45 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
 #endif
 }
 
+// The start of a launch.  The number of launches so far is kept on the device (control word 0) and is advanced by the
+// last workgroup to finish, so a launch carries no host-side state and the same launch can be replayed (stream
+// order guarantees the next launch sees the new value).  Its lowest bit picks which of the two counter areas this
+// launch uses; its low 10 bits mark the LL lines.  Returns that number.
+__device__ __forceinline__ u64 begin_launch(KernelParams& p) {
+  const u64 launch_no = load_counter(p.sync_base);
+  const u64 parity = launch_no & 1ull;
+  p.sync_cur = p.sync_base + kControlWords + parity * p.sync_words;
+  p.sync_nxt = p.sync_base + kControlWords + (parity ^ 1ull) * p.sync_words;
+  return launch_no;
+}
+
+// The end of a workgroup.  The last workgroup out re-arms the control block: the next launch uses the other counter
+// area.  "Last" is found group by group (the last of a group reports for the group), so that no address sees more
+// than a few dozen atomics.
+__device__ __forceinline__ void end_launch(const KernelParams& p, const u64 launch_no) {
+  if (threadIdx.x == 0) {
+    const unsigned per = p.finish_group, group = blockIdx.x / per, groups = (gridDim.x + per - 1) / per;
+    const unsigned members = group + 1 < groups ? per : gridDim.x - group * per;
+    u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
+    if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
+      publish(group_count, 0);
+      bool last = groups == 1;  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
+      if (!last && __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
+        publish(p.sync_base + 1, 0);
+        last = true;
+      }
+      if (last) {
+        // A launch that ran under a host's abort request says so itself: whoever replays it from a HIP graph passes
+        // by the host code that would have re-armed the counters, and must still learn that it did not run.
+        if (load_counter(p.sync_cur) == kAbortByHost &&
+            __hip_atomic_load(&p.host_status->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
+          __hip_atomic_store(&p.host_status->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        publish(p.sync_base, launch_no + 1);
+      }
+    }
+  }
+}
+
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
 // active context waits for (one round of loads covers all of them), finishes steps that move no data
 // on the spot, and picks a ready context whose step does move data; the whole workgroup then copies /
@@ -1335,13 +1374,8 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
   // replayed (stream order guarantees the next launch sees the new value).  Its lowest bit picks
   // which of the two counter areas this launch uses; its low 10 bits mark the LL lines.
   KernelParams p = launch_params;
-  const u64 launch_no = load_counter(p.sync_base);
+  const u64 launch_no = begin_launch(p);
   const uint32_t epoch = (uint32_t)launch_no & 0x3ffu;
-  {
-    const u64 parity = launch_no & 1ull;
-    p.sync_cur = p.sync_base + kControlWords + parity * p.sync_words;
-    p.sync_nxt = p.sync_base + kControlWords + (parity ^ 1ull) * p.sync_words;
-  }
   __shared__ int sh_choice;
   __shared__ Move sh_move;
   __shared__ uint32_t sh_seq[2];   // LL: numbers of the incoming and the outgoing message
@@ -1546,30 +1580,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
   }
   }  // hosted contexts
-  if (threadIdx.x == 0) {
-    // The last workgroup out re-arms the control block: the next launch uses the other counter area.
-    // "Last" is found group by group (the last of a group reports for the group), so that no
-    // address sees more than a few dozen atomics.
-    const unsigned per = p.finish_group, group = blockIdx.x / per, groups = (gridDim.x + per - 1) / per;
-    const unsigned members = group + 1 < groups ? per : gridDim.x - group * per;
-    u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
-    if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
-      publish(group_count, 0);
-      bool last = groups == 1;  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
-      if (!last && __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
-        publish(p.sync_base + 1, 0);
-        last = true;
-      }
-      if (last) {
-        // A launch that ran under a host's abort request says so itself: whoever replays it from a HIP graph passes
-        // by the host code that would have re-armed the counters, and must still learn that it did not run.
-        if (load_counter(abort_word) == kAbortByHost &&
-            __hip_atomic_load(&p.host_status->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
-          __hip_atomic_store(&p.host_status->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-        publish(p.sync_base, launch_no + 1);
-      }
-    }
-  }
+  end_launch(p, launch_no);
 #ifdef MSCCLX_PROFILE
   if (threadIdx.x == 0 && p.prof) {
     p.prof[(size_t)blockIdx.x * kProfWords + 0] = prof_wait;
@@ -1585,6 +1596,152 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
 }
 
+// Programs with folded nops on one-wave workgroups with one context each (the all-pairs family on small messages: the
+// all-reduce, all-gather and all-to-all plans below a few MiB per rank): a kernel of its own, so that neither loop pays
+// for the other's registers.  The step waits of such programs are many -- a step that stands for a run of nops waits for
+// each nop's threadblock, a receive that has taken over its sender's waits for those too -- and all of one kind: a
+// counter that must reach a value.  So every wait of a step sits in a lane of its own (the folded ones first, then the
+// step's own dependency, the incoming message's announcement, the outgoing connection's free slot), and one vector load
+// and one ballot check them all: one round trip per poll however many counters a step waits for, where the hosting loop
+// makes three in a row (its counters, the table of folded dependencies, their counters).  The table entries of the next
+// step are asked for while this step waits.  The moves are the hosting loop's own (do_move), with the wave as the workgroup.
+template <class R, bool RAGGED>
+__global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams launch_params) {
+  KernelParams p = launch_params;
+  const u64 launch_no = begin_launch(p);
+  const uint32_t lane = threadIdx.x;
+  const bool writer = lane == 0;
+  if (writer && blockIdx.x == 0) p.sync_nxt[0] = 0;
+  Hosted h;
+  uint32_t left;  // units of the slice still to do (this pass included)
+  u64 off;        // byte offset of this pass's piece inside every chunk
+  bool active;
+  {
+    Context first;
+    init_context<false, RAGGED>(h, first, p, 0, (int)blockIdx.x, writer);  // (a workgroup hosts the context of its own number)
+    active = first.active;
+    left = uniform(first.left);
+    off = uniform((uint64_t)first.off);
+  }
+  if (active) {
+    const ConstOps ops = (ConstOps)(p.ops + uniform(h.op_begin));
+    const uint2* const extras = (const uint2*)p.extra_deps;
+    const uint32_t end_clip = RAGGED ? uniform(h.clip) : 0u;
+    unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
+    unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
+    const u64* const flags = p.sync_cur + uniform(h.flags);
+    const u64* const in_head = p.sync_cur + uniform(h.head_in);
+    u64* const in_tail = p.sync_cur + uniform(h.tail_out);
+    u64* const out_head = p.sync_cur + uniform(h.head_out);
+    const u64* const out_tail = p.sync_cur + uniform(h.tail_in);
+    u64* const my_flag = p.sync_cur + uniform(h.my_flag);
+    const uint32_t piece = p.piece_units, depth = (uint32_t)p.depth, nops = (uint32_t)uniform(h.nops), npasses = uniform(h.npasses);
+    const uint32_t in_slot_bytes = uniform(h.in_slot_bytes), in_wrap = uniform(h.in_wrap), out_slot_bytes = uniform(h.out_slot_bytes), out_wrap = uniform(h.out_wrap);
+    const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
+    uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
+    DevOp op = fetch_step(ops);
+    uint2 entry = {0u, 0u};  // this lane's folded dependency of the step `op`, if it has one
+    if (lane < (op.extra & 255u)) entry = extras[(op.extra >> 8) + lane];
+    for (;;) {
+      const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+      uint2 next_entry = {0u, 0u};
+      if (lane < (after.extra & 255u)) next_entry = extras[(after.extra >> 8) + lane];
+      const uint32_t t = op.word & 15u;
+      const uint32_t cnt = op.word >> kOpCntShift;
+      const uint32_t n = left < piece ? left : piece;
+      const uint32_t rcv_bit = (0x7cu >> t) & 1u, snd_bit = (0x5au >> t) & 1u;  // r rcs rrs rrc rrcs / s rcs rrs rrcs
+      static_assert(MSCCLX_OP_SEND == 1 && MSCCLX_OP_RECV == 2 && MSCCLX_OP_RCS == 3 && MSCCLX_OP_RRS == 4 && MSCCLX_OP_RRC == 5 && MSCCLX_OP_RRCS == 6,
+                    "the two masks above list the receiving and the sending step types by their codes");
+      {  // what this lane waits for: nothing, or one counter and the value it must reach
+        const uint32_t folded = op.extra & 255u;
+        const u64* mine = nullptr;
+        uint32_t target = 0;
+        if (lane < folded) {
+          mine = flags + entry.x;
+          target = pass * (entry.y >> 16) + (entry.y & 0xffffu);
+        } else if (lane == folded) {
+          if (op.dep_tb >= 0) { mine = flags + (uint32_t)op.dep_tb * kSyncStrideWords; target = pass * (uint32_t)op.dep_nops + (uint32_t)op.dep_step + 1; }
+        } else if (lane == folded + 1) {
+          if (rcv_bit && !(op.steps & kStepsNoAnnouncement)) { mine = in_head; target = rseq + 1; }
+        } else if (lane == folded + 2) {
+          if (snd_bit && sseq >= depth) { mine = out_tail; target = sseq + 1 - depth; }
+        }
+        unsigned spins = 0;
+        u64 since = 0;
+        for (;;) {
+          u64 seen = ~0ull;
+          if (mine) seen = load_counter(mine);
+          const u64 behind = __builtin_amdgcn_ballot_w64(seen < (u64)target);
+          if (!behind) break;
+          MSCCLX_POLL_PAUSE();
+          if ((++spins & 0x3fu) == 0) {
+            const uint32_t who = (uint32_t)__ffsll((long long)behind) - 1u;  // the first lane still waiting names what the report says
+            since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, (int)step, watch.slice, (u64)pass,
+                                                       who <= folded ? 0 : who == folded + 1 ? 1 : 2));
+            if (since == ~0ull) break;
+          }
+        }
+        if (since == ~0ull) break;  // the launch is lost
+      }
+      if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) break;  // a host's abort request
+      const bool out_staged = (op.word & kOpOutStaged) != 0;
+      if (!(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !out_staged))) {
+        // the step's operands, as the hosting loop's describe_step works them out, in scalar registers
+        Move m;
+        const u64 out = (snd_bit && out_staged) ? (u64)(out_ring + sslot) : 0;
+        u64 in = 0;
+        int in_packed = kAPacked;
+        if (rcv_bit) {
+          if (op.word & kOpInPlace) { in = op.in_addr + off; in_packed = 0; }
+          else in = (u64)(in_ring + rslot);
+        }
+        m.n = n; m.rows = (int)cnt;
+        m.a = in; m.dst = op.dst_addr + off; m.out = out;
+        const int nt = (op.word & kOpNtStore) ? kNt1 : 0;
+        int kind = 0;
+        switch (t) {
+          case MSCCLX_OP_SEND: m.a = op.src_addr + off; kind = (int)kToSlot; break;
+          case MSCCLX_OP_RECV: kind = in_packed | nt; break;
+          case MSCCLX_OP_RCS: kind = in_packed | (out ? (int)kHasO2 : 0); break;
+          case MSCCLX_OP_RRC: kind = in_packed | kHasB; break;
+          case MSCCLX_OP_RRS: kind = in_packed | kHasB | kToSlot; break;
+          case MSCCLX_OP_RRCS: kind = in_packed | kHasB | (out ? (int)kHasO2 : 0); break;
+          case MSCCLX_OP_COPY: m.a = op.src_addr + off; kind = nt; break;
+          case MSCCLX_OP_REDUCE:
+            m.a = op.src_addr + off;
+            kind = kHasB;
+            if (op.in_addr) { m.out = op.in_addr; kind = kMany | nt; }  // several sources, in_addr bytes apart
+            break;
+          default: break;
+        }
+        if constexpr (RAGGED) kind |= left <= piece ? (int)end_clip << kClipShift : 0;
+        m.kind = kind;
+        do_move<R, false, 1, RAGGED>(m, p, 0u, 0u, 0u, 0, 0, 0, 0u);
+        __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged: the counters below may announce them
+      }
+      if (snd_bit && writer) publish(out_head, (u64)sseq + 1);
+      if (rcv_bit && writer) publish(in_tail, (u64)rseq + 1);
+      rseq += rcv_bit;
+      rslot += in_slot_bytes & (0u - rcv_bit);
+      rslot = rslot == in_wrap ? 0u : rslot;
+      sseq += snd_bit;
+      sslot += out_slot_bytes & (0u - snd_bit);
+      sslot = sslot == out_wrap ? 0u : sslot;
+      count += op.steps & ~kStepsNoAnnouncement;  // = pass * steps of the IR + IR step + 1: a step may stand for folded ones too
+      if ((op.word & kOpHasdep) && writer) publish(my_flag, (u64)count);
+      if (++step == nops) {
+        step = 0;
+        left -= n;
+        off += (u64)piece * 16;
+        if (++pass >= npasses) break;
+      }
+      op = after;
+      entry = next_entry;
+    }
+  }
+  end_launch(p, launch_no);
+}
+
 // ------------------------------------------------------------------------------------------------
 // kernel table of one element type
 // ------------------------------------------------------------------------------------------------
@@ -1592,9 +1749,11 @@ typedef void (*kernel_fn)(const KernelParams);
 
 // ragged: chunks that are no multiple of 16 bytes -- rows may end inside a unit; the other kernels carry none of that
 // fold: 0 = no step stands for folded nops, 1 = some do, at most kLaneExtraDeps each, 2 = some for more (the check
-// of those costs scalar registers the other programs' poll loop has no room for: a kernel of its own)
+// of those costs scalar registers the other programs' poll loop has no room for: a kernel of its own), 3 = the loop for
+// such programs on one-wave workgroups with one context each (exec_kernel_chain_fold)
 template <int DT, int OP, bool RAGGED> kernel_fn pick_variant(bool ll, int fold) {
   if (ll) return !fold ? (kernel_fn)exec_kernel<Reducer<DT, OP>, true, 0, RAGGED> : nullptr;
+  if (fold == 3) return (kernel_fn)exec_kernel_chain_fold<Reducer<DT, OP>, RAGGED>;
   if (fold == 2) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 2, RAGGED>;
   if (fold) return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 1, RAGGED>;
   return (kernel_fn)exec_kernel<Reducer<DT, OP>, false, 0, RAGGED>;

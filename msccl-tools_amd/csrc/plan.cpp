@@ -462,6 +462,13 @@ bool has_foldable_nops(const mscclx_plan& plan) {
   return false;
 }
 
+bool one_wave_each(const Geometry& g) {
+  if (g.threads != 64 || g.wg_begin.size() != g.ctx_tb.size() + 1) return false;
+  for (size_t w = 0; w < g.wg_begin.size(); ++w)
+    if (g.wg_begin[w] != (int32_t)w) return false;
+  return true;
+}
+
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out) {
   const int elem = dtype_size(dtype);

@@ -74,7 +74,12 @@ constexpr int kOpCntShift = 8;
 // threadblock and waits for nothing, so the payload is what the sender's buffer holds when the launch starts --
 // there is no announcement to wait for.  (Every later writer of those chunks comes after this receive, or the
 // payload would not be read in place at all; and a step without predecessors lies on no path between two steps.)
-constexpr uint32_t kStepsPayloadAtLaunch = 1u << 31;
+constexpr uint32_t kStepsNoAnnouncement = 1u << 31;
+// The same bit, in programs that run on exec_kernel_chain_fold, on a receive that has TAKEN OVER the waits of its send: where
+// the matching step is an `s` whose payload is read in place, that step does nothing but wait for its dependencies
+// and announce -- a hand-off the receive can do without by waiting for those dependencies itself (they are counters of
+// another rank's threadblocks, in the same area) and for the sending threadblock's steps in front of the send.
+constexpr int kMaxChainFoldDeps = 61;     // counters a step of that kernel may wait for through its table: one per lane, three lanes kept for the step's own
 // A run of `re` steps with one chunk each, the same destination and sources a fixed distance apart is
 // done as one step on the device -- dst = (..((dst + src0) + src1)..) + src[m-1]: an `re` whose
 // in_addr holds the distance between sources in bytes (0 for an ordinary `re`) and whose cnt holds m.
@@ -242,6 +247,8 @@ int simulate(const mscclx_plan& plan, int depth);
 // A nop that nobody depends on and that is not its threadblock's last step can be folded into the
 // step after it when the device tables are built; programs with such nops run on kernels of their own.
 bool has_foldable_nops(const mscclx_plan& plan);
+// Does this geometry give every context a one-wave workgroup of its own (workgroup w hosts context w)?
+bool one_wave_each(const Geometry& g);
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,
                     int num_cus, const int capacity_by_threads[kThreadChoices], uint64_t fifo_budget_bytes, Geometry* out);
 void destroy_device_state(DeviceState* d);

@@ -21,12 +21,12 @@ def test_library_exports_every_declared_symbol(mscclx_lib):
     assert declared == set(EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(mscclx_lib, name), name
-    assert mscclx_lib.mscclx_version() == 3
+    assert mscclx_lib.mscclx_version() == 4
 
 
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(binding.Config) == 48
-    assert ctypes.sizeof(binding.Info) == 72
+    assert ctypes.sizeof(binding.Info) == 80
     assert ctypes.sizeof(binding.Status) == 32
 
 
