@@ -445,12 +445,16 @@ static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img,
   kp.timeout_ticks = (uint64_t)plan.timeout_ms * 100000ull;  // wall_clock64 ticks at 100 MHz
   kp.piece_units = g.piece_units;
   kp.slice_grain = g.slice_grain;
-  {  // groups of about sqrt(workgroups), at most kFinishGroups of them; up to 64 workgroups are one group
-    uint32_t per = 1;
-    while ((uint64_t)per * per < (uint64_t)g.workgroups) ++per;
-    per = std::max<uint32_t>(per, ((uint32_t)g.workgroups + kFinishGroups - 1) / kFinishGroups);
-    if (g.workgroups <= 64) per = (uint32_t)g.workgroups;
-    kp.finish_group = per;
+  {  // as many counters of finished workgroups as there are workgroups, up to kFinishCounters; a power of two
+    uint32_t counters = 1;
+    while (counters * 2 <= (uint32_t)kFinishCounters && counters * 2 <= (uint32_t)g.workgroups) counters *= 2;
+    auto magic = [](uint32_t divisor) -> uint64_t {
+      return divisor <= 1 ? 0ull : (uint64_t)((((unsigned __int128)1 << 64) + divisor - 1) / divisor);
+    };
+    kp.finish_counters = counters;
+    kp.finish_more = (uint32_t)g.workgroups % counters;
+    kp.finish_magic_each = magic((uint32_t)g.workgroups / counters);
+    kp.finish_magic_more = magic((uint32_t)g.workgroups / counters + 1);
   }
   kp.slices = g.slices; kp.depth = g.depth; kp.ntbs = (int)plan.tbs.size(); kp.nconns = (int)plan.conns.size();
   kp.wg_begin = (const int32_t*)(tables + img.off_hosting);

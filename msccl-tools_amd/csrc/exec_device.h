@@ -376,7 +376,7 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
 // rows x n units.  Consecutive rows of an operand are `stride_*` BYTES apart: a chunk for rank
 // buffers, n units for the packed rows of a FIFO slot.  b (the local reduction operand) is always a rank
 // buffer, o2 (the forwarded copy) always a FIFO slot.  clip: see move_units.
-template <class R, bool HAS_B, bool HAS_O2, bool NT1 = false>
+template <class R, bool HAS_B, bool HAS_O2, bool NT1 = false, int RB = 4>
 __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1, unsigned char* o2, const unsigned char* a, uint64_t stride_a,
                                           const unsigned char* b, uint64_t stride_b, int rows, uint32_t n, uint32_t clip) {
   constexpr int W = 16;
@@ -387,8 +387,7 @@ __device__ __forceinline__ void move_rows(unsigned char* o1, uint64_t stride_o1,
     typedef Access<W> A;
     typedef typename A::word word;
     constexpr int XL = MSCCLX_AUX_LD, XS = MSCCLX_AUX_ST, X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
-    constexpr int RB = 4;
-    const uint32_t i = threadIdx.x;
+    const uint32_t i = threadIdx.x;  // (RB rows at a time: four, or eight where the kernel has the registers for them)
     if (i >= n) return;
     const uint32_t bytes = n * W - clip;
     for (int r0 = 0; r0 < rows; r0 += RB) {
@@ -493,6 +492,14 @@ __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t ll_flag(uint32_t epoch, u64 seq) { return ((epoch & 0x3ffu) << 22) | (uint32_t)((seq + 1) & 0x3fffffu); }
 __device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { return l0.y == f && l0.w == f && l1.y == f && l1.w == f; }
+
+// The area's abort word is raised.  If it was the host that raised it (mscclx_plan_abort), whoever sees it says so in the
+// launch's status: a launch replayed from a HIP graph passes by the host code that would have re-armed the counters, and
+// the caller must still learn from the wait that follows that this launch did not run.  (Out of line: the rare path.)
+__device__ __noinline__ void note_abort(const u64* abort_word, mscclx_status* hs) {
+  if (load_counter(abort_word) == kAbortByHost && __hip_atomic_load(&hs->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
+    __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // What a thread needs to give up on a message that never arrives.
 struct LLWatch {
@@ -798,7 +805,7 @@ __device__ __forceinline__ void init_context(Hosted& h, Context& c, const Kernel
 
 // The whole workgroup (or wave) copies / reduces one piece as `m` says.  rseq, sseq: numbers of the
 // incoming / outgoing message (LL flags); tb, step, slice, pass: for the LL watchdog's report.
-template <class R, bool LL, int FOLD, bool RAGGED>
+template <class R, bool LL, int FOLD, bool RAGGED, int ROWS_AT_ONCE = 4>
 __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, uint32_t epoch, uint32_t rseq, uint32_t sseq,
                                         int tb, int step, int slice, unsigned pass) {
   constexpr int W = 16;
@@ -838,8 +845,8 @@ __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, ui
     unsigned char* const o1 = (m.kind & kToSlot) ? out : dst;
     const u64 stride_o1 = (m.kind & kToSlot) ? packed : cs;
     switch (m.kind & 7) {
-      case 0: move_rows<R, false, false>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
-      case kNt1: move_rows<R, false, false, true>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case 0: move_rows<R, false, false, false, ROWS_AT_ONCE>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
+      case kNt1: move_rows<R, false, false, true, ROWS_AT_ONCE>(o1, stride_o1, nullptr, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
       case kHasO2: move_rows<R, false, true>(o1, stride_o1, out, a, stride_a, nullptr, 0, m.rows, m.n, clip); break;
       case kHasB: move_rows<R, true, false>(o1, stride_o1, nullptr, a, stride_a, dst, cs, m.rows, m.n, clip); break;
       case kHasB | kHasO2: move_rows<R, true, true>(o1, stride_o1, out, a, stride_a, dst, cs, m.rows, m.n, clip); break;
@@ -852,7 +859,10 @@ __device__ __forceinline__ void do_move(const Move& m, const KernelParams& p, ui
 // the time the wait began (to be handed in again), or ~0 when the wait must be abandoned -- the
 // launch is lost, by this wait's own expiry (which it reports) or by somebody else's.
 __device__ __noinline__ u64 chain_slow_check(u64* abort_word, mscclx_status* hs, u64 timeout_ticks, u64 since, int tb, int step, int slice, u64 pass, int waiting_on) {
-  if (load_counter(abort_word) != 0) return ~0ull;
+  if (load_counter(abort_word) != 0) {
+    note_abort(abort_word, hs);
+    return ~0ull;
+  }
   const u64 now = wall_clock64();
   if (!since) return now;
   if (now - since > timeout_ticks) {
@@ -1075,7 +1085,10 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
         }
       }
     }
-    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) return;  // a host's abort request, a lost launch
+    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) {  // a host's abort request, a lost launch
+      note_abort(watch.abort_word, watch.host_status);
+      return;
+    }
     u64 prof_floor = 0;
 #ifdef MSCCLX_PROFILE
     prof_floor = __builtin_amdgcn_s_memtime();
@@ -1245,7 +1258,10 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
         }
       }
     }
-    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) return;  // a host's abort request, a lost launch
+    if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) {  // a host's abort request, a lost launch
+      note_abort(watch.abort_word, watch.host_status);
+      return;
+    }
     MSCCLX_CHAIN_CLOCK(prof_ready);
     MSCCLX_CHAIN_ADD(0, prof_top, prof_ready);
     const bool rcv = rcv_bit != 0;
@@ -1321,43 +1337,33 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
 #endif
 }
 
-// The start of a launch.  The number of launches so far is kept on the device (control word 0) and is advanced by the
-// last workgroup to finish, so a launch carries no host-side state and the same launch can be replayed (stream
-// order guarantees the next launch sees the new value).  Its lowest bit picks which of the two counter areas this
-// launch uses; its low 10 bits mark the LL lines.  Returns that number.
+// The start of a launch.  The number of launches so far is kept on the device, so a launch carries no host-side state
+// and the same launch can be replayed: the control block holds up to kFinishCounters counters of finished workgroups,
+// workgroup w counting itself in counter w mod `finish_counters` when it ends.  Such a counter grows by a known number
+// per launch (the workgroups of its class), and a workgroup that reads its own class's counter when it starts finds
+// (launches so far) x (that number) + (workgroups of its class that have already ended in this launch) -- fewer than
+// the class has, the reader being one of them -- so the quotient is the launch's number however late the workgroup
+// starts, and however early others have ended.  (Stream order guarantees that every workgroup of the launches before has counted itself.)  The number's lowest
+// bit picks which of the two counter areas this launch uses; its low 10 bits mark the LL lines.  Returns that number.
 __device__ __forceinline__ u64 begin_launch(KernelParams& p) {
-  const u64 launch_no = load_counter(p.sync_base);
+  const uint32_t k = blockIdx.x & (p.finish_counters - 1u);
+  const u64 ended = load_counter(p.sync_base + 8 + (uint64_t)k * kFinishStrideWords);
+  // ended / (workgroups of my class), as a multiplication by ceil(2^64 / divisor), worked out on the host: exact for
+  // dividends below 2^57 and divisors up to 128 (0 stands for a divisor of 1)
+  const u64 magic = k < p.finish_more ? p.finish_magic_more : p.finish_magic_each;
+  const u64 launch_no = magic ? __umul64hi(ended, magic) : ended;  // (left in vector registers: the counter areas' addresses made from it cost scalar registers the step loops need)
   const u64 parity = launch_no & 1ull;
   p.sync_cur = p.sync_base + kControlWords + parity * p.sync_words;
   p.sync_nxt = p.sync_base + kControlWords + (parity ^ 1ull) * p.sync_words;
   return launch_no;
 }
 
-// The end of a workgroup.  The last workgroup out re-arms the control block: the next launch uses the other counter
-// area.  "Last" is found group by group (the last of a group reports for the group), so that no address sees more
-// than a few dozen atomics.
-__device__ __forceinline__ void end_launch(const KernelParams& p, const u64 launch_no) {
-  if (threadIdx.x == 0) {
-    const unsigned per = p.finish_group, group = blockIdx.x / per, groups = (gridDim.x + per - 1) / per;
-    const unsigned members = group + 1 < groups ? per : gridDim.x - group * per;
-    u64* const group_count = p.sync_base + 8 + (uint64_t)group * kFinishStrideWords;
-    if (__hip_atomic_fetch_add(group_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)members - 1) {
-      publish(group_count, 0);
-      bool last = groups == 1;  // (a small grid is one group: its last workgroup is the launch's last, without a second round trip)
-      if (!last && __hip_atomic_fetch_add(p.sync_base + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (u64)groups - 1) {
-        publish(p.sync_base + 1, 0);
-        last = true;
-      }
-      if (last) {
-        // A launch that ran under a host's abort request says so itself: whoever replays it from a HIP graph passes
-        // by the host code that would have re-armed the counters, and must still learn that it did not run.
-        if (load_counter(p.sync_cur) == kAbortByHost &&
-            __hip_atomic_load(&p.host_status->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
-          __hip_atomic_store(&p.host_status->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-        publish(p.sync_base, launch_no + 1);
-      }
-    }
-  }
+// The end of a workgroup: it counts itself, and does not wait for the answer -- the last workgroup to finish its work
+// used to find out that it was the last with one or two atomics that return, a microsecond at the end of every launch.
+__device__ __forceinline__ void end_launch(const KernelParams& p) {
+  if (threadIdx.x == 0)
+    (void)__hip_atomic_fetch_add(p.sync_base + 8 + (uint64_t)(blockIdx.x & (p.finish_counters - 1u)) * kFinishStrideWords, 1ull, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // A workgroup hosts up to 64 contexts, one per lane of wave 0.  Wave 0 polls the counters every
@@ -1369,10 +1375,6 @@ __device__ __forceinline__ void end_launch(const KernelParams& p, const u64 laun
 // programs without such steps do not pay for the check in the poll loop).
 template <class R, bool LL, int FOLD, bool RAGGED>
 __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) exec_kernel(const KernelParams launch_params) {
-  // The number of launches so far is kept on the device (control word 0) and is advanced by the
-  // last workgroup to finish, so a launch carries no host-side state and the same launch can be
-  // replayed (stream order guarantees the next launch sees the new value).  Its lowest bit picks
-  // which of the two counter areas this launch uses; its low 10 bits mark the LL lines.
   KernelParams p = launch_params;
   const u64 launch_no = begin_launch(p);
   const uint32_t epoch = (uint32_t)launch_no & 0x3ffu;
@@ -1475,7 +1477,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
           if (__builtin_expect((++busy_rounds & 0x3fu) == 0, 0)) {
             bool stop = false;
             if (lane == 0) stop = load_counter(abort_word) != 0;
-            if (__any(stop)) choice = -3;
+            if (__any(stop)) { if (lane == 0) note_abort(abort_word, p.host_status); choice = -3; }
           }
         } else if (!__any(c.active)) {
           choice = -1;  // every hosted context has run to its end
@@ -1488,7 +1490,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
             if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
             bool stop = false;
             if (lane == 0) stop = load_counter(abort_word) != 0;
-            if (__any(stop)) { choice = -3; }
+            if (__any(stop)) { if (lane == 0) note_abort(abort_word, p.host_status); choice = -3; }
             else if (now > deadline) {
               // report the first context that is still waiting
               const u64 stuck = __ballot(c.active);
@@ -1580,7 +1582,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 #endif
   }
   }  // hosted contexts
-  end_launch(p, launch_no);
+  end_launch(p);
 #ifdef MSCCLX_PROFILE
   if (threadIdx.x == 0 && p.prof) {
     p.prof[(size_t)blockIdx.x * kProfWords + 0] = prof_wait;
@@ -1608,7 +1610,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 template <class R, bool RAGGED>
 __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams launch_params) {
   KernelParams p = launch_params;
-  const u64 launch_no = begin_launch(p);
+  (void)begin_launch(p);
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
   if (writer && blockIdx.x == 0) p.sync_nxt[0] = 0;
@@ -1683,7 +1685,10 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
         }
         if (since == ~0ull) break;  // the launch is lost
       }
-      if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) break;  // a host's abort request
+      if (__builtin_expect((count & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) {  // a host's abort request
+        note_abort(watch.abort_word, watch.host_status);
+        break;
+      }
       const bool out_staged = (op.word & kOpOutStaged) != 0;
       if (!(t == MSCCLX_OP_NOP || (t == MSCCLX_OP_SEND && !out_staged))) {
         // the step's operands, as the hosting loop's describe_step works them out, in scalar registers
@@ -1716,7 +1721,7 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
         }
         if constexpr (RAGGED) kind |= left <= piece ? (int)end_clip << kClipShift : 0;
         m.kind = kind;
-        do_move<R, false, 1, RAGGED>(m, p, 0u, 0u, 0u, 0, 0, 0, 0u);
+        do_move<R, false, 1, RAGGED, 8>(m, p, 0u, 0u, 0u, 0, 0, 0, 0u);  // (short rows of a multi-chunk step go eight at a time here)
         __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged: the counters below may announce them
       }
       if (snd_bit && writer) publish(out_head, (u64)sseq + 1);
@@ -1739,7 +1744,7 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
       entry = next_entry;
     }
   }
-  end_launch(p, launch_no);
+  end_launch(p);
 }
 
 // ------------------------------------------------------------------------------------------------

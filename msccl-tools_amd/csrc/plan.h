@@ -158,7 +158,7 @@ struct KernelParams {
   const DevOp* ops;
   const DevConn* conns;
   const uint32_t* extra_deps;   // kExtraDepWords words per folded dependency
-  unsigned long long* sync_base; // control block (kControlWords): word 0 = launches finished so far (its parity picks the counter area)
+  unsigned long long* sync_base; // control block (kControlWords): counters of finished workgroups, from which a launch works out its number
   unsigned long long* sync_cur;  // this launch's counters   } both derived inside the kernel
   unsigned long long* sync_nxt;  // next launch's counters   } from the control block
   unsigned char* fifo;
@@ -172,7 +172,10 @@ struct KernelParams {
   uint64_t timeout_ticks;
   uint32_t piece_units;
   uint32_t slice_grain;
-  uint32_t finish_group;        // workgroups per group of the end-of-launch count
+  uint32_t finish_counters;     // counters of finished workgroups in use: a power of two, at most kFinishCounters; workgroup w counts in w mod that
+  uint32_t finish_more;         // the first so many counters count one workgroup more than the others
+  uint64_t finish_magic_each;   // ceil(2^64 / workgroups per counter), 0 if that is 1: a division as a multiplication ...
+  uint64_t finish_magic_more;   // ... the same for the counters that count one more
   int32_t slices, depth, ntbs, nconns;
   const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
   const DevCtx* ctxs;           // hosted contexts, grouped by workgroup
@@ -198,19 +201,16 @@ constexpr int kProfWords = 8 + kProfTrace;  // ... after its 8 words of totals
 constexpr int kLLUnitBytes = 32;       // a flag-in-data line pair: 16 bytes of payload in 32
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
-// The control block in front of the two counter areas: word 0 = launches finished so far, word 1 =
-// groups of workgroups finished, then one counter per group of workgroups (each alone in 128 bytes).
-// Workgroups report the end of a launch group by group: one counter for all of them would put one
-// returning atomic per workgroup on a single address at the end of every launch (measured 10 ns
-// each: 5 us of a 512-workgroup launch).
-constexpr int kStampWord = 2;  // control word 2: which plan's binding armed this workspace (see mscclx_plan_bind)
+// The control block in front of the two counter areas: word 2 = the stamp of the binding that armed the workspace, then
+// from word 8 the counters of finished workgroups, each alone in 128 bytes (exec_device.h: begin_launch).
+constexpr int kStampWord = 2;
 // Values of an area's abort word: raised by a workgroup whose watchdog expired (which then reports the step it
-// waited for), or by mscclx_plan_abort from the host (reported by the launch's last workgroup, so that a launch
+// waited for), or by mscclx_plan_abort from the host (reported by the workgroups that leave on seeing it, so that a launch
 // replayed from a HIP graph onto a raised word still tells the host that it did not run).
 constexpr unsigned long long kAbortByWatchdog = 1, kAbortByHost = 2;
-constexpr int kFinishGroups = 64;
+constexpr int kFinishCounters = 64;
 constexpr int kFinishStrideWords = 16;
-constexpr int kControlWords = 8 + kFinishGroups * kFinishStrideWords;
+constexpr int kControlWords = 8 + kFinishCounters * kFinishStrideWords;
 
 struct DeviceState;  // defined in exec.hip (host half of the ABI)
 
