@@ -140,7 +140,7 @@ typedef struct {
   int32_t waiting_ratio_x100; /* 100 * threadblocks * depth of the dataflow / moving steps: 100 = every threadblock always has work (a ring) */
   int32_t dataflow_depth;     /* moving steps on the longest chain through step order, dependencies and messages */
   int32_t kernel_loop; /* mscclx_loop: which of the kernels' step loops this geometry runs */
-  int32_t reserved;
+  int32_t cold_traffic_x100; /* 100 * share of the algorithmic bytes that memory sees once only: inputs read, results written */
   uint64_t workspace_bytes;
   uint64_t algorithmic_units; /* sum over ops of cnt * a(type); times chunk_bytes = algorithmic bytes */
 } mscclx_info;

@@ -582,7 +582,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     info->dataflow_depth = g.dataflow_depth;
     info->kernel_loop = !one_wave_each(g) ? MSCCLX_LOOP_HOSTED : g.ll ? MSCCLX_LOOP_CHAIN_LINES
                         : has_foldable_nops(*plan) ? MSCCLX_LOOP_CHAIN_FOLD : MSCCLX_LOOP_CHAIN_COUNTERS;
-    info->reserved = 0;
+    info->cold_traffic_x100 = (int32_t)(g.cold_fraction * 100.0 + 0.5);
     info->threads = g.threads;
     info->slices = g.slices;
     info->piece_bytes = (int32_t)(g.piece_units * g.unit_bytes);

@@ -496,10 +496,13 @@ __device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { retur
 // The area's abort word is raised.  If it was the host that raised it (mscclx_plan_abort), whoever sees it says so in the
 // launch's status: a launch replayed from a HIP graph passes by the host code that would have re-armed the counters, and
 // the caller must still learn from the wait that follows that this launch did not run.  (Out of line: the rare path.)
-__device__ __noinline__ void note_abort(const u64* abort_word, mscclx_status* hs) {
+__device__ __forceinline__ void note_abort_here(const u64* abort_word, mscclx_status* hs) {
   if (load_counter(abort_word) == kAbortByHost && __hip_atomic_load(&hs->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == (int)MSCCLX_OK)
     __hip_atomic_store(&hs->code, (int)MSCCLX_ERR_ABORTED, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
+// (out of line for the chain loops, which call their slow checks anyway; in line for the hosting loop, which calls nothing:
+// a single call would cost that whole kernel the registers a callee may clobber)
+__device__ __noinline__ void note_abort(const u64* abort_word, mscclx_status* hs) { note_abort_here(abort_word, hs); }
 
 // What a thread needs to give up on a message that never arrives.
 struct LLWatch {
@@ -1477,7 +1480,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
           if (__builtin_expect((++busy_rounds & 0x3fu) == 0, 0)) {
             bool stop = false;
             if (lane == 0) stop = load_counter(abort_word) != 0;
-            if (__any(stop)) { if (lane == 0) note_abort(abort_word, p.host_status); choice = -3; }
+            if (__any(stop)) { if (lane == 0) note_abort_here(abort_word, p.host_status); choice = -3; }
           }
         } else if (!__any(c.active)) {
           choice = -1;  // every hosted context has run to its end
@@ -1490,7 +1493,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
             if (!armed) { deadline = now + p.timeout_ticks; armed = true; }
             bool stop = false;
             if (lane == 0) stop = load_counter(abort_word) != 0;
-            if (__any(stop)) { if (lane == 0) note_abort(abort_word, p.host_status); choice = -3; }
+            if (__any(stop)) { if (lane == 0) note_abort_here(abort_word, p.host_status); choice = -3; }
             else if (now > deadline) {
               // report the first context that is still waiting
               const u64 stuck = __ballot(c.active);

@@ -380,6 +380,7 @@ static uint64_t tb_work(const mscclx_plan& plan, const Tb& tb, bool staging) {
   return w;
 }
 
+constexpr uint64_t kWidePieceBytes = 96 * 1024;  // pieces from which a workgroup of 1024 threads pays, for the programs it pays for at all
 // threads: enough to cover a piece with a few 16-byte loads per thread
 static int threads_for_piece(uint64_t piece_bytes) {
   return piece_bytes >= 48 * 1024 ? 512 : piece_bytes >= 24 * 1024 ? 256 : piece_bytes >= 12 * 1024 ? 128 : 64;
@@ -455,6 +456,59 @@ static double hosting_balance(const std::vector<uint64_t>& tb_works, int64_t sli
   return largest ? (double)total / (double)wgs / (double)largest : 1.0;
 }
 
+// The share of a program's algorithmic bytes that memory sees once only: reads of chunks no step of the program writes
+// (the collective's inputs) and writes of chunks no step reads again (its results).  Everything else is written by one step
+// and read by another soon after, out of the memory-side cache.  A ring re-reads nearly all it writes (all-gather ring of 8
+// ranks: 0.25); an all-to-all reads its input cold and writes its output for good (one-step: 1.0; hierarchical, a third of
+// whose bytes pass through scratch: 0.67); the all-pairs programs lie between.
+double cold_fraction(const mscclx_plan& plan) {
+  typedef std::pair<int, int> Span;  // [lo, hi) in chunks
+  std::vector<std::vector<Span>> written((size_t)plan.nranks * 3);
+  for (const Tb& tb : plan.tbs)
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      const Op& op = plan.ops[o];
+      if (touches_local_dst(op.type) && op.type != MSCCLX_OP_RRS) written[(size_t)tb.rank * 3 + op.dstbuf].push_back({op.dstoff, op.dstoff + op.cnt});
+    }
+  for (auto& v : written) {
+    std::sort(v.begin(), v.end());
+    size_t k = 0;
+    for (const Span& sp : v) {
+      if (k && sp.first <= v[k - 1].second) v[k - 1].second = std::max(v[k - 1].second, sp.second);
+      else v[k++] = sp;
+    }
+    v.resize(k);
+  }
+  auto never_written = [&](int rank, int buf, int lo, int cnt) {  // chunks of [lo, lo + cnt) outside every written span
+    if (buf < 0 || buf > 2) return 0;
+    int covered = 0;
+    for (const Span& sp : written[(size_t)rank * 3 + buf]) covered += std::max(0, std::min(sp.second, lo + cnt) - std::max(sp.first, lo));
+    return cnt - covered;
+  };
+  uint64_t total = 0, cold = 0;
+  for (const Tb& tb : plan.tbs)
+    for (int o = tb.op_begin; o < tb.op_end; ++o) {
+      const Op& op = plan.ops[o];
+      if (op.cnt <= 0) continue;
+      if (op.type == MSCCLX_OP_COPY || op.type == MSCCLX_OP_REDUCE) {  // the local source
+        total += op.cnt;
+        cold += never_written(tb.rank, op.srcbuf, op.srcoff, op.cnt);
+      }
+      if (is_recv_type(op.type) && op.match_send >= 0) {              // the payload, where the sender had it
+        const Op& sender = plan.ops[op.match_send];
+        const int sender_rank = plan.tbs[plan.conns[tb.recv_conn].send_tb].rank;
+        total += op.cnt;
+        if (sender.type == MSCCLX_OP_SEND) cold += never_written(sender_rank, sender.srcbuf, sender.srcoff, op.cnt);
+      }
+      if (is_reduce_type(op.type)) total += op.cnt;                     // the local operand: written by this very step, at the least
+      if (touches_local_dst(op.type) && op.type != MSCCLX_OP_RRS) {     // the local destination
+        total += op.cnt;
+        if (op.final_write) cold += op.cnt;
+      }
+      if (op.type == MSCCLX_OP_RRS) total += op.cnt;                    // its result, handed on
+    }
+  return total ? (double)cold / (double)total : 0.0;
+}
+
 bool has_foldable_nops(const mscclx_plan& plan) {
   for (const Tb& tb : plan.tbs)
     for (int o = tb.op_begin; o + 1 < tb.op_end; ++o)
@@ -501,6 +555,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   }
   g.depth = depth;
   g.waiting_ratio = waiting_ratio(plan, &g.dataflow_depth);
+  g.cold_fraction = cold_fraction(plan);
 
   // Slices are independent copies of the program on 1/slices of every chunk; they are what keeps
   // the chip busy while one copy waits on its dependency chain.
@@ -510,6 +565,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     return fail(MSCCLX_ERR_CAPACITY, std::to_string(ntbs) + " threadblocks but the device can host only " + std::to_string(host_limit) + " contexts");
   int64_t slices = cfg.slices;
   bool lines = cfg.protocol == MSCCLX_PROTO_LL;  // flag-in-data lines instead of counters
+  bool wide = false;                             // one workgroup of 1024 threads per compute unit, pieces of 128 KiB
   if (!slices) {
     const int64_t finest = (int64_t)(chunk_bytes / (32 * 1024));       // most slices of at least 32 KiB
     const int64_t to_fill = ((int64_t)2 * num_cus + ntbs - 1) / ntbs;  // fewest slices that give every compute unit a context or two
@@ -540,6 +596,16 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // pieces of 16 KiB only where 32 KiB pieces leave less than a quarter of the contexts wanted in (2)
       const int64_t finer = (double)(finest * ntbs) / (2.0 * num_cus) < wanted_per_wg / 4 ? (int64_t)(chunk_bytes / (16 * 1024)) : finest;
       const int64_t hi = std::max<int64_t>(lo, std::min<int64_t>(finer, ((int64_t)most_capacity * kMaxHosted) / ntbs));
+      // Programs whose traffic is mostly cold -- inputs read once, results written once, little re-read out of the
+      // memory-side cache: the all-to-alls -- and whose threadblocks wait for each other part of the time do better with
+      // one workgroup of 1024 threads per compute unit walking pieces of 128 KiB: nothing to share the compute unit with
+      // (two workgroups of 512 threads do not share it evenly: the earlier one runs 2.4 times faster and then polls), and
+      // half the hand-offs per byte.  Hierarchical all-to-all, 16 ranks, chunks of 2 / 4 / 8 / 32 MiB: 278 -> 253,
+      // 510 -> 485, 998 -> 943, 4421 -> 4004 us; with pieces of 64 KiB or less the wide workgroups lose (1 MiB chunks
+      // 134 -> 135 us, 512 KiB 76 -> 82 us), and so do rings, which re-read what they have just written.  More than
+      // eight passes over a slice cost such a program too (32 MiB chunks: 16 slices x 16 passes 4168 us, 32 x 8 4004 us).
+      wide = !cfg.threads && !cfg.piece_bytes && !cfg.workgroups && g.cold_fraction >= 0.6 && g.waiting_ratio >= 1.5 &&
+             capacity_by_threads[thread_index(1024)] >= num_cus;
       std::vector<int64_t> candidates = {lo, hi};
       for (int64_t base = 1; base <= hi; base *= 2)
         for (int64_t c : {base, base * 3})
@@ -558,7 +624,11 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
         // of them to a compute unit, and contexts per workgroup would not tell candidates apart.  The
         // unit is half a compute unit -- one workgroup of 512 threads.
         const double per_wg = std::max(1.0, (double)(c * ntbs) / (2.0 * num_cus));
-        const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / wanted_per_wg));
+        // (the slices of a wide program are scored as everybody's -- on the workgroups they would get with pieces of
+        // 64 KiB -- plus its passes of 128 KiB beyond eight; pieces and threads follow from the slices below)
+        const double wide_passes = std::ceil((double)slice_bytes / (128.0 * 1024.0));
+        const double score = hosting_balance(works, c, wgs) - 0.02 * std::fabs(std::log2(per_wg / wanted_per_wg)) -
+                             (wide && wide_passes > 8.0 ? 0.03 * std::log2(wide_passes / 8.0) : 0.0);
         if (score > best_score + 1e-9 || (std::fabs(score - best_score) <= 1e-9 && c < slices)) { best_score = score; slices = c; }
       }
       if (!slices) slices = lo;
@@ -661,6 +731,35 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       }
     }
   }
+  // A workgroup of one wave for every context -- the shape the kernels' chain loops are written for -- is worth more than
+  // the slices chosen above where pieces of at most 8 KiB (one wave's worth) can be had that way: a context that is hosted
+  // with others pays the hosting loop's hand-off (2 us against 1.4 to 1.7), one that has a workgroup of several waves pays
+  // its barrier.  Where more contexts were asked for than there are workgroups to give them one each, take the most
+  // slices that still do (two-level all-reduce of 32 ranks at 1 MiB per rank: 72 -> 66 us); where fewer were asked for,
+  // cut on down to 8 KiB (hierarchical all-to-all of 16 ranks at 1 / 2 MiB per rank: 21 -> 17, 29 -> 27 us; all-pairs
+  // all-gather at 128 / 256 KiB chunks 10.6 -> 8.6, 11.6 -> 9.6 us; over the programs msccl-tools ships at 64 KiB to 1 MiB
+  // chunks it changed 38 cases, 34 of them for the better by 2 to 19 %, all-to-next at 256 KiB chunks for the worse
+  // by 5 and 15 %).  Only where the launch is mostly hand-offs -- its bytes at 5 TB/s take at most six times its chain
+  // at 2 us a hop -- and not for the longest chains (64-rank ring, 126 hops, 128 KiB chunks: 485 -> 520 us).  Pieces of
+  // 16 KiB on one wave lose as often as they win (PCIe-hierarchical all-reduce at 256 KiB chunks 123 -> 140 us, chain
+  // all-reduce of 64 ranks 284 -> 375 us): those keep two waves, or their hosted contexts.
+  if (!cfg.slices && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups && !lines && slices >= 1) {
+    uint64_t moved = 0;  // in chunks
+    for (const Tb& tb : plan.tbs) moved += tb_work(plan, tb, cfg.staging != 0);
+    const double data_us = (double)moved * (double)chunk_bytes / 5e6, chain_us = 2.0 * (double)g.dataflow_depth;  // the bytes at 5 TB/s, 2 us a hop
+    const int64_t one_each = std::min<int64_t>(capacity_by_threads[thread_index(64)], (int64_t)num_cus * 16) / ntbs;  // most slices with a workgroup each
+    if (one_each >= 1) {
+      int64_t s = 1;
+      while (s * 2 <= one_each) s *= 2;
+      if (slices > s) {
+        if (chunk_bytes / (uint64_t)s <= 8 * 1024) slices = s;
+      } else if (g.dataflow_depth <= 32 && data_us <= 6.0 * chain_us) {  // (a launch that is mostly hand-offs, not mostly bytes)
+        int64_t finer = slices;
+        while (finer * 2 <= s && chunk_bytes / (uint64_t)finer > 8 * 1024) finer *= 2;
+        if (chunk_bytes / (uint64_t)finer <= 8 * 1024) slices = finer;
+      }
+    }
+  }
   slices = std::min<int64_t>(slices, (int64_t)g.chunk_units);
   if (slices < 1 || (cfg.slices && (uint64_t)cfg.slices > g.chunk_units)) return fail(MSCCLX_ERR_INVALID_ARG, "more slices than units in a chunk");
   if (slices * ntbs > host_limit) {
@@ -694,7 +793,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
   const uint64_t slack = 2048 / g.unit_bytes;
   if (!cfg.piece_bytes && longest_slice * g.unit_bytes > 128 * 1024 + 2048) {
     // equal passes of about 64 KiB (a short last pass costs as many hand-offs as a full one), on 256-byte boundaries
-    const uint64_t target = (uint64_t)(64 * 1024) / g.unit_bytes;
+    const uint64_t target = (uint64_t)(wide ? 128 * 1024 : 64 * 1024) / g.unit_bytes;
     const uint64_t passes = (longest_slice - slack + target - 1) / target;
     piece_units = (longest_slice + passes - 1) / passes;
     piece_units = (piece_units + g.slice_grain - 1) / g.slice_grain * g.slice_grain;
@@ -741,7 +840,7 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
     if (thread_index(threads) < 0) return fail(MSCCLX_ERR_INVALID_ARG, "threads must be 64, 128, 256, 512 or 1024");
   } else {
     const uint64_t piece_bytes = piece_units * g.unit_bytes;
-    threads = threads_for_piece(piece_bytes);
+    threads = wide && piece_bytes >= kWidePieceBytes ? 1024 : threads_for_piece(piece_bytes);
     while (threads > 64 && capacity_by_threads[thread_index(threads)] < 1) threads /= 2;
   }
   const int capacity = capacity_by_threads[thread_index(threads)];

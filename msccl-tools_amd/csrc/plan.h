@@ -145,6 +145,7 @@ struct Geometry {
   std::vector<int32_t> wg_begin, ctx_tb, ctx_slice;  // the hosting table
   int32_t passes = 0;
   double waiting_ratio = 1.0;     // threadblocks x depth of the dataflow / moving steps
+  double cold_fraction = 0.0;     // share of the algorithmic bytes that memory sees once only
   int32_t dataflow_depth = 1;
   uint64_t slice_fifo_units = 0;  // FIFO units one slice needs (all connections)
   uint64_t sync_words = 0;        // uint64 words of ONE synchronisation area (there are two)
@@ -247,6 +248,8 @@ int simulate(const mscclx_plan& plan, int depth);
 // A nop that nobody depends on and that is not its threadblock's last step can be folded into the
 // step after it when the device tables are built; programs with such nops run on kernels of their own.
 bool has_foldable_nops(const mscclx_plan& plan);
+// Share of the program's algorithmic bytes that are read or written once only (inputs read, results written).
+double cold_fraction(const mscclx_plan& plan);
 // Does this geometry give every context a one-wave workgroup of its own (workgroup w hosts context w)?
 bool one_wave_each(const Geometry& g);
 int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscclx_config& cfg,

@@ -67,7 +67,7 @@ class Info(ctypes.Structure):
                 ("zero_copy_messages", ctypes.c_int32), ("staged_messages", ctypes.c_int32),
                 ("max_hosted", ctypes.c_int32), ("protocol", ctypes.c_int32),
                 ("waiting_ratio_x100", ctypes.c_int32), ("dataflow_depth", ctypes.c_int32),
-                ("kernel_loop", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("kernel_loop", ctypes.c_int32), ("cold_traffic_x100", ctypes.c_int32),
                 ("workspace_bytes", ctypes.c_uint64), ("algorithmic_units", ctypes.c_uint64)]
 
     def as_dict(self):

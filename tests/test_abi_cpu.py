@@ -242,7 +242,7 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
     want = {
         "c1": (1024, 64, 128, 1024, 1, 1),      # latency bound: one workgroup of one wave per SIMD, one 16-byte unit per lane
         "c2": (512, 512, 64, 131072, 1, 4),     # a ring is always busy: 4 contexts per workgroup, one pass
-        "c3": (512, 512, 16, 65536, 4, 8),      # phases: 8 contexts per workgroup, 4 passes of 64 KiB
+        "c3": (256, 1024, 16, 131072, 2, 16),   # two thirds of its bytes are cold and its threadblocks wait half the time: a workgroup of 1024 threads per CU, 2 passes of 128 KiB
         "c4": (512, 512, 8, 65536, 4, 30),      # threadblocks mostly wait for each other: 30 per workgroup
         "c5": (512, 64, 8, 512, 1, 1),          # 126 hops: the smallest pieces allowed, flag-in-data lines
         "c5_chain": (4096, 64, 64, 4096, 1, 1),  # one buffer through 64 ranks: latency bound however big the chunk, one rank busy at a time: lines
@@ -251,6 +251,25 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
         assert i.protocol == binding.PROTOCOL_CODES["ll" if key in ("c5", "c5_chain") else "simple"], key
+
+
+def test_wide_workgroups_for_cold_traffic(mscclx_lib):
+    """Programs whose bytes are mostly read once and written once (the share is reported) and whose threadblocks wait part of
+    the time get one workgroup of 1024 threads per compute unit and pieces of 128 KiB, from slices of 96 KiB on, and at most
+    eight passes where more slices can be had; rings and all-reduces never do.  (workgroups, threads, slices, piece bytes, passes)"""
+    from msccl.executor.workloads import WORKLOADS
+    c3 = parse_algo_xml(WORKLOADS["c3"].build())
+    want = {1 << 20: (512, 512, 16, 65536, 1), 2 << 20: (256, 1024, 16, 131072, 1), 8 << 20: (256, 1024, 16, 131072, 4), 32 << 20: (256, 1024, 32, 131072, 8)}
+    for chunk_bytes, expect in want.items():
+        i = Plan(c3).configure(chunk_bytes, "uint8", max_workgroups=4096)
+        assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes) == expect, (chunk_bytes, (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes))
+        assert i.cold_traffic_x100 == 67 and 150 <= i.waiting_ratio_x100 <= 250
+    for key, cold in (("c2", 14), ("c4", 0), ("c1", 0)):
+        w = WORKLOADS[key].scaled(256 << 20)
+        i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
+        assert i.cold_traffic_x100 == cold and i.threads == 512 and i.piece_bytes <= 131072, (key, i.cold_traffic_x100, i.threads, i.piece_bytes)
+    i = Plan(parse_algo_xml(golden_util.load("allgather_allpairs_8r"))).configure(16 << 20, "int32", max_workgroups=4096)
+    assert i.cold_traffic_x100 == 100 and i.waiting_ratio_x100 == 100 and i.threads == 512     # all cold, but always busy: as before
 
 
 def test_geometry_between_the_benchmark_sizes(mscclx_lib):
@@ -262,16 +281,19 @@ def test_geometry_between_the_benchmark_sizes(mscclx_lib):
         ("c1", 16 << 10): (64, 8, 256),
         # threadblocks that mostly wait: more slices than the plain latency model gives, pieces of 4 KiB or more
         ("c4", 512 << 10): (64, 2, 4096),
-        ("c4", 1 << 20): (64, 4, 4096),
-        ("c3", 512 << 10): (128, 2, 16384),
+        # ... but a workgroup of one wave for every context where pieces of at most 8 KiB can be had that way
+        ("c4", 1 << 20): (64, 2, 8192),
+        ("c3", 512 << 10): (64, 4, 8192),
+        ("c3", 1 << 20): (64, 8, 8192),
+        ("c3", 2 << 20): (64, 16, 8192),
+        ("c1", 16 << 20): (64, 256, 8192),
         # between latency and bandwidth: contexts are counted per compute unit, whatever the workgroup size
-        ("c3", 1 << 20): (128, 4, 16384),
         ("c3", 4 << 20): (256, 8, 32768),
         ("c4", 4 << 20): (128, 4, 16384),
         ("c4", 8 << 20): (256, 4, 32768),
         # rings keep the largest pieces that still fill the chip
         ("c2", 4 << 20): (256, 32, 32768),
-        ("c1", 16 << 20): (256, 64, 32768),
+        ("c1", 32 << 20): (256, 128, 32768),
     }
     for (key, nbytes), expect in want.items():
         w = WORKLOADS[key].scaled(nbytes)
@@ -289,7 +311,7 @@ def test_small_chunks_are_cut_one_unit_per_lane(mscclx_lib):
         ("pipeline_a100_allpairs_8r", 16 << 10): (2176, 64, 16, 1024, 1),
         ("allreduce_1step_4r", 64 << 10): (1024, 64, 64, 1024, 1),
         ("allreduce_allpairs_8r_2inst", 16 << 10): (2048, 64, 16, 1024, 1),            # some threadblocks wait: up to two busy contexts per SIMD
-        ("allreduce_allpairs_8r_2inst", 64 << 10): (512, 128, 4, 16384, 1),            # 8192 or 4096 contexts would be more: the latency model's 4
+        ("allreduce_allpairs_8r_2inst", 64 << 10): (1024, 64, 8, 8192, 1),             # 8192 or 4096 contexts would be more: the latency model's 4, cut on down to 8 KiB, a wave each
         ("allreduce_a100_allpairs_8r", 20000): (1536, 64, 24, 928, 1),                  # 1250 units: 24 slices, a multiple of 8, not 32
         ("c5_allreduce_ring_64r_1ch_1inst", 16 << 10): (1024, 64, 16, 1024, 1),        # every threadblock busy: one context per SIMD ...
         ("c5_allreduce_ring_64r_1ch_1inst", 64 << 10): (512, 64, 8, 8192, 1),          # ... and no more

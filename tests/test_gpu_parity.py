@@ -743,6 +743,54 @@ def test_ll_launch_number_wraps(knobs):
     ex.wait()
 
 
+def test_which_step_loop_runs():
+    """mscclx_info.kernel_loop: the all-pairs family on small messages -- programs with folded nops, one-wave workgroups, one
+    context each -- runs on exec_kernel_chain_fold (3); rings on the chain loops for counters (2) and for lines (1); a
+    geometry that hosts several contexts on a workgroup on the hosting loop (0).  Every one bit-exact against the interpreter."""
+    allpairs = golden_util.load("allreduce_a100_allpairs_8r")   # (as msccl-tools' compiler wrote it: runs of nops in front of the folds and the sends)
+    cases = [(allpairs, 256, {}, 3), (allpairs, 256, dict(workgroups=8), 0),
+             (ir_samples.ring_allreduce_xml(8), 4096, dict(protocol="simple"), 2), (ir_samples.ring_allreduce_xml(8), 256, dict(protocol="ll"), 1),
+             (ir_samples.reduce_chain_xml(5, 3), 700, {}, 3)]
+    for xml, elems, knobs, loop in cases:
+        got, ref, _, info = run_both(xml, elems, "float32", seed=91, **knobs)
+        assert info.kernel_loop == loop, (knobs, info.kernel_loop, info.workgroups, info.threads, info.max_hosted)
+        assert_same(got, ref)
+
+
+def test_receives_that_take_over_their_senders_waits():
+    """In exec_kernel_chain_fold a receive whose payload is read in place waits for its sender's dependencies itself instead
+    of for the sender's announcement.  Programs in which such sends have dependencies of every kind -- their own, folded
+    nops in front of them, steps in front of them in their threadblock -- in several passes over the step list, with
+    ragged chunks, against the interpreter; every buffer of every rank compared."""
+    import golden_util
+    for name, elems, knobs in (("allreduce_a100_allpairs_8r", 333, {}), ("allreduce_a100_pcie_hierarchical_8r", 1001, {}),
+                               ("pipeline_a100_allpairs_8r", 257, {}), ("c3_alltoall_two_step_2x8", 4000, dict(slices=2, threads=64, piece_bytes=2048)),
+                               ("allreduce_a100_multinode_allpairs_16r", 129, {}), ("allreduce_a100_allpairs_8r", 3000, dict(slices=4, threads=64, piece_bytes=1024))):
+        xml = golden_util.load(name)
+        algo = oi.parse_xml(xml)
+        rng = np.random.default_rng(17)
+        init = [{b: (rng.random(n * elems, dtype=np.float32) * 2 - 1) for b, n in (("i", g.i_chunks), ("o", g.o_chunks), ("s", g.s_chunks))} for g in algo.gpus]
+        want = [{b: v.copy() for b, v in d.items()} for d in init]
+        oi.Interpreter(algo).run(want, elems, "float32")
+        from msccl.executor import Executor
+        ex = Executor(xml)
+        print(f"case: takeover {name} elems={elems} knobs={knobs}", flush=True)
+        info = ex.setup(elems * 4, "float32", **knobs)
+        assert info.kernel_loop == 3 and (not knobs or info.passes > 1), (name, info.kernel_loop, info.passes)
+        ins = [torch.from_numpy(d["i"]).cuda() if d["i"].size else None for d in init]
+        outs = [torch.from_numpy(d["o"]).cuda() if d["o"].size else None for d in init]
+        for r, d in enumerate(init):
+            if d["s"].size:
+                ex._scratch[r].view(torch.float32).copy_(torch.from_numpy(d["s"]))
+        ex.run(ins, outs)
+        torch.cuda.synchronize()
+        for r in range(algo.ngpus):
+            got = {"i": ins[r], "o": outs[r], "s": None if ex._scratch[r] is None else ex._scratch[r].view(torch.float32)}
+            for b in "ios":
+                if want[r][b].size:
+                    assert np.array_equal(got[b].cpu().numpy().view(np.uint32), want[r][b].view(np.uint32)), (name, r, b)
+
+
 def test_protocol_from_the_ir():
     """protocol="ir": the <algo proto=...> attribute picks the protocol (LL, LL128 -> lines)."""
     xml = ir_samples.ring_allreduce_xml(4)
