@@ -246,6 +246,14 @@ struct SubDword {
   }
 };
 
+#ifdef MSCCLX_LDS_STAGING
+// (one area for every instantiation of the movers: 64 KiB, so that two workgroups of 512 threads still share a compute unit)
+__device__ __noinline__ u32x4* lds_stage_area() {
+  __shared__ u32x4 area[(kUnroll / 2 > 0 ? kUnroll / 2 : 1) * 1024];
+  return area;
+}
+#endif
+
 // o1 = a [(+) b] over `bytes` bytes in units of W, UA units in flight per thread and operand: the loop of
 // move_units, for the part of a row that starts on a line of its destination.
 template <class R, bool HAS_B, bool NT1, int UA>
@@ -358,8 +366,22 @@ __device__ __forceinline__ void move_units(unsigned char* o1, unsigned char* o2,
 #pragma unroll
     for (int u = 0; u < UA; ++u) x[u] = A::template ld<XL>(ra, (int)((i + u * T) * W));
     if (HAS_B) {
+#ifdef MSCCLX_LDS_STAGING
+      // Experiment, off by default: the local operand of a reduction goes from memory straight into LDS (16 bytes per
+      // lane, a wave's 1 KiB at a time) and is read from there when the payload has arrived, instead of waiting in
+      // vector registers.  Measured slower everywhere (the registers are there, and LDS adds a trip): kept for the record.
+      u32x4* const lds_stage = lds_stage_area();
+#pragma unroll
+      for (int u = 0; u < UA; ++u)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)&lds_stage[u * T + (threadIdx.x & ~63u)], 16,
+                                             (int)((i + u * T) * W), 0, 0, XL);
+      __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+      for (int u = 0; u < UA; ++u) y[u] = i + u * T < n ? lds_stage[u * T + threadIdx.x] : word{0, 0, 0, 0};
+#else
 #pragma unroll
       for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * W));
+#endif
 #pragma unroll
       for (int u = 0; u < UA; ++u) x[u] = R::combine(y[u], x[u]);
     }
@@ -492,6 +514,8 @@ __device__ __forceinline__ bool is_send(int t) { return t == MSCCLX_OP_SEND || t
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t ll_flag(uint32_t epoch, u64 seq) { return ((epoch & 0x3ffu) << 22) | (uint32_t)((seq + 1) & 0x3fffffu); }
 __device__ __forceinline__ bool ll_valid(u32x4 l0, u32x4 l1, uint32_t f) { return l0.y == f && l0.w == f && l1.y == f && l1.w == f; }
+// The same question in integers, nonzero while a flag is missing (no `&&` whose early exits a lane would have to branch around).
+__device__ __forceinline__ uint32_t ll_stale(u32x4 l0, u32x4 l1, uint32_t f) { return (l0.y ^ f) | (l0.w ^ f) | (l1.y ^ f) | (l1.w ^ f); }
 
 // The area's abort word is raised.  If it was the host that raised it (mscclx_plan_abort), whoever sees it says so in the
 // launch's status: a launch replayed from a HIP graph passes by the host code that would have re-armed the counters, and
@@ -907,12 +931,16 @@ struct ChainWatch {
 // reach gate_target before the outgoing slot may be written, or null.  The polling is uniform: all
 // lanes ask again until every lane has its lines (a line that is there stays until this context frees
 // the slot) -- no per-lane masks to keep, a fifth less time per hop than lane-by-lane retries.
-template <class R, int U>
+template <class R, int U, int T>
 __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rout, const __amdgpu_buffer_rsrc_t rsrc,
-                                            const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool rcv, const bool snd,
-                                            const bool from_src, const bool has_b, const bool to_local, const bool nt, const uint32_t fin,
+                                            const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool nt, const uint32_t fin,
                                             const uint32_t fout, const u64* gate, const u64 gate_target, const ChainWatch& watch, const int step,
                                             const uint32_t pass, u64* prof_acc, u64& prof_mark, const u64 prof_floor) {
+  // what a step of type T does, known where the code is generated: one straight run of instructions per type
+  constexpr bool rcv = ((0x7cu >> T) & 1u) != 0, snd = ((0x5au >> T) & 1u) != 0;
+  constexpr bool from_src = T == MSCCLX_OP_SEND || T == MSCCLX_OP_COPY || T == MSCCLX_OP_REDUCE;
+  constexpr bool has_b = T == MSCCLX_OP_RRC || T == MSCCLX_OP_RRS || T == MSCCLX_OP_RRCS || T == MSCCLX_OP_REDUCE;
+  constexpr bool to_local = T == MSCCLX_OP_RECV || T == MSCCLX_OP_RCS || T == MSCCLX_OP_RRC || T == MSCCLX_OP_RRCS || T == MSCCLX_OP_COPY || T == MSCCLX_OP_REDUCE;
   typedef Access<16> A;
   constexpr int XL = MSCCLX_AUX_LD, XP = (int)(0x80000000u | MSCCLX_AUX), XF = MSCCLX_AUX, XS = MSCCLX_AUX_ST, XN = MSCCLX_AUX_ST_FINAL;
   u32x4 lo[U], hi[U], x[U], y[U];
@@ -924,25 +952,25 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
   for (int u = 0; u < U; ++u) {
     const uint32_t i = i0 + 64u * (uint32_t)u;
     lo[u] = hi[u] = x[u] = y[u] = u32x4{0, 0, 0, 0};
-    if (rcv) {
+    if constexpr (rcv) {
       lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
       hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
-    } else if (from_src) {
+    } else if constexpr (from_src) {
       x[u] = A::template ld<XL>(rsrc, (int)(i * 16));
     }
   }
-  if (has_b) {
+  if constexpr (has_b) {
 #pragma unroll
     for (int u = 0; u < U; ++u) y[u] = A::template ld<XL>(rdst, (int)((i0 + 64u * (uint32_t)u) * 16));
   }
-  u64 gate_seen = gate ? load_counter(gate) : ~0ull;
+  u64 gate_seen = snd && gate ? load_counter(gate) : ~0ull;
   bool lost = false;
-  if (rcv) {
+  if constexpr (rcv) {
     auto all_there = [&]() {
-      bool mine = true;
+      uint32_t missing = 0;
 #pragma unroll
-      for (int u = 0; u < U; ++u) mine = mine && (i0 + 64u * (uint32_t)u >= n || ll_valid(lo[u], hi[u], fin));
-      return __builtin_amdgcn_ballot_w64(!mine) == 0;
+      for (int u = 0; u < U; ++u) missing |= i0 + 64u * (uint32_t)u < n ? ll_stale(lo[u], hi[u], fin) : 0u;
+      return __builtin_amdgcn_ballot_w64(missing != 0) == 0;
     };
     unsigned spins = 0;
     u64 since = 0;
@@ -981,11 +1009,11 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
   }
   MSCCLX_CHAIN_CLOCK(prof_got);
   MSCCLX_CHAIN_ADD(1, prof_ld, prof_got);
-  if (has_b) {
+  if constexpr (has_b) {
 #pragma unroll
     for (int u = 0; u < U; ++u) x[u] = R::combine(y[u], x[u]);
   }
-  if (gate) {  // the slot may still be being read
+  if (snd && gate) {  // the slot may still be being read
     unsigned spins = 0;
     u64 since = 0;
     while (uniform((uint64_t)gate_seen) < gate_target && !lost) {
@@ -998,7 +1026,7 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
     }
   }
   if (lost) return false;  // (the same in all lanes: every wait above is uniform)
-  if (snd) {  // the forwarded lines first: the next rank is waiting for them
+  if constexpr (snd) {  // the forwarded lines first: the next rank is waiting for them
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + 64u * (uint32_t)u;
@@ -1006,7 +1034,7 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
       A::template st<XF>(rout, (int)(i * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
     }
   }
-  if (to_local) {
+  if constexpr (to_local) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + 64u * (uint32_t)u;
@@ -1030,6 +1058,59 @@ __device__ __forceinline__ DevOp fetch_step(ConstOps e) {  // (field by field: a
   r.word = e->word; r.dep_tb = e->dep_tb; r.dep_step = e->dep_step; r.dep_nops = e->dep_nops;
   r.extra = e->extra; r.steps = e->steps;
   r.src_addr = e->src_addr; r.dst_addr = e->dst_addr; r.in_addr = e->in_addr;
+  return r;
+}
+
+// The rows of one step of type T (run_chain): packed in the slots, a chunk apart in the rank's buffers.
+template <class R, int T>
+__device__ __forceinline__ bool chain_rows(const unsigned char* in_row, unsigned char* out_row, u64 src_row, u64 dst_row, const u64 row_stride,
+                                           const uint32_t cnt, const uint32_t n, const uint32_t row_line_bytes, const uint32_t local_bytes,
+                                           const uint32_t lane, const bool nt, const uint32_t fin, const uint32_t fout, const u64* gate,
+                                           const u64 gate_target, const ChainWatch& watch, const int step, const uint32_t pass, u64* prof_acc,
+                                           u64& prof_mark, const u64 prof_floor) {
+  for (uint32_t row = 0; row < cnt; ++row) {
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, row_line_bytes), rout = make_rsrc(out_row, row_line_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, local_bytes), rdst = make_rsrc((const void*)dst_row, local_bytes);
+    if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
+      if (!chain_round<R, 1, T>(rin, rout, rsrc, rdst, lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark, prof_floor)) return false;
+      gate = nullptr;
+    } else {
+      for (uint32_t base = 0; base < n; base += 128) {
+        if (!chain_round<R, 2, T>(rin, rout, rsrc, rdst, base + lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark, prof_floor))
+          return false;
+        gate = nullptr;
+      }
+    }
+    in_row += row_line_bytes; out_row += row_line_bytes;
+    src_row += row_stride; dst_row += row_stride;
+  }
+  return true;
+}
+
+// A step's table entry asked for ahead of time.  Scalar loads would bring it straight to scalar registers, but
+// they complete out of order, so the first wait for any scalar value -- a spilled register is enough -- waits
+// for the entry as well, and an entry is used once per pass: most of these loads miss the scalar cache.  Asked
+// for with vector loads (every lane the same address), the entry arrives behind the loads issued before it and
+// ahead of the lines that the wave polls for; twelve moves then carry it to scalar registers.
+struct StepAhead {
+  u32x4 a, b, c;  // a: word dep_tb dep_step dep_nops, b: extra steps src_addr, c: dst_addr in_addr
+};
+static_assert(offsetof(DevOp, extra) == 16 && offsetof(DevOp, dst_addr) == 32, "StepAhead names DevOp's fields by their place");
+__device__ __forceinline__ StepAhead ask_step(const __amdgpu_buffer_rsrc_t table, uint32_t index) {
+  StepAhead r;
+  const int at = (int)(index * (uint32_t)sizeof(DevOp));
+  r.a = Access<16>::template lds<0>(table, 0, at);
+  r.b = Access<16>::template lds<0>(table, 16, at);
+  r.c = Access<16>::template lds<0>(table, 32, at);
+  return r;
+}
+__device__ __forceinline__ DevOp take_step(const StepAhead& e) {
+  DevOp r;
+  r.word = uniform(e.a.x); r.dep_tb = (int32_t)uniform(e.a.y); r.dep_step = (int32_t)uniform(e.a.z); r.dep_nops = (int32_t)uniform(e.a.w);
+  r.extra = uniform(e.b.x); r.steps = uniform(e.b.y);
+  r.src_addr = (u64)uniform(e.b.z) | (u64)uniform(e.b.w) << 32;
+  r.dst_addr = (u64)uniform(e.c.x) | (u64)uniform(e.c.y) << 32;
+  r.in_addr = (u64)uniform(e.c.z) | (u64)uniform(e.c.w) << 32;
   return r;
 }
 
@@ -1064,13 +1145,14 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
   const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
   uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
   DevOp op = fetch_step(ops);
+  const __amdgpu_buffer_rsrc_t table = make_rsrc(p.ops + uniform(h.op_begin), nops * (uint32_t)sizeof(DevOp));
   MSCCLX_CHAIN_CLOCK(prof_begin);
   u64 prof_mark = 0;  // profiling builds: when the previous step's stores were issued
 #ifdef MSCCLX_PROFILE
   prof_mark = prof_begin;
 #endif
   for (;;) {
-    const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+    const StepAhead after = ask_step(table, step + 1 == nops ? 0 : step + 1);  // (it arrives while the wave waits)
     MSCCLX_CHAIN_CLOCK(prof_dep0);
     const int t = (int)(op.word & 15u);
     const uint32_t cnt = op.word >> kOpCntShift;
@@ -1097,39 +1179,33 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
     prof_floor = __builtin_amdgcn_s_memtime();
     prof_acc[0] += prof_floor - prof_dep0;
 #endif
-    const bool rcv = is_recv(t), snd = is_send(t);
-    const bool from_src = t == MSCCLX_OP_SEND || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
-    const bool has_b = t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRS || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_REDUCE;
-    const bool to_local = t == MSCCLX_OP_RECV || t == MSCCLX_OP_RCS || t == MSCCLX_OP_RRC || t == MSCCLX_OP_RRCS || t == MSCCLX_OP_COPY || t == MSCCLX_OP_REDUCE;
+    const bool snd = ((0x5au >> t) & 1u) != 0;
     const bool nt = (op.word & kOpNtStore) != 0;
     const uint32_t fin = ll_flag(epoch, rseq), fout = ll_flag(epoch, sseq);
     const u64* gate = (snd && sseq >= depth) ? out_tail : nullptr;  // looked at in the step's first round only
     const u64 gate_target = (u64)sseq + 1 - depth;
-    // the step's rows: packed in the slots, a chunk apart in the rank's buffers
-    const unsigned char* in_row = in_ring + rslot;
-    unsigned char* out_row = out_ring + sslot;
-    u64 src_row = op.src_addr + off, dst_row = op.dst_addr + off;
     const uint32_t row_line_bytes = n * kLLUnitBytes;
     const uint32_t local_bytes = n * 16 - (left <= piece ? end_clip : 0u);  // rank-buffer rows may end inside their last unit; lines are whole
-    if (t != MSCCLX_OP_NOP) {
-      for (uint32_t row = 0; row < cnt; ++row) {
-        const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, row_line_bytes), rout = make_rsrc(out_row, row_line_bytes);
-        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, local_bytes), rdst = make_rsrc((const void*)dst_row, local_bytes);
-        if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
-          if (!chain_round<R, 1>(rin, rout, rsrc, rdst, lane, n, rcv, snd, from_src, has_b, to_local, nt, fin, fout, gate, gate_target, watch, (int)step, pass,
-                                 prof_acc, prof_mark, prof_floor)) return;
-          gate = nullptr;
-        } else {
-          for (uint32_t base = 0; base < n; base += 128) {
-            if (!chain_round<R, 2>(rin, rout, rsrc, rdst, base + lane, n, rcv, snd, from_src, has_b, to_local, nt, fin, fout, gate, gate_target, watch, (int)step,
-                                   pass, prof_acc, prof_mark, prof_floor)) return;
-            gate = nullptr;
-          }
-        }
-        in_row += row_line_bytes; out_row += row_line_bytes;
-        src_row += row_stride; dst_row += row_stride;
-      }
+    bool ok = true;
+#define MSCCLX_CHAIN_CASE(T)                                                                                                                                     \
+  case T:                                                                                                                                                        \
+    ok = chain_rows<R, T>(in_ring + rslot, out_ring + sslot, op.src_addr + off, op.dst_addr + off, row_stride, cnt, n, row_line_bytes, local_bytes, lane, nt, fin, \
+                          fout, gate, gate_target, watch, (int)step, pass, prof_acc, prof_mark, prof_floor);                                                    \
+    break
+    switch (t) {  // (one copy of the step's instructions per type, with nothing left to decide inside)
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_SEND);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_RECV);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_RCS);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_RRS);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_RRC);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_RRCS);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_COPY);
+      MSCCLX_CHAIN_CASE(MSCCLX_OP_REDUCE);
+      default: break;  // nop
     }
+#undef MSCCLX_CHAIN_CASE
+    if (!ok) return;
+    const bool rcv = ((0x7cu >> t) & 1u) != 0;
     // (in integers, not under `if (rcv)`: the compiler turns such an `if` into a per-lane select and
     // the running values would move to vector registers, and every address made from them with them)
     const uint32_t rcv_bit = (0x7cu >> t) & 1u, snd_bit = (0x5au >> t) & 1u;  // r rcs rrs rrc rrcs / s rcs rrs rrcs
@@ -1156,7 +1232,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       }
     }
     if (rcv && writer) publish(in_tail, (u64)rseq);
-    op = after;
+    op = take_step(after);
   }
 #ifdef MSCCLX_PROFILE
   prof_acc[4] = __builtin_amdgcn_s_memtime() - prof_begin;
@@ -1228,12 +1304,13 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
   const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
   uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
   DevOp op = fetch_step(ops);
+  const __amdgpu_buffer_rsrc_t table = make_rsrc(p.ops + uniform(h.op_begin), nops * (uint32_t)sizeof(DevOp));
   // (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for the step's counters, 1 moving its rows,
   // 2 waiting for the stores' acknowledgement, 3 on the bookkeeping between steps, 4 in all)
   MSCCLX_CHAIN_CLOCK(prof_begin);
   for (;;) {
     MSCCLX_CHAIN_CLOCK(prof_top);
-    const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+    const StepAhead after = ask_step(table, step + 1 == nops ? 0 : step + 1);  // (it arrives while the wave waits)
     const uint32_t t = op.word & 15u;
     const uint32_t cnt = op.word >> kOpCntShift;
     const uint32_t n = left < piece ? left : piece;
@@ -1330,7 +1407,7 @@ __device__ __forceinline__ void run_chain_counters(const KernelParams& p, int ct
       off += (u64)piece * 16;
       if (++pass >= npasses) break;
     }
-    op = after;
+    op = take_step(after);
 #ifdef MSCCLX_PROFILE
     prof_acc[3] += __builtin_amdgcn_s_memtime() - prof_moved;
 #endif
@@ -1645,12 +1722,19 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
     const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
     uint32_t step = 0, pass = 0, rseq = 0, sseq = 0, rslot = 0, sslot = 0, count = 0;
     DevOp op = fetch_step(ops);
+    const __amdgpu_buffer_rsrc_t table = make_rsrc(p.ops + uniform(h.op_begin), nops * (uint32_t)sizeof(DevOp));
     uint2 entry = {0u, 0u};  // this lane's folded dependency of the step `op`, if it has one
     if (lane < (op.extra & 255u)) entry = extras[(op.extra >> 8) + lane];
+    // The table is read two steps ahead: the entry of the step after this one is there when this step begins, so
+    // that its lanes can ask for their folded dependencies, and the entry of the step after that is on its way.
+    StepAhead after = ask_step(table, nops > 1 ? 1u : 0u);
     for (;;) {
-      const DevOp after = fetch_step(ops + (step + 1 == nops ? 0 : step + 1));  // (it arrives while the wave waits)
+      uint32_t second = step + 2;
+      second = second >= nops ? second - nops : second;
+      second = second >= nops ? 0u : second;  // (a table of one step)
+      const StepAhead after_that = ask_step(table, second);
       uint2 next_entry = {0u, 0u};
-      if (lane < (after.extra & 255u)) next_entry = extras[(after.extra >> 8) + lane];
+      if (lane < (after.b.x & 255u)) next_entry = extras[(after.b.x >> 8) + lane];  // (b.x: DevOp::extra)
       const uint32_t t = op.word & 15u;
       const uint32_t cnt = op.word >> kOpCntShift;
       const uint32_t n = left < piece ? left : piece;
@@ -1743,7 +1827,8 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
         off += (u64)piece * 16;
         if (++pass >= npasses) break;
       }
-      op = after;
+      op = take_step(after);
+      after = after_that;
       entry = next_entry;
     }
   }
