@@ -40,7 +40,7 @@ for p in (ROOT, os.path.join(ROOT, "msccl-tools_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0
-PMC_SUMMARY = os.path.join(ROOT, "profiles", "exec_kernel_c2_c3_c4_pmc.txt")
+PMC_SUMMARY = os.path.join(ROOT, "profiles", "exec_kernel_hbm_traffic_pmc.txt")
 ROOFLINE_NOTE = ("achieved = algorithmic bytes per launch / mean launch duration (HIP events); traffic = rocprofv3 FETCH_SIZE + "
                  "WRITE_SIZE per launch, counted between L2 and the fabric, so reads served by the memory-side cache are "
                  "included: the fraction is algorithmic bytes over the HBM peak, not proven DRAM traffic")
@@ -256,6 +256,48 @@ def run_workload(key, steps, warmup, device="cuda:0", bytes_per_rank=None, host_
 CPU_SAMPLE_BYTES = {"c1": 1 << 20, "c2": 32 << 20, "c3": 64 << 20, "c4": 128 << 20, "c5": 256 << 10, "c5_chain": 256 << 10}
 
 
+def parse_knobs(text):
+    knobs = {}
+    for kv in filter(None, (text or "").split(",")):
+        k, _, v = kv.partition("=")
+        knobs[k] = v if k == "protocol" else int(v)
+    return knobs
+
+
+def time_program(path, chunk_sizes, steps, warmup, knobs):
+    """Kernel time of one MSCCL-IR document at the given chunk sizes: HIP events around each of `steps` queued launches on the
+    launch stream, median and mean.  Inputs are random; an all-reduce keeps reducing what the launch before left (finite for
+    the few launches timed here)."""
+    import gzip
+    import torch
+    from msccl.executor import Executor, parse_algo_xml
+    from msccl.executor.binding import LOOP_NAMES
+    from msccl.executor.workloads import HBM_PEAK_BYTES_PER_S
+    opener = gzip.open if path.endswith(".gz") else open
+    with opener(path, "rt") as f:
+        tables = parse_algo_xml(f.read())
+    for cb in chunk_sizes:
+        ins = [torch.rand(int(tables.rank_chunks[r, 0]) * cb // 4, device="cuda:0") * 1e-3 if tables.rank_chunks[r, 0] else None for r in range(tables.ngpus)]
+        outs = [torch.zeros(int(tables.rank_chunks[r, 1]) * cb // 4, device="cuda:0") if tables.rank_chunks[r, 1] else None for r in range(tables.ngpus)]
+        ex = Executor(tables)
+        info = ex.setup(cb, "float32", **knobs)
+        ex.bind(ins, outs)
+        for _ in range(max(1, warmup)):
+            ex.launch()
+        ex.wait()
+        ts = sorted(ex.time(steps))
+        ex.wait()
+        med, mean = ts[len(ts) // 2] * 1e-3, sum(ts) / len(ts) * 1e-3
+        ab = ex.algorithmic_bytes()
+        print(json.dumps({"program": os.path.basename(path), "ranks": int(tables.ngpus), "collective": tables.coll, "chunk_bytes": cb,
+                          "us_per_launch_median": round(med * 1e6, 2), "us_per_launch_mean": round(mean * 1e6, 2), "launches": steps,
+                          "algorithmic_bytes": int(ab), "algorithmic_GBps": round(ab / med / 1e9, 1), "hbm_fraction": round(ab / med / HBM_PEAK_BYTES_PER_S, 4),
+                          "step_loop": LOOP_NAMES.get(int(info.kernel_loop), str(int(info.kernel_loop))),
+                          "geometry": {k: int(getattr(info, k)) for k in ("workgroups", "threads", "slices", "piece_bytes", "passes", "max_hosted", "protocol")},
+                          "knobs": knobs}), flush=True)
+        del ex, ins, outs
+
+
 def cpu_baseline(key):
     """NumPy interpreter (oracle/) on the same IR and input distribution, host cores of this box."""
     import numpy as np
@@ -305,6 +347,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy baseline")
     ap.add_argument("--sweep", metavar="LO:HI", help="instead of the benchmark line: time the chosen algorithm on LO, 2*LO, ... HI bytes per "
                     "rank (same inputs, same timing; results not verified) and print one JSON line holding the list")
+    ap.add_argument("--xml", metavar="PATH", help="instead of the benchmark line: time the MSCCL-IR program in PATH (.xml or .xml.gz) on random "
+                    "float32 inputs, automatic geometry unless --knobs says otherwise, one JSON line per chunk size (results not verified)")
+    ap.add_argument("--chunk-bytes", default="4096", metavar="N[,N...]", help="with --xml: bytes of one IR chunk")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run five plain device copies of 1 GiB (known traffic: 1 GiB read + 1 GiB written each), "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -318,6 +363,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the executor has no CPU path", file=sys.stderr)
         sys.exit(3)
+
+    if args.xml:
+        time_program(args.xml, [int(b) for b in args.chunk_bytes.split(",")], args.steps, args.warmup, parse_knobs(args.knobs))
+        return
 
     if args.calibrate_copy:
         src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda:0")
@@ -340,10 +389,7 @@ def main():
         print(json.dumps({"sweep": args.config, "workload": r["workload"].split(";")[0], "dtype": r["dtype"], "steps": args.steps, "rows": rows}))
         return
     traffic = measured_traffic()
-    knobs = {}
-    for kv in filter(None, args.knobs.split(",")):
-        k, _, v = kv.partition("=")
-        knobs[k] = v if k == "protocol" else int(v)
+    knobs = parse_knobs(args.knobs)
     head = run_workload(args.config, args.steps, args.warmup, host_costs=True, knobs=knobs)
     line = {
         "metric": "algbw_GBps", "value": head["algbw_GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -556,10 +556,14 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
   constexpr int XL = MSCCLX_AUX_LD, XF = MSCCLX_AUX, XV = (int)(0x80000000u | MSCCLX_AUX), X1 = NT1 ? MSCCLX_AUX_ST_FINAL : MSCCLX_AUX_ST;
   // (rank buffers end `clip` bytes inside their last unit; lines are always whole: their flags must arrive)
   const uint32_t local_bytes = n * 16 - clip;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, IN_LL ? n * kLLUnitBytes : local_bytes);
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, HAS_B ? local_bytes : (IN_LL ? n * kLLUnitBytes : local_bytes));
+  // (a row of lines: the first halves of its n units, then the second halves -- see kLLUnitBytes; one descriptor per half,
+  // so that lanes past the row's end load zeros and store nothing in either)
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, IN_LL ? n * 16 : local_bytes);
+  const __amdgpu_buffer_rsrc_t ra2 = make_rsrc(a + (IN_LL ? n * 16 : 0), IN_LL ? n * 16 : 0);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(HAS_B ? b : a, HAS_B ? local_bytes : (IN_LL ? n * 16 : local_bytes));
   const __amdgpu_buffer_rsrc_t r1 = make_rsrc(HAS_O1 ? o1 : const_cast<unsigned char*>(a), HAS_O1 ? local_bytes : 0);
-  const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * kLLUnitBytes : 0);
+  const __amdgpu_buffer_rsrc_t rl = make_rsrc(OUT_LL ? llo : const_cast<unsigned char*>(a), OUT_LL ? n * 16 : 0);
+  const __amdgpu_buffer_rsrc_t rl2 = make_rsrc(OUT_LL ? llo + n * 16 : const_cast<unsigned char*>(a), OUT_LL ? n * 16 : 0);
   const uint32_t T = blockDim.x;
   constexpr int UA = 2;  // small pieces: few lines per thread, few registers
   for (uint32_t i = threadIdx.x; i < n; i += UA * T) {
@@ -567,8 +571,8 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
     if (IN_LL) {
       static_assert(UA == 2, "the retry below names its two units");
       const uint32_t ia = i, ib = i + T;
-      u32x4 a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)), a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16));
-      u32x4 b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)), b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16));
+      u32x4 a0 = A::template ld<XV>(ra, (int)(ia * 16)), a1 = A::template ld<XV>(ra2, (int)(ia * 16));
+      u32x4 b0 = A::template ld<XV>(ra, (int)(ib * 16)), b1 = A::template ld<XV>(ra2, (int)(ib * 16));
       if (HAS_B) {
 #pragma unroll
         for (int u = 0; u < UA; ++u) y[u] = A::template ld<XL>(rb, (int)((i + u * T) * 16));
@@ -579,8 +583,8 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
         const bool ok_a = ll_valid(a0, a1, fin), ok_b = ib >= n || ll_valid(b0, b1, fin);
         if (ok_a && ok_b) break;
         MSCCLX_POLL_PAUSE();
-        if (!ok_a) { a0 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes)); a1 = A::template ld<XV>(ra, (int)(ia * kLLUnitBytes + 16)); }
-        if (!ok_b) { b0 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes)); b1 = A::template ld<XV>(ra, (int)(ib * kLLUnitBytes + 16)); }
+        if (!ok_a) { a0 = A::template ld<XV>(ra, (int)(ia * 16)); a1 = A::template ld<XV>(ra2, (int)(ia * 16)); }
+        if (!ok_b) { b0 = A::template ld<XV>(ra, (int)(ib * 16)); b1 = A::template ld<XV>(ra2, (int)(ib * 16)); }
         if ((++spins & 0x7fu) == 0) {
           const u64 now = wall_clock64();
           if (!since) since = now;
@@ -606,8 +610,8 @@ __device__ __forceinline__ void move_units_ll(unsigned char* o1, unsigned char* 
     if (OUT_LL) {  // the forwarded lines first: the next rank is waiting for them
 #pragma unroll
       for (int u = 0; u < UA; ++u) {
-        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes), u32x4{x[u].x, fout, x[u].y, fout});
-        A::template st<XF>(rl, (int)((i + u * T) * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
+        A::template st<XF>(rl, (int)((i + u * T) * 16), u32x4{x[u].x, fout, x[u].y, fout});
+        A::template st<XF>(rl2, (int)((i + u * T) * 16), u32x4{x[u].z, fout, x[u].w, fout});
       }
     }
     if (HAS_O1) {
@@ -745,7 +749,7 @@ __device__ __forceinline__ void describe_step(Context& c, const Hosted& h, const
     if (in_place) { in = op.in_addr + c.off; in_packed = 0; }
     else in = (u64)p.fifo + (u64)h.in_slots * 16 + c.rslot;
     if (LL) {
-      c.w1 = (const u64*)(in + ((uint64_t)((uint32_t)cnt * n) - 1) * kLLUnitBytes + 24);
+      c.w1 = (const u64*)(in + (uint64_t)((uint32_t)cnt * n) * kLLUnitBytes - 8);  // the last word and flag of the last row's last unit
       c.t1 = ll_flag(epoch, c.rseq);
     } else if (!(in_place && (op.steps & kStepsNoAnnouncement))) {
       c.w1 = p.sync_cur + h.head_in;
@@ -932,8 +936,8 @@ struct ChainWatch {
 // lanes ask again until every lane has its lines (a line that is there stays until this context frees
 // the slot) -- no per-lane masks to keep, a fifth less time per hop than lane-by-lane retries.
 template <class R, int U, int T>
-__device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rout, const __amdgpu_buffer_rsrc_t rsrc,
-                                            const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool nt, const uint32_t fin,
+__device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rin2, const __amdgpu_buffer_rsrc_t rout,
+                                            const __amdgpu_buffer_rsrc_t rout2, const __amdgpu_buffer_rsrc_t rsrc, const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool nt, const uint32_t fin,
                                             const uint32_t fout, const u64* gate, const u64 gate_target, const ChainWatch& watch, const int step,
                                             const uint32_t pass, u64* prof_acc, u64& prof_mark, const u64 prof_floor) {
   // what a step of type T does, known where the code is generated: one straight run of instructions per type
@@ -953,8 +957,8 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
     const uint32_t i = i0 + 64u * (uint32_t)u;
     lo[u] = hi[u] = x[u] = y[u] = u32x4{0, 0, 0, 0};
     if constexpr (rcv) {
-      lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
-      hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
+      lo[u] = A::template ld<XP>(rin, (int)(i * 16));
+      hi[u] = A::template ld<XP>(rin2, (int)(i * 16));
     } else if constexpr (from_src) {
       x[u] = A::template ld<XL>(rsrc, (int)(i * 16));
     }
@@ -981,9 +985,9 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
         // and again costs memory traffic that the ranks at work pay for -- 4096 waiting waves ask for
         // 16 MiB a round.  Watch the round's last line alone until it is there, then ask for all.
         const uint32_t round_end = i0 - threadIdx.x + 64u * (uint32_t)U;
-        const int watched = (int)(((round_end < n ? round_end : n) - 1u) * kLLUnitBytes + 16u);
+        const int watched = (int)(((round_end < n ? round_end : n) - 1u) * 16u);  // (its second half)
         for (;;) {
-          const u32x4 w = A::template ld<XP>(rin, watched);
+          const u32x4 w = A::template ld<XP>(rin2, watched);
           if (uniform(w.y) == fin && uniform(w.w) == fin) break;
           MSCCLX_POLL_PAUSE();
           if ((++spins & 0x3fu) == 0) {
@@ -996,8 +1000,8 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t i = i0 + 64u * (uint32_t)u;
-        lo[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes));
-        hi[u] = A::template ld<XP>(rin, (int)(i * kLLUnitBytes + 16));
+        lo[u] = A::template ld<XP>(rin, (int)(i * 16));
+        hi[u] = A::template ld<XP>(rin2, (int)(i * 16));
       }
       if ((++spins & 0x3fu) == 0) {
         since = uniform((uint64_t)chain_slow_check(watch.abort_word, watch.host_status, watch.timeout_ticks, since, watch.tb, step, watch.slice, (u64)pass, 1));
@@ -1030,8 +1034,8 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + 64u * (uint32_t)u;
-      A::template st<XF>(rout, (int)(i * kLLUnitBytes), u32x4{x[u].x, fout, x[u].y, fout});
-      A::template st<XF>(rout, (int)(i * kLLUnitBytes + 16), u32x4{x[u].z, fout, x[u].w, fout});
+      A::template st<XF>(rout, (int)(i * 16), u32x4{x[u].x, fout, x[u].y, fout});
+      A::template st<XF>(rout2, (int)(i * 16), u32x4{x[u].z, fout, x[u].w, fout});
     }
   }
   if constexpr (to_local) {
@@ -1069,14 +1073,20 @@ __device__ __forceinline__ bool chain_rows(const unsigned char* in_row, unsigned
                                            const u64 gate_target, const ChainWatch& watch, const int step, const uint32_t pass, u64* prof_acc,
                                            u64& prof_mark, const u64 prof_floor) {
   for (uint32_t row = 0; row < cnt; ++row) {
-    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, row_line_bytes), rout = make_rsrc(out_row, row_line_bytes);
+    // (a row of lines: the first halves of its n units, then the second halves; a descriptor for each)
+    const uint32_t half = row_line_bytes >> 1;
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_row, half), rin2 = make_rsrc(in_row + half, half);
+    const __amdgpu_buffer_rsrc_t rout = make_rsrc(out_row, half), rout2 = make_rsrc(out_row + half, half);
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, local_bytes), rdst = make_rsrc((const void*)dst_row, local_bytes);
     if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
-      if (!chain_round<R, 1, T>(rin, rout, rsrc, rdst, lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark, prof_floor)) return false;
+      if (!chain_round<R, 1, T>(rin, rin2, rout, rout2, rsrc, rdst, lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark,
+                                prof_floor))
+        return false;
       gate = nullptr;
     } else {
       for (uint32_t base = 0; base < n; base += 128) {
-        if (!chain_round<R, 2, T>(rin, rout, rsrc, rdst, base + lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark, prof_floor))
+        if (!chain_round<R, 2, T>(rin, rin2, rout, rout2, rsrc, rdst, base + lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark,
+                                  prof_floor))
           return false;
         gate = nullptr;
       }

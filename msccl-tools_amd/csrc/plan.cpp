@@ -705,27 +705,34 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
       // message cost more than the hand-off saves (8-rank ring on 1 MiB: 38 us either way; on 2 MiB
       // 59 against 40 us).  Programs whose nops can be folded keep the counters: folding, and chains
       // of local reduces done as one step, are worth more there.  Only when every knob is automatic.
+      // Since a row of lines is laid out halves apart (plan.h, kLLUnitBytes) and the chain loop has one copy of a step's
+      // instructions per step type, lines also win with four such workgroups per compute unit (8-rank ring on 1 MiB per
+      // rank 30.5 -> 27.0 us, 16-rank ring on 1 MiB 57.7 -> 53.4 us), with pieces of 2 KiB where a ring is 32 hand-offs
+      // or longer (32-rank ring on 2 MiB per rank 146 -> 130 us; the 8- and 16-rank rings tie there; the 64-rank chain, in
+      // which one rank works at a time, loses 5 %), and for chains of
+      // seven hand-offs (8-rank ring all-gather and reduce-scatter at 1 to 128 KiB chunks: 0.7 to 1.5 us off 15 to 18).
       if (cfg.protocol == MSCCLX_PROTO_AUTO && chunk_bytes % 4 == 0 && !cfg.staging && !cfg.piece_bytes && !cfg.threads && !cfg.workgroups &&
-          depth_of_dataflow >= 8 && !has_foldable_nops(plan)) {
+          depth_of_dataflow >= 7 && !has_foldable_nops(plan)) {
         int64_t s = slices;
         // Where the chain is long (12 hand-offs or more) the two per compute unit are taken among the contexts busy at a
         // time, contexts over 1.6 x waiting_ratio: 32-rank two-level all-reduce at 0.5 to 2 KiB chunks 42-45 -> 34-40 us,
         // pipelined ring at 12 to 32 KiB 29-32 -> 25-28 us, 64-rank chain at 12 to 64 KiB 172-181 -> 119-126 us.  (Over
         // 2 x waiting_ratio the pipelined ring lost 23 % at 64 KiB; a chain of 8 hand-offs lost 6 to 10 %.)
-        const double lines_most = depth_of_dataflow >= 12 ? std::max(2.0, 1.6 * ratio) * (double)num_cus : 2.0 * (double)num_cus;
-        while (chunk_bytes / (uint64_t)s > 1024 && (double)(s * 2 * ntbs) <= lines_most && (uint64_t)(s * 2) <= g.chunk_units) s *= 2;
+        const double lines_most = depth_of_dataflow >= 12 ? std::max(4.0, 1.6 * ratio) * (double)num_cus : 4.0 * (double)num_cus;
+        const uint64_t lines_piece = depth_of_dataflow >= 32 && ratio < 2.0 ? 2048 : 1024;  // (a ring: every threadblock busy all the time)
+        while (chunk_bytes / (uint64_t)s > lines_piece && (double)(s * 2 * ntbs) <= lines_most && (uint64_t)(s * 2) <= g.chunk_units) s *= 2;
         int64_t most_msgs = 0;
         for (const Conn& c : plan.conns) most_msgs = std::max<int64_t>(most_msgs, c.nmsg);
-        if (chunk_bytes / (uint64_t)s <= 1024 && (double)(s * ntbs) <= lines_most && s * ntbs <= capacity_by_threads[thread_index(64)] &&
+        if (chunk_bytes / (uint64_t)s <= lines_piece && (double)(s * ntbs) <= lines_most && s * ntbs <= capacity_by_threads[thread_index(64)] &&
             most_msgs < (1 << 22) - 1) {
           slices = s;
           lines = true;
-        } else if (depth_of_dataflow >= 12 && chunk_bytes / (uint64_t)slices <= 4096 && (double)(slices * ntbs) <= ratio * 0.25 * (double)num_cus &&
+        } else if (depth_of_dataflow >= 12 && chunk_bytes / (uint64_t)slices <= 8192 && (double)(slices * ntbs) <= ratio * 0.25 * (double)num_cus &&
                    slices * ntbs <= std::min<int64_t>(capacity_by_threads[thread_index(64)], (int64_t)num_cus * 16) &&   // a workgroup each
                    most_msgs < (1 << 22) - 1) {
           // A long chain in which hardly anything is busy at a time -- a quarter of the compute units at most -- is all
-          // hand-offs: the doubled slot traffic is free there, and lines win with pieces of up to 4 KiB too
-          // (64-rank reduce chain + broadcast chain on one 128 / 256 KiB chunk: 204 -> 154, 217 -> 171 us).
+          // hand-offs: the doubled slot traffic is free there, and lines win with pieces of up to 8 KiB too
+          // (64-rank reduce chain + broadcast chain on one 128 / 256 / 512 KiB chunk: 204 -> 154, 217 -> 171, 253 -> 143 us).
           lines = true;
         }
       }

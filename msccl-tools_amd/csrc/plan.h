@@ -199,7 +199,11 @@ MSCCLX_HOST_DEVICE inline uint64_t slice_begin(uint64_t chunk_units, uint32_t gr
 constexpr int kMaxHosted = 64;        // contexts per workgroup: one per lane of the polling wave
 constexpr int kProfTrace = 248;       // MSCCLX_PROFILE builds: moves logged per workgroup ...
 constexpr int kProfWords = 8 + kProfTrace;  // ... after its 8 words of totals
-constexpr int kLLUnitBytes = 32;       // a flag-in-data line pair: 16 bytes of payload in 32
+// A unit under the flag-in-data protocol: 16 bytes of payload travel as two 16-byte halves (word flag word flag), 32 bytes
+// in all.  A row of n units is laid out as the n first halves followed by the n second halves, so that each of the two
+// store instructions that write a row covers whole cache lines (unit by unit, each would write half of every 32 bytes:
+// twice the write transactions, and a step of a 64-rank ring 5 to 19 % longer).
+constexpr int kLLUnitBytes = 32;
 constexpr int kSyncStrideWords = 8;   // every counter sits alone in 64 bytes
 constexpr int kSyncHeaderWords = 8;   // word 0 of an area = abort flag
 // The control block in front of the two counter areas: word 2 = the stamp of the binding that armed the workspace, then

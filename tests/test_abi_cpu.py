@@ -250,7 +250,7 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
     for key, w in WORKLOADS.items():
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
-        assert i.protocol == binding.PROTOCOL_CODES["ll" if key in ("c5", "c5_chain") else "simple"], key
+        assert i.protocol == binding.PROTOCOL_CODES["ll" if key in ("c1", "c5", "c5_chain") else "simple"], key  # (c1: lines at four one-wave workgroups per compute unit)
 
 
 def test_wide_workgroups_for_cold_traffic(mscclx_lib):
