@@ -727,13 +727,19 @@ int decide_geometry(mscclx_plan& plan, size_t chunk_bytes, int dtype, const mscc
             most_msgs < (1 << 22) - 1) {
           slices = s;
           lines = true;
-        } else if (depth_of_dataflow >= 12 && chunk_bytes / (uint64_t)slices <= 8192 && (double)(slices * ntbs) <= ratio * 0.25 * (double)num_cus &&
-                   slices * ntbs <= std::min<int64_t>(capacity_by_threads[thread_index(64)], (int64_t)num_cus * 16) &&   // a workgroup each
-                   most_msgs < (1 << 22) - 1) {
+        } else if (depth_of_dataflow >= 12 && most_msgs < (1 << 22) - 1) {
           // A long chain in which hardly anything is busy at a time -- a quarter of the compute units at most -- is all
-          // hand-offs: the doubled slot traffic is free there, and lines win with pieces of up to 8 KiB too
+          // hand-offs: the doubled slot traffic is free there, and lines win with pieces of up to 8 KiB too, on as many
+          // slices as still give every context a workgroup
           // (64-rank reduce chain + broadcast chain on one 128 / 256 / 512 KiB chunk: 204 -> 154, 217 -> 171, 253 -> 143 us).
-          lines = true;
+          const double few = std::min(ratio * 0.25 * (double)num_cus,
+                                      (double)std::min<int64_t>(capacity_by_threads[thread_index(64)], (int64_t)num_cus * 16));  // a workgroup each
+          int64_t fewer = slices;
+          while (fewer > 1 && (double)(fewer * ntbs) > few && chunk_bytes / (uint64_t)(fewer / 2) <= 8192) fewer /= 2;
+          if (chunk_bytes / (uint64_t)fewer <= 8192 && (double)(fewer * ntbs) <= few) {
+            slices = fewer;
+            lines = true;
+          }
         }
       }
     }
