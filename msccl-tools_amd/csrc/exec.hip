@@ -53,6 +53,7 @@ struct DeviceImage {
   bool one_each = false;              // workgroup w hosts context w and no other
   bool long_folds = false;            // some step stands for more folded nops than a lane checks by itself
   bool chain_fold = false;            // folded nops on one-wave workgroups with one context each: exec_kernel_chain_fold
+  bool flat = false;                  // the step table holds FlatOp records: every step's slots and flags worked out here
   std::vector<int32_t> dev_op_begin;  // per threadblock: its first step in the device's list ...
   std::vector<int32_t> dev_ir_step;   // ... and, per device step, the IR step it stands for (runs of nops are folded)
   kernel_fn kernel = nullptr;
@@ -153,6 +154,22 @@ static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<
   bytes.resize(off + n * sizeof(T), 0);
   if (!v.empty()) std::memcpy(bytes.data() + off, v.data(), v.size() * sizeof(T));
   return off;
+}
+
+// Whether a launch's step table can hold FlatOp records (plan.h): lines on one-wave workgroups, one pass, one row of at
+// most 64 whole units per step, and no step that waits for, or is waited for by, another threadblock of its rank.
+// (Not in profiling builds, whose clocks live in the general loop.)
+static bool flat_steps(const mscclx_plan& plan, const Geometry& g) {
+#ifdef MSCCLX_PROFILE
+  return false;
+#endif
+  if (!g.ll || !one_wave_each(g) || g.passes != 1 || g.piece_units > 64 || plan.chunk_bytes % 16 != 0) return false;
+  uint64_t most_slot = 0;
+  for (const Conn& c : plan.conns) most_slot = std::max<uint64_t>(most_slot, (uint64_t)c.max_cnt * g.piece_units * kLLUnitBytes);
+  if (most_slot * (uint64_t)g.depth > 0xffffffffull) return false;
+  for (const Op& op : plan.ops)
+    if (op.type == MSCCLX_OP_NOP || op.cnt != 1 || op.depid >= 0 || op.hasdep) return false;
+  return true;
 }
 
 // The device's tables for the configured geometry and these buffers.  Pure host work.
@@ -369,6 +386,34 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
       }
     }
   }
+  // Lines on one-wave workgroups, one pass, one row of at most 64 units per step, no waits between the threadblocks of a
+  // rank (the rings): which slot of its connections' rings a step uses, which flags it reads and writes, and what the
+  // counters must show are then the same in every launch, and the step table says so (FlatOp) -- the chain loop's
+  // bookkeeping, some hundred instructions per step of a lone wave, is done here instead, once.
+  d->flat = flat_steps(*plan, g);
+  for (size_t t = 0; d->flat && t < ntb; ++t) {
+    const uint64_t in_slot = htb[t].recv_conn >= 0 ? (uint64_t)hcn[(size_t)htb[t].recv_conn].slot_units * kLLUnitBytes : 0;
+    const uint64_t out_slot = htb[t].send_conn >= 0 ? (uint64_t)hcn[(size_t)htb[t].send_conn].slot_units * kLLUnitBytes : 0;
+    uint64_t rseq = 0, sseq = 0;
+    for (int32_t i = htb[t].op_begin; i < htb[t].op_begin + htb[t].nops; ++i) {
+      const DevOp dv = hop[(size_t)i];
+      const int type = (int)(dv.word & 15u);
+      FlatOp f{};
+      f.word = dv.word; f.src_addr = dv.src_addr; f.dst_addr = dv.dst_addr;
+      if (is_recv_type(type)) {
+        f.in_off = (uint32_t)((rseq % (uint64_t)g.depth) * in_slot);
+        f.fin = (uint32_t)((rseq + 1) & 0x3fffffu);
+        f.tail = ++rseq;
+      }
+      if (is_send_type(type)) {
+        f.out_off = (uint32_t)((sseq % (uint64_t)g.depth) * out_slot);
+        f.fout = (uint32_t)((sseq + 1) & 0x3fffffu);
+        f.gate = sseq >= (uint64_t)g.depth ? (uint32_t)(sseq + 1 - (uint64_t)g.depth) : 0u;
+        ++sseq;
+      }
+      std::memcpy(&hop[(size_t)i], &f, sizeof f);
+    }
+  }
   img->kernel = pick_kernel(plan->dtype, plan->redop, g.ll != 0, d->chain_fold ? 3 : fold ? (img->long_folds ? 2 : 1) : 0, plan->chunk_bytes % 16 != 0);
   if (!img->kernel) return fail(MSCCLX_ERR_UNSUPPORTED, "no kernel for this dtype/reduction");
   // One record per hosted context, in hosting order: where its counters and slots are, its slice's bounds.
@@ -460,6 +505,7 @@ static KernelParams make_params(const mscclx_plan& plan, const DeviceImage& img,
   kp.wg_begin = (const int32_t*)(tables + img.off_hosting);
   kp.ctxs = (const DevCtx*)(tables + img.off_ctxs);
   kp.one_each = img.one_each ? 1u : 0u;
+  kp.flat = img.flat ? 1u : 0u;
   return kp;
 }
 
@@ -580,7 +626,7 @@ int mscclx_plan_configure(mscclx_plan* plan, size_t chunk_bytes, int32_t dtype, 
     info->protocol = g.ll ? MSCCLX_PROTO_LL : MSCCLX_PROTO_SIMPLE;
     info->waiting_ratio_x100 = (int32_t)std::min(2.0e9, g.waiting_ratio * 100.0 + 0.5);
     info->dataflow_depth = g.dataflow_depth;
-    info->kernel_loop = !one_wave_each(g) ? MSCCLX_LOOP_HOSTED : g.ll ? MSCCLX_LOOP_CHAIN_LINES
+    info->kernel_loop = !one_wave_each(g) ? MSCCLX_LOOP_HOSTED : g.ll ? (flat_steps(*plan, g) ? MSCCLX_LOOP_CHAIN_LINES_FLAT : MSCCLX_LOOP_CHAIN_LINES)
                         : has_foldable_nops(*plan) ? MSCCLX_LOOP_CHAIN_FOLD : MSCCLX_LOOP_CHAIN_COUNTERS;
     info->cold_traffic_x100 = (int32_t)(g.cold_fraction * 100.0 + 0.5);
     info->threads = g.threads;

@@ -930,6 +930,43 @@ struct ChainWatch {
   int tb, slice;
 };
 
+// A step's table entry asked for ahead of time.  Scalar loads would bring it straight to scalar registers, but
+// they complete out of order, so the first wait for any scalar value -- a spilled register is enough -- waits
+// for the entry as well, and an entry is used once per pass: most of these loads miss the scalar cache.  Asked
+// for with vector loads (every lane the same address), the entry arrives behind the loads issued before it and
+// ahead of the lines that the wave polls for; twelve moves then carry it to scalar registers.
+struct StepAhead {
+  u32x4 a, b, c;  // a: word dep_tb dep_step dep_nops, b: extra steps src_addr, c: dst_addr in_addr
+};
+static_assert(offsetof(DevOp, extra) == 16 && offsetof(DevOp, dst_addr) == 32, "StepAhead names DevOp's fields by their place");
+__device__ __forceinline__ StepAhead ask_step(const __amdgpu_buffer_rsrc_t table, uint32_t index) {
+  StepAhead r;
+  const int at = (int)(index * (uint32_t)sizeof(DevOp));
+  r.a = Access<16>::template lds<0>(table, 0, at);
+  r.b = Access<16>::template lds<0>(table, 16, at);
+  r.c = Access<16>::template lds<0>(table, 32, at);
+  return r;
+}
+__device__ __forceinline__ DevOp take_step(const StepAhead& e) {
+  DevOp r;
+  r.word = uniform(e.a.x); r.dep_tb = (int32_t)uniform(e.a.y); r.dep_step = (int32_t)uniform(e.a.z); r.dep_nops = (int32_t)uniform(e.a.w);
+  r.extra = uniform(e.b.x); r.steps = uniform(e.b.y);
+  r.src_addr = (u64)uniform(e.b.z) | (u64)uniform(e.b.w) << 32;
+  r.dst_addr = (u64)uniform(e.c.x) | (u64)uniform(e.c.y) << 32;
+  r.in_addr = (u64)uniform(e.c.z) | (u64)uniform(e.c.w) << 32;
+  return r;
+}
+
+__device__ __forceinline__ FlatOp take_flat_step(const StepAhead& e) {
+  FlatOp r;
+  r.word = uniform(e.a.x); r.in_off = uniform(e.a.y); r.out_off = uniform(e.a.z); r.fin = uniform(e.a.w);
+  r.fout = uniform(e.b.x); r.gate = uniform(e.b.y);
+  r.src_addr = (u64)uniform(e.b.z) | (u64)uniform(e.b.w) << 32;
+  r.dst_addr = (u64)uniform(e.c.x) | (u64)uniform(e.c.y) << 32;
+  r.tail = (u64)uniform(e.c.z);  // (message numbers stay below 2^22)
+  return r;
+}
+
 // One round of a step of run_chain: units i0, i0 + 64, ... (U of them per lane) of one row of n units.
 // Returns false when the launch is lost (the same answer in all lanes).  gate: the counter that must
 // reach gate_target before the outgoing slot may be written, or null.  The polling is uniform: all
@@ -939,7 +976,8 @@ template <class R, int U, int T>
 __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, const __amdgpu_buffer_rsrc_t rin2, const __amdgpu_buffer_rsrc_t rout,
                                             const __amdgpu_buffer_rsrc_t rout2, const __amdgpu_buffer_rsrc_t rsrc, const __amdgpu_buffer_rsrc_t rdst, const uint32_t i0, const uint32_t n, const bool nt, const uint32_t fin,
                                             const uint32_t fout, const u64* gate, const u64 gate_target, const ChainWatch& watch, const int step,
-                                            const uint32_t pass, u64* prof_acc, u64& prof_mark, const u64 prof_floor) {
+                                            const uint32_t pass, const __amdgpu_buffer_rsrc_t table, const uint32_t ask_index, StepAhead& asked, u64* prof_acc,
+                                            u64& prof_mark, const u64 prof_floor) {
   // what a step of type T does, known where the code is generated: one straight run of instructions per type
   constexpr bool rcv = ((0x7cu >> T) & 1u) != 0, snd = ((0x5au >> T) & 1u) != 0;
   constexpr bool from_src = T == MSCCLX_OP_SEND || T == MSCCLX_OP_COPY || T == MSCCLX_OP_REDUCE;
@@ -968,6 +1006,11 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
     for (int u = 0; u < U; ++u) y[u] = A::template ld<XL>(rdst, (int)((i0 + 64u * (uint32_t)u) * 16));
   }
   u64 gate_seen = snd && gate ? load_counter(gate) : ~0ull;
+  // The table entry of a step further on is asked for here, behind the step's own loads: answers come back in the order of
+  // the requests, so the wait for the lines leaves this request outstanding, and it has the whole step to arrive.  (Asked
+  // for in front of the lines, the first look at them waited for the entry as well -- an entry is read once per pass,
+  // and every third one comes from memory.)
+  if (ask_index != ~0u) asked = ask_step(table, ask_index);
   bool lost = false;
   if constexpr (rcv) {
     auto all_there = [&]() {
@@ -1070,8 +1113,9 @@ template <class R, int T>
 __device__ __forceinline__ bool chain_rows(const unsigned char* in_row, unsigned char* out_row, u64 src_row, u64 dst_row, const u64 row_stride,
                                            const uint32_t cnt, const uint32_t n, const uint32_t row_line_bytes, const uint32_t local_bytes,
                                            const uint32_t lane, const bool nt, const uint32_t fin, const uint32_t fout, const u64* gate,
-                                           const u64 gate_target, const ChainWatch& watch, const int step, const uint32_t pass, u64* prof_acc,
-                                           u64& prof_mark, const u64 prof_floor) {
+                                           const u64 gate_target, const ChainWatch& watch, const int step, const uint32_t pass,
+                                           const __amdgpu_buffer_rsrc_t table, uint32_t ask_index, StepAhead& asked, u64* prof_acc, u64& prof_mark,
+                                           const u64 prof_floor) {
   for (uint32_t row = 0; row < cnt; ++row) {
     // (a row of lines: the first halves of its n units, then the second halves; a descriptor for each)
     const uint32_t half = row_line_bytes >> 1;
@@ -1079,49 +1123,24 @@ __device__ __forceinline__ bool chain_rows(const unsigned char* in_row, unsigned
     const __amdgpu_buffer_rsrc_t rout = make_rsrc(out_row, half), rout2 = make_rsrc(out_row + half, half);
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)src_row, local_bytes), rdst = make_rsrc((const void*)dst_row, local_bytes);
     if (n <= 64) {  // the shape of the smallest messages: one unit per lane, half the instructions
-      if (!chain_round<R, 1, T>(rin, rin2, rout, rout2, rsrc, rdst, lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark,
-                                prof_floor))
+      if (!chain_round<R, 1, T>(rin, rin2, rout, rout2, rsrc, rdst, lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, table, ask_index, asked,
+                                prof_acc, prof_mark, prof_floor))
         return false;
       gate = nullptr;
+      ask_index = ~0u;  // (the step's first round has asked)
     } else {
       for (uint32_t base = 0; base < n; base += 128) {
-        if (!chain_round<R, 2, T>(rin, rin2, rout, rout2, rsrc, rdst, base + lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, prof_acc, prof_mark,
-                                  prof_floor))
+        if (!chain_round<R, 2, T>(rin, rin2, rout, rout2, rsrc, rdst, base + lane, n, nt, fin, fout, gate, gate_target, watch, step, pass, table, ask_index,
+                                  asked, prof_acc, prof_mark, prof_floor))
           return false;
         gate = nullptr;
+        ask_index = ~0u;
       }
     }
     in_row += row_line_bytes; out_row += row_line_bytes;
     src_row += row_stride; dst_row += row_stride;
   }
   return true;
-}
-
-// A step's table entry asked for ahead of time.  Scalar loads would bring it straight to scalar registers, but
-// they complete out of order, so the first wait for any scalar value -- a spilled register is enough -- waits
-// for the entry as well, and an entry is used once per pass: most of these loads miss the scalar cache.  Asked
-// for with vector loads (every lane the same address), the entry arrives behind the loads issued before it and
-// ahead of the lines that the wave polls for; twelve moves then carry it to scalar registers.
-struct StepAhead {
-  u32x4 a, b, c;  // a: word dep_tb dep_step dep_nops, b: extra steps src_addr, c: dst_addr in_addr
-};
-static_assert(offsetof(DevOp, extra) == 16 && offsetof(DevOp, dst_addr) == 32, "StepAhead names DevOp's fields by their place");
-__device__ __forceinline__ StepAhead ask_step(const __amdgpu_buffer_rsrc_t table, uint32_t index) {
-  StepAhead r;
-  const int at = (int)(index * (uint32_t)sizeof(DevOp));
-  r.a = Access<16>::template lds<0>(table, 0, at);
-  r.b = Access<16>::template lds<0>(table, 16, at);
-  r.c = Access<16>::template lds<0>(table, 32, at);
-  return r;
-}
-__device__ __forceinline__ DevOp take_step(const StepAhead& e) {
-  DevOp r;
-  r.word = uniform(e.a.x); r.dep_tb = (int32_t)uniform(e.a.y); r.dep_step = (int32_t)uniform(e.a.z); r.dep_nops = (int32_t)uniform(e.a.w);
-  r.extra = uniform(e.b.x); r.steps = uniform(e.b.y);
-  r.src_addr = (u64)uniform(e.b.z) | (u64)uniform(e.b.w) << 32;
-  r.dst_addr = (u64)uniform(e.c.x) | (u64)uniform(e.c.y) << 32;
-  r.in_addr = (u64)uniform(e.c.z) | (u64)uniform(e.c.w) << 32;
-  return r;
 }
 
 // (prof_acc, profiling builds only: fine-clock ticks spent 0 waiting for a dependency, 1 from the first
@@ -1161,8 +1180,15 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
 #ifdef MSCCLX_PROFILE
   prof_mark = prof_begin;
 #endif
+  // The table is read two steps ahead: the entry of the step after this one arrived while the step before ran; the entry
+  // of the step after that is asked for behind this step's own loads (chain_round says why there).
+  StepAhead after = ask_step(table, nops > 1 ? 1u : 0u);
   for (;;) {
-    const StepAhead after = ask_step(table, step + 1 == nops ? 0 : step + 1);  // (it arrives while the wave waits)
+    uint32_t second = step + 2;
+    second = second >= nops ? second - nops : second;
+    second = second >= nops ? 0u : second;  // (a table of one step)
+    StepAhead after_that;
+    after_that.a = after_that.b = after_that.c = u32x4{0, 0, 0, 0};
     MSCCLX_CHAIN_CLOCK(prof_dep0);
     const int t = (int)(op.word & 15u);
     const uint32_t cnt = op.word >> kOpCntShift;
@@ -1200,7 +1226,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
 #define MSCCLX_CHAIN_CASE(T)                                                                                                                                     \
   case T:                                                                                                                                                        \
     ok = chain_rows<R, T>(in_ring + rslot, out_ring + sslot, op.src_addr + off, op.dst_addr + off, row_stride, cnt, n, row_line_bytes, local_bytes, lane, nt, fin, \
-                          fout, gate, gate_target, watch, (int)step, pass, prof_acc, prof_mark, prof_floor);                                                    \
+                          fout, gate, gate_target, watch, (int)step, pass, table, second, after_that, prof_acc, prof_mark, prof_floor);                         \
     break
     switch (t) {  // (one copy of the step's instructions per type, with nothing left to decide inside)
       MSCCLX_CHAIN_CASE(MSCCLX_OP_SEND);
@@ -1211,7 +1237,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       MSCCLX_CHAIN_CASE(MSCCLX_OP_RRCS);
       MSCCLX_CHAIN_CASE(MSCCLX_OP_COPY);
       MSCCLX_CHAIN_CASE(MSCCLX_OP_REDUCE);
-      default: break;  // nop
+      default: after_that = ask_step(table, second); break;  // nop
     }
 #undef MSCCLX_CHAIN_CASE
     if (!ok) return;
@@ -1243,10 +1269,81 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
     }
     if (rcv && writer) publish(in_tail, (u64)rseq);
     op = take_step(after);
+    after = after_that;
   }
 #ifdef MSCCLX_PROFILE
   prof_acc[4] = __builtin_amdgcn_s_memtime() - prof_begin;
 #endif
+}
+
+// run_chain for a launch whose step table holds FlatOp records (plan.h): one pass, one row of at most 64 units per step,
+// no waits between the threadblocks of a rank, and every step's slots, flags and counter values worked out when the
+// buffers were bound.  What is left per step is its one round and the request for the step after.
+template <class R>
+__device__ __forceinline__ void run_chain_flat(const KernelParams& p, uint32_t epoch, int ctx) {
+  const uint32_t lane = threadIdx.x;
+  const bool writer = lane == 0;
+  const DevCtx rec = p.ctxs[ctx];
+  const Hosted h = rec.h;
+  if (writer) {  // (as init_context: this context's counters in the area of the launch after this one)
+    p.sync_nxt[h.my_flag] = 0;
+    if (h.head_out) p.sync_nxt[h.head_out] = 0;
+    if (h.tail_out) p.sync_nxt[h.tail_out] = 0;
+  }
+  const uint32_t nops = (uint32_t)uniform(h.nops);
+  if (nops == 0 || uniform(h.npasses) == 0) return;
+  const uint32_t n = uniform(rec.left);  // the units of this context's one piece
+  const u64 off = uniform((uint64_t)rec.off);
+  const unsigned char* const in_ring = p.fifo + (u64)uniform(h.in_slots) * 16;
+  unsigned char* const out_ring = p.fifo + (u64)uniform(h.out_slots) * 16;
+  const u64* const out_tail = p.sync_cur + uniform(h.tail_in);
+  u64* const in_tail = p.sync_cur + uniform(h.tail_out);
+  const ChainWatch watch{p.sync_cur, p.host_status, p.timeout_ticks, uniform(h.tb), uniform(h.slice)};
+  const uint32_t flag_high = (epoch & 0x3ffu) << 22, half = n * 16;
+  const __amdgpu_buffer_rsrc_t table = make_rsrc(p.ops + uniform(h.op_begin), nops * (uint32_t)sizeof(DevOp));
+  FlatOp op = take_flat_step(ask_step(table, 0));
+  StepAhead after = ask_step(table, nops > 1 ? 1u : 0u);  // (the table is read two steps ahead, as in run_chain)
+  u64 no_clock = 0;
+  for (uint32_t step = 0;;) {
+    uint32_t second = step + 2;
+    second = second >= nops ? second - nops : second;
+    second = second >= nops ? 0u : second;
+    StepAhead after_that;
+    after_that.a = after_that.b = after_that.c = u32x4{0, 0, 0, 0};
+    if (__builtin_expect((step & 0x3fu) == 0x3fu, 0) && uniform((uint64_t)load_counter(watch.abort_word)) != 0) {  // a host's abort request, a lost launch
+      note_abort(watch.abort_word, watch.host_status);
+      return;
+    }
+    const uint32_t t = op.word & 15u;
+    const bool nt = (op.word & kOpNtStore) != 0;
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in_ring + op.in_off, half), rin2 = make_rsrc(in_ring + op.in_off + half, half);
+    const __amdgpu_buffer_rsrc_t rout = make_rsrc(out_ring + op.out_off, half), rout2 = make_rsrc(out_ring + op.out_off + half, half);
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc((const void*)(op.src_addr + off), half), rdst = make_rsrc((const void*)(op.dst_addr + off), half);
+    const u64* const gate = op.gate ? out_tail : nullptr;
+    bool ok = true;
+#define MSCCLX_FLAT_CASE(T)                                                                                                                                  \
+  case T:                                                                                                                                                    \
+    ok = chain_round<R, 1, T>(rin, rin2, rout, rout2, rsrc, rdst, lane, n, nt, flag_high | op.fin, flag_high | op.fout, gate, (u64)op.gate, watch, (int)step, 0u, \
+                              table, second, after_that, nullptr, no_clock, 0);                                                                              \
+    break
+    switch (t) {
+      MSCCLX_FLAT_CASE(MSCCLX_OP_SEND);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_RECV);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_RCS);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_RRS);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_RRC);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_RRCS);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_COPY);
+      MSCCLX_FLAT_CASE(MSCCLX_OP_REDUCE);
+      default: break;
+    }
+#undef MSCCLX_FLAT_CASE
+    if (!ok) return;
+    if (op.tail && writer) publish(in_tail, op.tail);
+    if (++step == nops) break;
+    op = take_flat_step(after);
+    after = after_that;
+  }
 }
 
 // One round of a step of run_chain_counters: units i0, i0 + 64, ... (U per lane) of one row of n
@@ -1497,7 +1594,10 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
     prof_fin = chain_acc[0]; prof_wait = chain_acc[1]; prof_move = chain_acc[2]; prof_ack = chain_acc[3];
     if (threadIdx.x == 0 && p.prof) p.prof[(size_t)blockIdx.x * kProfWords + 8] = chain_acc[4];
 #else
-    if constexpr (LL) run_chain<R, RAGGED>(p, epoch, ctx_begin);
+    if constexpr (LL) {
+      if (!RAGGED && p.flat) run_chain_flat<R>(p, epoch, ctx_begin);
+      else run_chain<R, RAGGED>(p, epoch, ctx_begin);
+    }
 #endif
   } else if (!LL && !FOLD && hosted == 1 && blockDim.x == 64) {
 #ifdef MSCCLX_PROFILE

@@ -1,5 +1,6 @@
 // Internal host/device structures of the MSCCL-IR executor (not part of the C ABI).
 #pragma once
+#include <cstddef>
 #include <cstdint>
 #include <string>
 #include <vector>
@@ -68,6 +69,22 @@ struct DevOp {
   uint64_t in_addr;          // in_place: the chunk of the sending rank's buffer that holds the payload
 };
 static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
+// The same 48 bytes for a launch whose every step's place in its connections' rings is known when buffers are bound
+// (flag-in-data lines on one-wave workgroups, one pass, one row of at most 64 units per step, no step that waits for or is
+// waited for by another threadblock of its rank: KernelParams::flat).  The device then works nothing out per step:
+struct FlatOp {
+  uint32_t word;          // as DevOp::word
+  uint32_t in_off;        // byte offset of the step's slot in the incoming connection's ring (receiving steps)
+  uint32_t out_off;       // the same for the outgoing connection (sending steps)
+  uint32_t fin;           // low 22 bits of the flag its incoming lines carry
+  uint32_t fout;          // ... and of the flag it writes
+  uint32_t gate;          // what the outgoing connection's tail must have reached before the slot may be written; 0: nothing
+  uint64_t src_addr;      // as DevOp
+  uint64_t dst_addr;
+  uint64_t tail;          // what the incoming connection's tail reads once this step has its lines (receiving steps)
+};
+static_assert(sizeof(FlatOp) == sizeof(DevOp) && offsetof(FlatOp, src_addr) == offsetof(DevOp, src_addr) && offsetof(FlatOp, dst_addr) == offsetof(DevOp, dst_addr),
+              "a flat step lies where the step it was made from lay");
 constexpr uint32_t kOpHasdep = 1u << 4, kOpOutStaged = 1u << 5, kOpNtStore = 1u << 6, kOpInPlace = 1u << 7;
 constexpr int kOpCntShift = 8;
 // Bit 31 of DevOp::steps, on a receive that reads its payload in place: the matching send is the first step of its
@@ -181,6 +198,7 @@ struct KernelParams {
   const int32_t* wg_begin;      // [workgroups+1] first hosted context of each workgroup
   const DevCtx* ctxs;           // hosted contexts, grouped by workgroup
   uint32_t one_each;            // 1: workgroup w hosts context w and no other (wg_begin need not be read)
+  uint32_t flat;                // 1: the step table holds FlatOp records (see there)
 };
 
 #ifdef __HIPCC__

@@ -24,7 +24,7 @@ DTYPE_CODES = {"uint8": 0, "int8": 1, "int32": 2, "uint32": 3, "int64": 4, "uint
 DTYPE_SIZES = {"uint8": 1, "int8": 1, "int32": 4, "uint32": 4, "int64": 8, "uint64": 8,
                "float16": 2, "bfloat16": 2, "float32": 4, "float64": 8}
 REDOP_CODES = {"sum": 0, "prod": 1, "max": 2, "min": 3}
-LOOP_NAMES = {0: "hosted", 1: "chain, lines", 2: "chain, counters", 3: "chain, folded nops"}  # mscclx_loop
+LOOP_NAMES = {0: "hosted", 1: "chain, lines", 2: "chain, counters", 3: "chain, folded nops", 4: "chain, lines, steps worked out at bind"}  # mscclx_loop
 PROTOCOL_CODES = {"auto": 0, "simple": 1, "ll": 2, "Simple": 1, "LL": 2}
 
 # every symbol include/mscclx.h declares
