@@ -160,7 +160,7 @@ static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<
 // most 64 whole units per step, and no step that waits for, or is waited for by, another threadblock of its rank.
 // (Not in profiling builds, whose clocks live in the general loop.)
 static bool flat_steps(const mscclx_plan& plan, const Geometry& g) {
-#ifdef MSCCLX_PROFILE
+#if defined(MSCCLX_PROFILE) || defined(MSCCLX_EXP_NO_FLAT)
   return false;
 #endif
   if (!g.ll || !one_wave_each(g) || g.passes != 1 || g.piece_units > 64 || plan.chunk_bytes % 16 != 0) return false;

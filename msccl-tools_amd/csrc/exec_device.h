@@ -1006,10 +1006,10 @@ __device__ __forceinline__ bool chain_round(const __amdgpu_buffer_rsrc_t rin, co
     for (int u = 0; u < U; ++u) y[u] = A::template ld<XL>(rdst, (int)((i0 + 64u * (uint32_t)u) * 16));
   }
   u64 gate_seen = snd && gate ? load_counter(gate) : ~0ull;
-  // The table entry of a step further on is asked for here, behind the step's own loads: answers come back in the order of
-  // the requests, so the wait for the lines leaves this request outstanding, and it has the whole step to arrive.  (Asked
-  // for in front of the lines, the first look at them waited for the entry as well -- an entry is read once per pass,
-  // and every third one comes from memory.)
+  // run_chain_flat asks for the table entry of the step after next here, behind the step's own loads: answers come back in
+  // the order of the requests, so the wait for the lines leaves this request outstanding, and it has a whole step to arrive.
+  // (That loop measured 188 us on the 64-rank ring with the request at its top, one step ahead, and 147 with it here; the
+  // general loop 178 at its top and 206 here.  Each keeps what it measured best with.)
   if (ask_index != ~0u) asked = ask_step(table, ask_index);
   bool lost = false;
   if constexpr (rcv) {
@@ -1180,15 +1180,9 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
 #ifdef MSCCLX_PROFILE
   prof_mark = prof_begin;
 #endif
-  // The table is read two steps ahead: the entry of the step after this one arrived while the step before ran; the entry
-  // of the step after that is asked for behind this step's own loads (chain_round says why there).
-  StepAhead after = ask_step(table, nops > 1 ? 1u : 0u);
   for (;;) {
-    uint32_t second = step + 2;
-    second = second >= nops ? second - nops : second;
-    second = second >= nops ? 0u : second;  // (a table of one step)
-    StepAhead after_that;
-    after_that.a = after_that.b = after_that.c = u32x4{0, 0, 0, 0};
+    const StepAhead after = ask_step(table, step + 1 == nops ? 0 : step + 1);  // (it arrives while the wave waits)
+    StepAhead not_asked;  // (only run_chain_flat asks from inside a round: measured, each loop as it runs fastest)
     MSCCLX_CHAIN_CLOCK(prof_dep0);
     const int t = (int)(op.word & 15u);
     const uint32_t cnt = op.word >> kOpCntShift;
@@ -1226,7 +1220,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
 #define MSCCLX_CHAIN_CASE(T)                                                                                                                                     \
   case T:                                                                                                                                                        \
     ok = chain_rows<R, T>(in_ring + rslot, out_ring + sslot, op.src_addr + off, op.dst_addr + off, row_stride, cnt, n, row_line_bytes, local_bytes, lane, nt, fin, \
-                          fout, gate, gate_target, watch, (int)step, pass, table, second, after_that, prof_acc, prof_mark, prof_floor);                         \
+                          fout, gate, gate_target, watch, (int)step, pass, table, ~0u, not_asked, prof_acc, prof_mark, prof_floor);                             \
     break
     switch (t) {  // (one copy of the step's instructions per type, with nothing left to decide inside)
       MSCCLX_CHAIN_CASE(MSCCLX_OP_SEND);
@@ -1237,7 +1231,7 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
       MSCCLX_CHAIN_CASE(MSCCLX_OP_RRCS);
       MSCCLX_CHAIN_CASE(MSCCLX_OP_COPY);
       MSCCLX_CHAIN_CASE(MSCCLX_OP_REDUCE);
-      default: after_that = ask_step(table, second); break;  // nop
+      default: break;  // nop
     }
 #undef MSCCLX_CHAIN_CASE
     if (!ok) return;
@@ -1269,7 +1263,6 @@ __device__ __forceinline__ void run_chain(const KernelParams& p, uint32_t epoch,
     }
     if (rcv && writer) publish(in_tail, (u64)rseq);
     op = take_step(after);
-    after = after_that;
   }
 #ifdef MSCCLX_PROFILE
   prof_acc[4] = __builtin_amdgcn_s_memtime() - prof_begin;
