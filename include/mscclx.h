@@ -86,7 +86,7 @@ typedef enum { MSCCLX_PROTO_AUTO = 0, MSCCLX_PROTO_SIMPLE = 1, MSCCLX_PROTO_LL =
  * FOLD for counters in programs whose nop steps are folded into the steps behind them (msccl/language/ir.py:296-311
  * gives a step one dependency and puts a nop in front of it for every other: the all-pairs family); LINES_FLAT for lines
  * where every step's slots, flags and counter values could be worked out when the buffers were bound (one pass, one row
- * of at most 64 units per step, no waits between the threadblocks of a rank: the rings on small messages). */
+ * of at most 128 units per step, no waits between the threadblocks of a rank: the rings on small messages). */
 typedef enum { MSCCLX_LOOP_HOSTED = 0, MSCCLX_LOOP_CHAIN_LINES = 1, MSCCLX_LOOP_CHAIN_COUNTERS = 2, MSCCLX_LOOP_CHAIN_FOLD = 3, MSCCLX_LOOP_CHAIN_LINES_FLAT = 4 } mscclx_loop;
 
 typedef enum { MSCCLX_SUM = 0, MSCCLX_PROD = 1, MSCCLX_MAX = 2, MSCCLX_MIN = 3, MSCCLX_NUM_REDOPS = 4 } mscclx_redop;

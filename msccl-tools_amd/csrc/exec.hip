@@ -157,13 +157,13 @@ static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<
 }
 
 // Whether a launch's step table can hold FlatOp records (plan.h): lines on one-wave workgroups, one pass, one row of at
-// most 64 whole units per step, and no step that waits for, or is waited for by, another threadblock of its rank.
+// most 128 whole units per step, and no step that waits for, or is waited for by, another threadblock of its rank.
 // (Not in profiling builds, whose clocks live in the general loop.)
 static bool flat_steps(const mscclx_plan& plan, const Geometry& g) {
 #if defined(MSCCLX_PROFILE) || defined(MSCCLX_EXP_NO_FLAT)
   return false;
 #endif
-  if (!g.ll || !one_wave_each(g) || g.passes != 1 || g.piece_units > 64 || plan.chunk_bytes % 16 != 0) return false;
+  if (!g.ll || !one_wave_each(g) || g.passes != 1 || g.piece_units > 128 || plan.chunk_bytes % 16 != 0) return false;
   uint64_t most_slot = 0;
   for (const Conn& c : plan.conns) most_slot = std::max<uint64_t>(most_slot, (uint64_t)c.max_cnt * g.piece_units * kLLUnitBytes);
   if (most_slot * (uint64_t)g.depth > 0xffffffffull) return false;
@@ -386,7 +386,7 @@ static int build_image(const mscclx_plan& plan_ref, const std::vector<void*>& bu
       }
     }
   }
-  // Lines on one-wave workgroups, one pass, one row of at most 64 units per step, no waits between the threadblocks of a
+  // Lines on one-wave workgroups, one pass, one row of at most 128 units per step, no waits between the threadblocks of a
   // rank (the rings): which slot of its connections' rings a step uses, which flags it reads and writes, and what the
   // counters must show are then the same in every launch, and the step table says so (FlatOp) -- the chain loop's
   // bookkeeping, some hundred instructions per step of a lone wave, is done here instead, once.

@@ -70,7 +70,7 @@ struct DevOp {
 };
 static_assert(sizeof(DevOp) == 48, "three 16-byte loads fetch a step");
 // The same 48 bytes for a launch whose every step's place in its connections' rings is known when buffers are bound
-// (flag-in-data lines on one-wave workgroups, one pass, one row of at most 64 units per step, no step that waits for or is
+// (flag-in-data lines on one-wave workgroups, one pass, one row of at most 128 units per step, no step that waits for or is
 // waited for by another threadblock of its rank: KernelParams::flat).  The device then works nothing out per step:
 struct FlatOp {
   uint32_t word;          // as DevOp::word

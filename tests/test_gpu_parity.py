@@ -746,7 +746,7 @@ def test_ll_launch_number_wraps(knobs):
 def test_which_step_loop_runs():
     """mscclx_info.kernel_loop: the all-pairs family on small messages -- programs with folded nops, one-wave workgroups, one
     context each -- runs on exec_kernel_chain_fold (3); rings on the chain loops for counters (2) and for lines: with every
-    step's slots and flags worked out at bind where a step is one row of at most 64 units in one pass (4), the general loop
+    step's slots and flags worked out at bind where a step is one row of at most 128 units in one pass (4), the general loop
     for lines where a slice takes several passes (1); a geometry that hosts several contexts on a workgroup on the hosting
     loop (0).  Every one bit-exact against the interpreter."""
     allpairs = golden_util.load("allreduce_a100_allpairs_8r")   # (as msccl-tools' compiler wrote it: runs of nops in front of the folds and the sends)
