@@ -251,6 +251,10 @@ def test_geometry_of_the_benchmark_workloads(mscclx_lib):
         i = Plan(parse_algo_xml(w.build())).configure(w.chunk_bytes, w.dtype, max_workgroups=4096)
         assert (i.workgroups, i.threads, i.slices, i.piece_bytes, i.passes, i.max_hosted) == want[key], key
         assert i.protocol == binding.PROTOCOL_CODES["ll" if key in ("c1", "c5", "c5_chain") else "simple"], key  # (c1: lines at four one-wave workgroups per compute unit)
+        # which step loop they run: the rings on lines have their steps worked out at bind (one pass, one row of at most 128 units per
+        # step, no waits between a rank's threadblocks); the chain's rows of 256 units take the general loop for lines; the others host
+        loop = {"c1": 4, "c5": 4, "c5_chain": 1}.get(key, 0)
+        assert i.kernel_loop == loop, (key, i.kernel_loop, binding.LOOP_NAMES[i.kernel_loop])
 
 
 def test_wide_workgroups_for_cold_traffic(mscclx_lib):
