@@ -760,6 +760,90 @@ def test_which_step_loop_runs():
         assert_same(got, ref)
 
 
+@pytest.mark.parametrize("elems,slices", [(4, 1), (68, 1), (256, 1), (260, 1), (400, 1), (512, 1), (4096, 8), (4100, 8), (3000, 4), (8192, 32)])
+def test_steps_worked_out_at_bind(elems, slices):
+    """Rings on flag-in-data lines whose every step is one row of at most 128 units in one pass run with their steps' slots,
+    flags and counter values worked out when the buffers are bound (mscclx_info.kernel_loop 4).  Rows of 1 to 128 units, one
+    and two units per lane, slices of unequal length, connections whose ring of slots wraps many times (8, 16 and 64 ranks,
+    up to 126 messages through two slots), all element widths that lines carry; launched three times on one binding (the
+    flags carry the launch number); every byte against the interpreter."""
+    from msccl.executor import Executor, collective_buffers, DTYPE_SIZES
+    for xml, dtype in ((ir_samples.ring_allreduce_xml(8), "float32"), (golden_util.load("c5_allreduce_ring_64r_1ch_1inst"), "float16"),
+                       (golden_util.load("c2_allgather_ring_8r_1ch_4inst"), "int32"), (golden_util.load("reducescatter_ring_8r_1ch_4inst"), "float64")):
+        if elems * DTYPE_SIZES[dtype] % 16:
+            continue  # (chunks that end inside a unit run on the general loop: covered elsewhere)
+        got, ref, ex, info = run_both(xml, elems, dtype, seed=elems + slices, protocol="ll", slices=slices, threads=64)
+        flat = info.passes == 1 and info.piece_bytes <= 2048 and info.max_hosted == 1  # (wider elements make longer rows: those take the general loop)
+        assert info.kernel_loop == (4 if flat else 1 if info.max_hosted == 1 else 0), (info.kernel_loop, info.piece_bytes, info.passes, info.max_hosted)
+        assert_same(got, ref)
+    # the same binding launched again and again: an all-gather leaves its inputs alone, so every launch must leave the same bytes
+    xml = golden_util.load("c2_allgather_ring_8r_1ch_4inst")
+    algo = oi.parse_xml(xml)
+    x = make_inputs(algo.ngpus, algo.gpus[0].o_chunks * elems // algo.ngpus, "int32", 5)
+    ex = Executor(xml)
+    info = ex.setup(elems * 4, "int32", protocol="ll", slices=slices, threads=64)
+    ins, outs, res = collective_buffers(ex.tables, elems * 4, "int32", inputs=[to_torch(v, "int32") for v in x])
+    ex.bind(ins, outs)
+    want = np.concatenate(x)
+    for launch in range(3):
+        for r in range(algo.ngpus):
+            others = torch.ones_like(res[r]) * 7
+            others[r * x[r].size:(r + 1) * x[r].size] = res[r][r * x[r].size:(r + 1) * x[r].size]
+            res[r].copy_(others)  # (everything but the rank's own contribution overwritten before each launch)
+        ex.launch()
+        ex.wait()
+        for r in range(algo.ngpus):
+            assert np.array_equal(to_numpy(res[r], "int32"), want), (launch, r)
+
+
+def test_watchdog_and_abort_where_steps_are_worked_out_at_bind():
+    """The loop for steps worked out at bind carries the watchdog and sees the host's abort like the others: rank 1's
+    receive of one 2 KiB row waits while rank 0 makes 20 000 local copies of it first (tens of milliseconds) -- with a
+    1 ms limit it gives up cleanly and names the step; with the default limit and an abort from the host the launch ends
+    early with ABORTED; left alone it delivers."""
+    import time
+    from msccl.executor import Executor, MscclxError, collective_buffers
+    from msccl.executor.binding import ERR_ABORTED
+    xml = ir_samples.slow_producer_xml(20000)
+    nbytes = 2048
+    x = [torch.arange(nbytes, dtype=torch.int32).to(torch.uint8), torch.zeros(nbytes, dtype=torch.uint8)]
+    ex = Executor(xml)
+    info = ex.setup(nbytes, "uint8", timeout_ms=1, protocol="ll", slices=1, threads=64)
+    assert info.kernel_loop == 4 and info.workgroups == 2
+    ins, outs, _ = collective_buffers(ex.tables, nbytes, "uint8", inputs=x)
+    ex.bind(ins, outs)
+    print("case: watchdog where steps are worked out at bind", flush=True)
+    ex.launch()
+    with pytest.raises(MscclxError) as e:
+        ex.wait()
+    assert "watchdog" in str(e.value) and "rank 1 tb 0 step 0" in str(e.value) and "incoming message" in str(e.value)
+    torch.cuda.synchronize()
+    ex2 = Executor(xml)
+    assert ex2.setup(nbytes, "uint8", protocol="ll", slices=1, threads=64).kernel_loop == 4
+    ins, outs, _ = collective_buffers(ex2.tables, nbytes, "uint8", inputs=x)
+    ex2.bind(ins, outs)
+    print("case: full run for reference", flush=True)
+    t0 = time.perf_counter()
+    ex2.launch()
+    ex2.wait()
+    full = time.perf_counter() - t0
+    assert torch.equal(outs[1].cpu(), x[0])
+    outs[1].zero_()
+    print("case: abort from the host", flush=True)
+    ex2.launch()
+    time.sleep(full / 20)
+    ex2.abort()
+    t0 = time.perf_counter()
+    with pytest.raises(MscclxError) as e:
+        ex2.wait()
+    assert e.value.code == ERR_ABORTED
+    assert time.perf_counter() - t0 < full / 2
+    print("case: the same binding after the abort", flush=True)
+    ex2.launch()
+    ex2.wait()
+    assert torch.equal(outs[1].cpu(), x[0])
+
+
 def test_receives_that_take_over_their_senders_waits():
     """In exec_kernel_chain_fold a receive whose payload is read in place waits for its sender's dependencies itself instead
     of for the sender's announcement.  Programs in which such sends have dependencies of every kind -- their own, folded
