@@ -819,8 +819,8 @@ __device__ __forceinline__ void finish_step(Context& c, const Hosted& entry, con
 // bound), its state in `c`, standing at its first step.  `writer` also clears, for the next launch,
 // the counters this context alone writes.
 template <bool LL, bool RAGGED>
-__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int ctx, bool writer) {
-  const DevCtx rec = p.ctxs[ctx];
+__device__ __forceinline__ void init_context(Hosted& h, Context& c, const KernelParams& p, uint32_t epoch, int ctx, bool writer, const DevCtx* given = nullptr) {
+  const DevCtx rec = given ? *given : p.ctxs[ctx];  // (given: a record that the caller asked for earlier)
   h = rec.h;
   c.step = 0; c.pass = 0; c.count = 0; c.sseq = c.rseq = 0; c.sslot = c.rslot = 0;
   c.left = rec.left;
@@ -1797,6 +1797,8 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)
 template <class R, bool RAGGED>
 __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams launch_params) {
   KernelParams p = launch_params;
+  // (the context's record is asked for in front of the launch's number: two round trips of a workgroup's start side by side)
+  const DevCtx record = launch_params.ctxs[blockIdx.x];
   (void)begin_launch(p);
   const uint32_t lane = threadIdx.x;
   const bool writer = lane == 0;
@@ -1807,7 +1809,7 @@ __global__ void __launch_bounds__(64) exec_kernel_chain_fold(const KernelParams 
   bool active;
   {
     Context first;
-    init_context<false, RAGGED>(h, first, p, 0, (int)blockIdx.x, writer);  // (a workgroup hosts the context of its own number)
+    init_context<false, RAGGED>(h, first, p, 0, (int)blockIdx.x, writer, &record);  // (a workgroup hosts the context of its own number)
     active = first.active;
     left = uniform(first.left);
     off = uniform((uint64_t)first.off);
