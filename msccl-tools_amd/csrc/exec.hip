@@ -158,9 +158,10 @@ static size_t append_table(std::vector<unsigned char>& bytes, const std::vector<
 
 // Whether a launch's step table can hold FlatOp records (plan.h): lines on one-wave workgroups, one pass, one row of at
 // most 128 whole units per step, and no step that waits for, or is waited for by, another threadblock of its rank.
-// (Not in profiling builds, whose clocks live in the general loop.)
+// (Not in profiling builds, whose clocks live in the general loop; -DMSCCLX_NO_FLAT_STEPS builds a library that always runs
+// the general loop, to measure one against the other.)
 static bool flat_steps(const mscclx_plan& plan, const Geometry& g) {
-#if defined(MSCCLX_PROFILE) || defined(MSCCLX_EXP_NO_FLAT)
+#if defined(MSCCLX_PROFILE) || defined(MSCCLX_NO_FLAT_STEPS)
   return false;
 #endif
   if (!g.ll || !one_wave_each(g) || g.passes != 1 || g.piece_units > 128 || plan.chunk_bytes % 16 != 0) return false;
