@@ -587,3 +587,26 @@ def test_init_to_run_flow(capsys):
     ex.run(ins, outs)
     want = oc.expected_allreduce(y, 64, oc.allpairs_allreduce_orders(8), "float32")
     assert all(np.array_equal(res[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)) for r in range(8))
+
+
+def test_bench_times_any_ir_file():
+    """`bench.py --xml FILE --chunk-bytes A,B` times one MSCCL-IR document by itself: one JSON line per chunk size, with the
+    geometry and the step loop it ran on; `bench.py --gpus 2` refuses (every rank is a virtual rank on one GPU)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    fixture = os.path.join(root, "tests", "golden", "reference_xml", "allreduce_a100_allpairs_8r.xml.gz")
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--xml", fixture, "--chunk-bytes", "1024,65536", "--steps", "5", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(l) for l in r.stdout.splitlines() if l.startswith("{")]
+    assert [l["chunk_bytes"] for l in lines] == [1024, 65536]
+    for l in lines:
+        assert l["ranks"] == 8 and l["collective"] == "allreduce" and l["launches"] == 5
+        assert 1.0 < l["us_per_launch_median"] < 10000.0 and l["algorithmic_bytes"] > 0
+        assert set(l["geometry"]) >= {"workgroups", "threads", "slices", "piece_bytes", "passes"}
+    assert lines[0]["step_loop"] == "chain, folded nops"   # (small chunks: one-wave workgroups, one context each)
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr
