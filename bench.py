@@ -269,13 +269,21 @@ def time_program(path, chunk_sizes, steps, warmup, knobs):
     launch stream, median and mean.  Inputs are random; an all-reduce keeps reducing what the launch before left (finite for
     the few launches timed here)."""
     import gzip
-    import torch
-    from msccl.executor import Executor, parse_algo_xml
-    from msccl.executor.binding import LOOP_NAMES
-    from msccl.executor.workloads import HBM_PEAK_BYTES_PER_S
+    from msccl.executor import parse_algo_xml
     opener = gzip.open if path.endswith(".gz") else open
     with opener(path, "rt") as f:
         tables = parse_algo_xml(f.read())
+    for row in time_tables(tables, os.path.basename(path), chunk_sizes, steps, warmup, knobs):
+        print(json.dumps(row), flush=True)
+
+
+def time_tables(tables, name, chunk_sizes, steps, warmup, knobs):
+    """time_program's rows for tables that are already parsed."""
+    import torch
+    from msccl.executor import Executor
+    from msccl.executor.binding import LOOP_NAMES
+    from msccl.executor.workloads import HBM_PEAK_BYTES_PER_S
+    rows = []
     for cb in chunk_sizes:
         ins = [torch.rand(int(tables.rank_chunks[r, 0]) * cb // 4, device="cuda:0") * 1e-3 if tables.rank_chunks[r, 0] else None for r in range(tables.ngpus)]
         outs = [torch.zeros(int(tables.rank_chunks[r, 1]) * cb // 4, device="cuda:0") if tables.rank_chunks[r, 1] else None for r in range(tables.ngpus)]
@@ -289,13 +297,14 @@ def time_program(path, chunk_sizes, steps, warmup, knobs):
         ex.wait()
         med, mean = ts[len(ts) // 2] * 1e-3, sum(ts) / len(ts) * 1e-3
         ab = ex.algorithmic_bytes()
-        print(json.dumps({"program": os.path.basename(path), "ranks": int(tables.ngpus), "collective": tables.coll, "chunk_bytes": cb,
+        rows.append({"program": name, "ranks": int(tables.ngpus), "collective": tables.coll, "chunk_bytes": cb,
                           "us_per_launch_median": round(med * 1e6, 2), "us_per_launch_mean": round(mean * 1e6, 2), "launches": steps,
                           "algorithmic_bytes": int(ab), "algorithmic_GBps": round(ab / med / 1e9, 1), "hbm_fraction": round(ab / med / HBM_PEAK_BYTES_PER_S, 4),
                           "step_loop": LOOP_NAMES.get(int(info.kernel_loop), str(int(info.kernel_loop))),
                           "geometry": {k: int(getattr(info, k)) for k in ("workgroups", "threads", "slices", "piece_bytes", "passes", "max_hosted", "protocol")},
-                          "knobs": knobs}), flush=True)
+                          "knobs": knobs})
         del ex, ins, outs
+    return rows
 
 
 def cpu_baseline(key):
@@ -418,6 +427,12 @@ def main():
             line["others"][key] = {k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items() if k != "geometry"}
             line["others"][key].update(r["geometry"])
             line["others"][key]["traffic"] = traffic.get(key)
+        # what msccl.init('mi355x', ...) hands out for an all-reduce below 16 MB per rank: the all-pairs program (msccl-tools'
+        # msccl/programs/allreduce_allpairs.py), here on 8 ranks at 64 KiB and 4 MiB per rank (64 chunks of 1 KiB and of 64 KiB)
+        from msccl.executor import parse_algo_xml
+        from msccl.programs import catalog
+        line["small_message_default"] = time_tables(parse_algo_xml(catalog.allpairs_allreduce(8, 1)), "allpairs_allreduce(8 ranks)", [1024, 65536],
+                                                   max(5, args.steps // 2), args.warmup, {})
     print(json.dumps(line))
 
 
